@@ -1,0 +1,300 @@
+"""Pins the CPU oracle: library equivalence, closed forms, invariants, brute force.
+
+The reference (llm-core/llm_core/model.py:308-325, nn_functional.py:8-11) ships
+no tests or fixtures, so the oracle is pinned by what the mathematics fixes and
+by the library routine the reference itself treats as interchangeable
+(model.py:381-385).  Each check is chosen so a plausible slip (dropped scale,
+wrong mask polarity, transposed operand, wrong head mapping) fails it.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention_oracle as orc
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+# ---- library equivalence ---------------------------------------------------
+@pytest.mark.parametrize("S,D", [(1, 8), (17, 16), (64, 64), (130, 128)])
+def test_dense_equals_torch_sdpa_causal(S, D):
+    Q, K, V = rnd(2, 3, S, D, seed=1), rnd(2, 3, S, D, seed=2), rnd(2, 3, S, D, seed=3)
+    got = orc.scaled_dot_product_attention(Q, K, V, orc.causal_keep_mask(S))
+    want = torch.nn.functional.scaled_dot_product_attention(Q, K, V, is_causal=True)
+    torch.testing.assert_close(got, want, atol=2e-5, rtol=1e-5)
+
+
+def test_dense_equals_torch_sdpa_nomask_and_boolmask():
+    Q, K, V = rnd(2, 2, 9, 16, seed=4), rnd(2, 2, 13, 16, seed=5), rnd(2, 2, 13, 24, seed=6)
+    got = orc.scaled_dot_product_attention(Q, K, V)
+    want = torch.nn.functional.scaled_dot_product_attention(Q, K, V)
+    torch.testing.assert_close(got, want, atol=2e-5, rtol=1e-5)
+    g = torch.Generator().manual_seed(7)
+    keep = torch.rand(9, 13, generator=g) > 0.4
+    keep[:, 0] = True
+    got = orc.scaled_dot_product_attention(Q, K, V, keep)
+    want = torch.nn.functional.scaled_dot_product_attention(Q, K, V, attn_mask=keep)
+    torch.testing.assert_close(got, want, atol=2e-5, rtol=1e-5)
+
+
+def test_softmax_equals_torch_and_shift_invariant():
+    x = rnd(5, 7, seed=8, scale=4.0)
+    torch.testing.assert_close(orc.softmax(x, -1), torch.softmax(x, -1))
+    torch.testing.assert_close(orc.softmax(x, 0), torch.softmax(x, 0))
+    torch.testing.assert_close(orc.softmax(x + 1000.0, -1), orc.softmax(x, -1), atol=1e-6, rtol=1e-4)
+    assert torch.isnan(orc.softmax(torch.full((1, 4), float("-inf")), -1)).all()
+
+
+# ---- closed forms ----------------------------------------------------------
+def test_single_key_returns_its_value():
+    Q, K, V = rnd(3, 5, 8, seed=9), rnd(3, 1, 8, seed=10), rnd(3, 1, 6, seed=11)
+    out = orc.scaled_dot_product_attention(Q, K, V)
+    torch.testing.assert_close(out, V.expand(3, 5, 6))
+
+
+def test_identical_keys_give_mean_of_values():
+    Q = rnd(4, 8, seed=12)
+    K = rnd(1, 8, seed=13).expand(6, 8)
+    V = rnd(6, 5, seed=14)
+    out = orc.scaled_dot_product_attention(Q, K, V)
+    torch.testing.assert_close(out, V.mean(0, keepdim=True).expand(4, 5), atol=1e-6, rtol=1e-5)
+
+
+def test_constant_values_pass_through():
+    Q, K = rnd(4, 8, seed=15), rnd(9, 8, seed=16)
+    V = torch.full((9, 3), 2.5)
+    torch.testing.assert_close(orc.scaled_dot_product_attention(Q, K, V), torch.full((4, 3), 2.5))
+
+
+def test_zero_query_causal_is_cumulative_mean():
+    S = 11
+    K, V = rnd(S, 8, seed=17), rnd(S, 4, seed=18)
+    out = orc.scaled_dot_product_attention(torch.zeros(S, 8), K, V, orc.causal_keep_mask(S))
+    want = torch.cumsum(V, 0) / torch.arange(1, S + 1).unsqueeze(1)
+    torch.testing.assert_close(out, want, atol=1e-6, rtol=1e-5)
+    torch.testing.assert_close(out[0], V[0])                 # causal row 0 sees key 0 only
+
+
+def test_dominant_score_selects_value_and_scale_is_one_over_sqrt_d():
+    d = 16
+    K = torch.eye(5, d)
+    V = rnd(5, 3, seed=19)
+    Q = torch.zeros(1, d)
+    Q[0, 2] = 400.0                                          # score 100 for key 2, 0 for others
+    torch.testing.assert_close(orc.scaled_dot_product_attention(Q, K, V)[0], V[2])
+    # exact weights pin the 1/sqrt(d) scale: scores (ln 3)·e_0 -> weights 3/7, 1/7 ...
+    Q = torch.zeros(1, d)
+    Q[0, 0] = math.log(3.0) * math.sqrt(d)
+    out = orc.scaled_dot_product_attention(Q, K, V)[0]
+    w = torch.tensor([3.0, 1, 1, 1, 1]) / 7.0
+    torch.testing.assert_close(out, w @ V, atol=1e-6, rtol=1e-5)
+
+
+def test_mask_polarity_true_means_keep():
+    Q, K, V = rnd(2, 4, seed=20), rnd(3, 4, seed=21), rnd(3, 2, seed=22)
+    keep = torch.tensor([[True, False, False], [False, False, True]])
+    out = orc.scaled_dot_product_attention(Q, K, V, keep)
+    torch.testing.assert_close(out, torch.stack([V[0], V[2]]))
+
+
+def test_causal_mask_square_is_tril_and_rect_is_bottom_right():
+    assert torch.equal(orc.causal_keep_mask(6), torch.tril(torch.ones(6, 6, dtype=torch.bool)))
+    m = orc.causal_keep_mask(2, 5)
+    assert m.tolist() == [[True, True, True, True, False], [True] * 5]
+
+
+# ---- invariants ------------------------------------------------------------
+def test_key_permutation_invariance():
+    Q, K, V = rnd(4, 8, seed=23), rnd(10, 8, seed=24), rnd(10, 8, seed=25)
+    p = torch.randperm(10, generator=torch.Generator().manual_seed(1))
+    torch.testing.assert_close(orc.scaled_dot_product_attention(Q, K[p], V[p]),
+                               orc.scaled_dot_product_attention(Q, K, V), atol=1e-6, rtol=1e-5)
+
+
+def test_output_in_convex_hull():
+    Q, K, V = rnd(6, 8, seed=26), rnd(12, 8, seed=27), rnd(12, 4, seed=28)
+    out = orc.scaled_dot_product_attention(Q, K, V)
+    assert (out <= V.max(0)[0] + 1e-6).all() and (out >= V.min(0)[0] - 1e-6).all()
+
+
+def test_custom_scale_equals_scaled_keys():
+    q, k, v = rnd(1, 2, 7, 16, seed=29), rnd(1, 2, 7, 16, seed=30), rnd(1, 2, 7, 16, seed=31)
+    a = orc.prefill_reference(q, k, v, causal=True, softmax_scale=0.7)
+    b = orc.prefill_reference(q, k * (0.7 * 4.0), v, causal=True)      # default 1/sqrt(16)=1/4
+    torch.testing.assert_close(a, b, atol=1e-5, rtol=1e-5)
+
+
+def test_gqa_equals_mha_on_repeated_heads_and_head_mapping():
+    q = rnd(2, 6, 9, 8, seed=32)
+    k, v = rnd(2, 2, 9, 8, seed=33), rnd(2, 2, 9, 8, seed=34)
+    a = orc.prefill_reference(q, k, v, causal=True, head_chunk=4)
+    kk, vv = k.repeat_interleave(3, 1), v.repeat_interleave(3, 1)
+    b = orc.scaled_dot_product_attention(q, kk, vv, orc.causal_keep_mask(9))
+    torch.testing.assert_close(a, b, atol=1e-6, rtol=1e-5)
+    # head 3 must read kv head 1 (3 // 3), not 3 % 2
+    c = orc.scaled_dot_product_attention(q[:, 3], k[:, 1], v[:, 1], orc.causal_keep_mask(9))
+    torch.testing.assert_close(a[:, 3], c, atol=1e-6, rtol=1e-5)
+
+
+def test_varlen_equals_per_sequence_dense():
+    lens = [5, 1, 12]
+    cu = torch.tensor([0, 5, 6, 18], dtype=torch.int32)
+    q, k, v = rnd(18, 4, 8, seed=35), rnd(18, 2, 8, seed=36), rnd(18, 2, 8, seed=37)
+    out = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True)
+    off = 0
+    for L in lens:
+        qb = q[off:off + L].transpose(0, 1)[None]
+        kb = k[off:off + L].transpose(0, 1)[None]
+        vb = v[off:off + L].transpose(0, 1)[None]
+        want = orc.prefill_reference(qb, kb, vb, causal=True)[0].transpose(0, 1)
+        torch.testing.assert_close(out[off:off + L], want)
+        off += L
+
+
+def test_batch_elements_independent():
+    q, k, v = rnd(3, 2, 6, 8, seed=38), rnd(3, 2, 6, 8, seed=39), rnd(3, 2, 6, 8, seed=40)
+    full = orc.prefill_reference(q, k, v)
+    one = orc.prefill_reference(q[1:2], k[1:2], v[1:2])
+    torch.testing.assert_close(full[1:2], one)
+
+
+# ---- brute force -----------------------------------------------------------
+@pytest.mark.parametrize("S", [1, 2, 15, 16, 17, 33])
+def test_dense_vs_float64_loops(S):
+    Q, K, V = rnd(S, 8, seed=41 + S), rnd(S, 8, seed=42 + S), rnd(S, 5, seed=43 + S)
+    keep = orc.causal_keep_mask(S)
+    want = orc.bruteforce_attention_f64(Q.numpy(), K.numpy(), V.numpy(), keep.tolist())
+    got = orc.scaled_dot_product_attention(Q, K, V, keep).numpy()
+    np.testing.assert_allclose(got, want, atol=2e-6, rtol=1e-5)
+
+
+# ---- paged decode ----------------------------------------------------------
+def _paged(ctx, seed=0, Hq=4, Hkv=2, D=8, bs=16, pool_factor=1.5):
+    return orc.make_paged_case(batch=len(ctx), n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D,
+                               block_size=bs, context_lens=ctx, pool_factor=pool_factor, seed=seed)
+
+
+@pytest.mark.parametrize("ctx", [[1], [15, 16, 17], [255, 256, 257], [33, 1, 64]])
+def test_paged_decode_vs_float64_loops(ctx):
+    q, kc, vc, bt, cl = _paged(ctx, seed=3)
+    got = orc.paged_decode_reference(q, kc, vc, bt, cl)
+    Hq, Hkv, bs = q.shape[1], kc.shape[1], kc.shape[2]
+    for b in range(len(ctx)):
+        for h in range(Hq):
+            g = h // (Hq // Hkv)
+            rows_k = [kc[int(bt[b, t // bs]), g, t % bs] for t in range(ctx[b])]   # token-by-token walk
+            rows_v = [vc[int(bt[b, t // bs]), g, t % bs] for t in range(ctx[b])]
+            want = orc.bruteforce_attention_f64(q[b, h][None].numpy(), torch.stack(rows_k).numpy(),
+                                                torch.stack(rows_v).numpy())
+            np.testing.assert_allclose(got[b, h].numpy(), want[0], atol=2e-6, rtol=1e-5)
+
+
+def test_paged_decode_invariant_to_physical_placement_and_pool_garbage():
+    ctx = [40, 7, 100]
+    q, kc, vc, bt, cl = _paged(ctx, seed=5, pool_factor=2.0)
+    base = orc.paged_decode_reference(q, kc, vc, bt, cl)
+    # move every used block to a new physical slot
+    pool = kc.shape[0]
+    perm = torch.randperm(pool, generator=torch.Generator().manual_seed(9))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(pool)
+    kc2, vc2 = kc[perm], vc[perm]                 # new slot i holds old block perm[i]
+    bt2 = inv[bt.long()].to(torch.int32)
+    torch.testing.assert_close(orc.paged_decode_reference(q, kc2, vc2, bt2, cl), base)
+    # garbage in unused blocks and in the tail of the last block must not matter
+    used = torch.zeros(pool, dtype=torch.bool)
+    for b, c in enumerate(ctx):
+        used[bt[b, :(c + 15) // 16].long()] = True
+    kc3, vc3 = kc.clone(), vc.clone()
+    kc3[~used] = 1e4
+    vc3[~used] = -1e4
+    for b, c in enumerate(ctx):
+        if c % 16:
+            last = int(bt[b, (c - 1) // 16])
+            kc3[last, :, c % 16:] = 1e4
+            vc3[last, :, c % 16:] = 1e4
+    torch.testing.assert_close(orc.paged_decode_reference(q, kc3, vc3, bt, cl), base)
+
+
+def test_paged_decode_equals_dense_last_row_of_causal_prefill():
+    S, Hq, Hkv, D = 37, 4, 2, 8
+    q, k, v = rnd(1, Hq, S, D, seed=50), rnd(1, Hkv, S, D, seed=51), rnd(1, Hkv, S, D, seed=52)
+    dense = orc.prefill_reference(q, k, v, causal=True)[0, :, -1]          # (Hq,D)
+    nblk = (S + 15) // 16
+    kc = torch.zeros(nblk + 2, Hkv, 16, D)
+    vc = torch.zeros(nblk + 2, Hkv, 16, D)
+    table = torch.tensor([[2, 0, 4]], dtype=torch.int32)
+    for t in range(S):
+        kc[int(table[0, t // 16]), :, t % 16] = k[0, :, t]
+        vc[int(table[0, t // 16]), :, t % 16] = v[0, :, t]
+    got = orc.paged_decode_reference(q[:, :, -1], kc, vc, table, torch.tensor([S], dtype=torch.int32))
+    torch.testing.assert_close(got[0], dense, atol=1e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("bounds", [[(0, 50)], [(0, 16), (16, 50)], [(0, 1), (1, 2), (2, 49), (49, 50)]])
+def test_split_combine_independent_of_splits(bounds):
+    q, k, v = rnd(8, seed=60), rnd(50, 8, seed=61), rnd(50, 8, seed=62)
+    want = orc.scaled_dot_product_attention(q[None], k, v)[0]
+    got = orc.combine_splits_reference(orc.split_partials_reference(q, k, v, bounds))
+    torch.testing.assert_close(got, want, atol=1e-6, rtol=1e-5)
+
+
+# ---- fp8 KV ----------------------------------------------------------------
+def test_fp8_quantiser_properties():
+    x = rnd(6, 2, 16, 32, seed=70).to(torch.bfloat16)
+    x[3] = 0                                                    # all-zero blocks
+    q8, sc = orc.quantize_kv_fp8(x)
+    assert q8.dtype == torch.uint8 and sc.shape == (6, 2) and sc.dtype == torch.float32
+    assert (sc[3] == 1.0).all() and (q8[3] == 0).all()
+    torch.testing.assert_close(sc[:3], x[:3].float().abs().amax((2, 3)) / 448.0)
+    dq = orc.dequantize_kv_fp8(q8, sc)
+    xf = x.float()
+    # absmax element maps to +-448 exactly
+    for b in (0, 1, 2, 4, 5):
+        for h in range(2):
+            i = xf[b, h].abs().argmax()
+            assert abs(q8[b, h].view(torch.float8_e4m3fn).float().flatten()[i]) == 448.0
+    # e4m3 keeps 3 mantissa bits: relative error <= 2^-4 for normals (|y| >= 2^-6 after scaling)
+    y = xf / sc[:, :, None, None]
+    normal = y.abs() >= 2.0 ** -6
+    rel = ((dq - xf).abs() / xf.abs().clamp_min(1e-30))[normal]
+    assert rel.max() <= 2.0 ** -4 + 1e-6
+    # subnormals: absolute error <= half of the subnormal step 2^-9, times scale
+    err_sub = ((dq - xf).abs() / sc[:, :, None, None])[~normal]
+    assert err_sub.numel() == 0 or err_sub.max() <= 2.0 ** -10 + 1e-9
+
+
+def test_fp8_e4m3_bit_patterns_are_ocp():
+    # OCP e4m3fn: 0x7E = 448, 0x38 = 1.0, 0x01 = 2^-9, 0x7F = NaN (no infinities)
+    b = torch.tensor([0x7E, 0x38, 0x01, 0xB8], dtype=torch.uint8).view(torch.float8_e4m3fn).float()
+    assert b.tolist() == [448.0, 1.0, 2.0 ** -9, -1.0]
+
+
+def test_paged_decode_fp8_equals_oracle_on_dequantised_cache():
+    ctx = [45, 16]
+    q, kc, vc, bt, cl = _paged(ctx, seed=8, D=16)
+    k8, ks = orc.quantize_kv_fp8(kc)
+    v8, vs = orc.quantize_kv_fp8(vc)
+    a = orc.paged_decode_reference(q, k8, v8, bt, cl, k_scale=ks, v_scale=vs)
+    b = orc.paged_decode_reference(q, orc.dequantize_kv_fp8(k8, ks), orc.dequantize_kv_fp8(v8, vs), bt, cl)
+    torch.testing.assert_close(a, b)
+    full = orc.paged_decode_reference(q, kc, vc, bt, cl)
+    assert (a - full).abs().max() < 0.15                       # quantisation noise only
+
+
+# ---- workload generators ---------------------------------------------------
+def test_workload_generators_are_seeded_and_well_formed():
+    c1 = orc.draw_context_lens("uniform", 128, 512, 16384, 0)
+    c2 = orc.draw_context_lens("uniform", 128, 512, 16384, 0)
+    assert torch.equal(c1, c2) and c1.min() >= 512 and c1.max() <= 16384
+    c3 = orc.draw_context_lens("loguniform", 256, 128, 32768, 0)
+    assert c3.min() >= 128 and c3.max() <= 32768 and c3.float().median() < 5000
+    q, kc, vc, bt, cl = orc.make_paged_case(batch=4, n_q_heads=8, n_kv_heads=8, head_dim=64, block_size=16,
+                                            context_lens=[256] * 4, seed=0)
+    assert kc.shape == (64, 8, 16, 64) and bt.shape == (4, 16)
+    assert sorted(bt.flatten().tolist()) == list(range(64))     # a permutation of the 64 physical blocks
