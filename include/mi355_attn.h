@@ -1,0 +1,115 @@
+/*
+ * mi355_attn.h -- C ABI of libmi355attn.so: the attention hot path (causal
+ * prefill forward + paged-KV decode) as hand-written HIP kernels for gfx950.
+ *
+ * Conventions shared by every entry point
+ *   - all data pointers are DEVICE pointers owned by the caller; the library
+ *     never allocates or frees device memory and never synchronises the host;
+ *   - all work is enqueued on `stream` (a hipStream_t passed as void*; NULL is
+ *     the default stream);
+ *   - the return value is 0 on success, a negative MI355_E* code for a rejected
+ *     argument, or a positive hipError_t from the launch; mi355_last_error()
+ *     returns a thread-local message for the last non-zero return;
+ *   - strides are in ELEMENTS; the innermost (head_dim) stride is always 1;
+ *   - head_dim in {32, 64, 128}; GQA: query head h reads kv head h / (Hq / Hkv).
+ */
+#ifndef MI355_ATTN_H
+#define MI355_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    MI355_OK = 0,
+    MI355_EINVAL = -1,      /* bad shape / unsupported head_dim / null pointer   */
+    MI355_EWORKSPACE = -2,  /* workspace too small                               */
+    MI355_EDTYPE = -3       /* unsupported dtype code                            */
+};
+
+/* element type codes */
+enum {
+    MI355_BF16 = 0,         /* bfloat16 q/k/v/out and bf16 KV cache              */
+    MI355_FP8_E4M3 = 1      /* OCP fp8-e4m3 KV cache (max 448) + fp32 scales     */
+};
+
+/* mask modes of the prefill entry point */
+enum {
+    MI355_MASK_NONE = 0,
+    MI355_MASK_CAUSAL = 1,  /* query i keeps key j iff j <= i + (Sk - Sq)        */
+    MI355_MASK_BOOL = 2     /* explicit uint8 keep-mask (non-zero = attend)      */
+};
+
+/*
+ * Prefill attention forward: out = softmax(q k^T * softmax_scale [masked]) v.
+ *
+ * Replaces, in the reference, the attention slot of
+ * CausalMultiHeadSelfAttention.forward -- llm-core/llm_core/model.py:380-385 --
+ * i.e. torch.nn.functional.scaled_dot_product_attention(Q, K, V, is_causal=True)
+ * (model.py:382) and scaled_dot_product_attention(Q, K, V, mask)
+ * (model.py:308-325, softmax at llm-core/llm_core/nn_functional.py:8-11).
+ *
+ * Dense layout (cu_seqlens_q == NULL): tensors are (B, H, S, D) addressed as
+ *   base + b*strides[0] + h*strides[1] + s*strides[2] + d, so the reference's
+ *   contiguous Q/K and its strided V view (model.py:367-370) are both accepted.
+ * Packed layout (cu_seqlens_q != NULL): tensors are (T, H, D) addressed as
+ *   base + t*strides[2] + h*strides[1] + d (strides[0] ignored); sequence b
+ *   owns rows [cu_seqlens[b], cu_seqlens[b+1]); cu_seqlens are int32 (B+1).
+ * mask (MI355_MASK_BOOL only): uint8, element (b,h,i,j) at
+ *   mask + b*mask_strides[0] + h*mask_strides[1] + i*mask_strides[2] + j
+ *   (use stride 0 to broadcast); dense layout only.  A query row with every key
+ *   masked yields NaN, as the reference's softmax does.
+ * Sq_max/Sk_max: the (maximum) query/key sequence lengths.
+ */
+int mi355_prefill_fwd(const void* q, const void* k, const void* v, void* out,
+                      const int64_t q_strides[3], const int64_t k_strides[3],
+                      const int64_t v_strides[3], const int64_t o_strides[3],
+                      const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                      const uint8_t* mask, const int64_t mask_strides[3],
+                      int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
+                      float softmax_scale, int mask_mode, int dtype, void* stream);
+
+/*
+ * Paged-KV decode attention, one query token per sequence (split-K + combine).
+ *
+ * No counterpart exists in the reference: it is what a KV-cached replacement of
+ * TransformerLM.generate (llm-core/llm_core/model.py:187-236, which re-runs the
+ * full forward per token at :218) calls every step.  Its result is defined by
+ * reduction to model.py:308-325 on the gathered KV.
+ *
+ *   q, out        : (B, Hq, D) bf16, contiguous
+ *   k_cache/v_cache: (num_blocks, Hkv, block_size, D), bf16 (kv_dtype MI355_BF16)
+ *                   or fp8-e4m3 bytes (MI355_FP8_E4M3); block_size must be 16
+ *   block_tables  : int32, row b at block_tables + b*bt_row_stride; entry j is
+ *                   the physical block of tokens [16j, 16j+16); entries past
+ *                   ceil(context_lens[b]/16) are never read
+ *   context_lens  : int32 (B), each >= 1 (0 leaves that row of `out` unwritten)
+ *   k_scale/v_scale: fp32 (num_blocks, Hkv), required iff kv_dtype is fp8;
+ *                   real value = fp8 value * scale
+ *   workspace     : >= mi355_paged_decode_workspace_bytes(...) bytes, 16-byte
+ *                   aligned, contents irrelevant on entry (split-K partials)
+ *   max_ctx       : upper bound on every context_lens[b] (sizes the grid)
+ */
+int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
+                           const int32_t* block_tables, int64_t bt_row_stride,
+                           const int32_t* context_lens,
+                           const float* k_scale, const float* v_scale,
+                           void* workspace, size_t workspace_bytes,
+                           int B, int Hq, int Hkv, int D, int block_size, int max_ctx,
+                           float softmax_scale, int kv_dtype, void* stream);
+
+size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx);
+
+/* Tokens of one sequence handled by one workgroup of the split-K pass. */
+int mi355_paged_decode_chunk_tokens(void);
+
+const char* mi355_last_error(void);
+const char* mi355_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_ATTN_H */

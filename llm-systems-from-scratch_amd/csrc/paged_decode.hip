@@ -1,0 +1,409 @@
+// Paged-KV decode attention for gfx950: split-K pass + combine.
+//
+// Work item of the split-K pass = (sequence, kv head, chunk of kChunk tokens).
+// One workgroup of 4 wavefronts per work item; each wavefront streams its own
+// quarter of the chunk, 32 keys (two 16-token cache blocks) per step:
+//
+//   S^T (keys x queries) = K . Q^T      v_mfma_f32_16x16x32_bf16, the Hq/Hkv query
+//                                       heads that share the kv head are the N
+//                                       columns (padded to 16), so every KV byte
+//                                       is fetched once per GQA group
+//   online softmax on S^T               each lane owns ONE query column and 8 keys;
+//                                       max/sum across the 4 lanes of a column
+//   O^T (d x queries) += V^T . P^T      V^T fragments come from a wavefront-private
+//                                       LDS tile through ds_read_b64_tr_b16
+//
+// K goes global -> registers directly in MFMA A-operand layout; V goes
+// global -> registers (fully coalesced 1 KiB per instruction) -> LDS -> transposed
+// read.  The next step's K/V loads are issued before the current step's math.
+// The four wavefronts merge their (m, l, O) in LDS; a sequence that fits one
+// chunk is normalised and written straight to `out`, otherwise the chunk's
+// partial goes to the workspace and the combine kernel finishes it:
+//   o = sum_c 2^(m_c - m) o_c / sum_c 2^(m_c - m) l_c      (m = max_c m_c).
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace mi355 {
+
+constexpr int kDecodeWaves = 4;
+constexpr int kTokensPerWave = 256;
+constexpr int kChunk = kDecodeWaves * kTokensPerWave;   // tokens per workgroup
+constexpr int kBlock = 16;                              // tokens per cache block
+constexpr int kStage = 32;                              // keys per step (2 blocks)
+
+struct DecodeParams {
+    const __bf16* q;
+    const void* k_cache;
+    const void* v_cache;
+    __bf16* out;
+    const int32_t* block_tables;
+    int64_t bt_row_stride;
+    const int32_t* context_lens;
+    const float* k_scale;
+    const float* v_scale;
+    float* ws_o;
+    float* ws_m;
+    float* ws_l;
+    int B, Hq, Hkv, max_chunks, max_ctx;
+    float scale_log2;
+};
+
+template <int D>
+struct DecodeLds {
+    static constexpr int kVRow = D * 2 + 32;                 // bytes per staged V row (padded)
+    static constexpr int kVBytes = kStage * kVRow;           // per-wavefront V tile
+    static constexpr int kPartFloats = 16 * D + 32;          // per-wavefront (O, m, l)
+    static constexpr int kWaveBytes = kVBytes > kPartFloats * 4 ? kVBytes : kPartFloats * 4;
+};
+
+template <int D, bool FP8>
+__global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(DecodeParams p) {
+    constexpr int NS = D / 32;                       // MFMA k-steps of K.Q^T
+    constexpr int NT = D / 16;                       // 16-row tiles of O^T
+    constexpr int KL = FP8 ? (D / 64) : NS;          // 16-byte K loads per lane per block
+    constexpr int VL = FP8 ? (D / 64) : (D / 32);    // 16-byte V loads per lane per block
+    constexpr int kVRow = DecodeLds<D>::kVRow;
+    constexpr int kWaveBytes = DecodeLds<D>::kWaveBytes;
+    static_assert(!FP8 || D >= 64, "fp8 KV needs head_dim >= 64");
+
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kDecodeWaves * kWaveBytes];
+
+    const int chunk = blockIdx.x;
+    const int hk = blockIdx.y;
+    const int b = blockIdx.z;
+    const int ctx = min(p.context_lens[b], p.max_ctx);     // a length beyond the promised bound is truncated, never chased
+    const int chunk_start = chunk * kChunk;
+    if (chunk_start >= ctx) return;
+
+    const int G = p.Hq / p.Hkv;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 15;          // key row of K / query column of S^T / d row of V^T
+    const int kg = lane >> 4;         // 0..3
+
+    unsigned char* wsm = smem + wave * kWaveBytes;
+
+    // ---- Q^T B-operand fragments (zero for padded query columns) ----------
+    // bf16 cache: step s covers d = 32s + 8kg + j.
+    // fp8 cache : one 16-byte K load carries d = 64t + 16kg + (0..15); step s = 2t+e
+    //             covers d = 64t + 16kg + 8e + j, so Q uses the same d order.
+    bf16x8 qf[NS];
+    {
+        const __bf16* qrow = p.q + ((int64_t)b * p.Hq + (int64_t)hk * G + r) * D;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const int d0 = FP8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
+            u32x4 t = {0u, 0u, 0u, 0u};
+            if (r < G) t = *reinterpret_cast<const u32x4*>(qrow + d0);
+            qf[s] = as_bf16x8(t);
+        }
+    }
+
+    const int t0 = chunk_start + wave * kTokensPerWave;
+    const int t1 = min(ctx, t0 + kTokensPerWave);
+    const int n_iter = t1 > t0 ? (t1 - t0 + kStage - 1) / kStage : 0;
+    const int last_blk = (ctx - 1) / kBlock;
+    const int32_t* bt = p.block_tables + (int64_t)b * p.bt_row_stride;
+
+    struct Stage {
+        u32x4 k[2][KL];
+        u32x4 v[2][VL];
+        float ks[2], vs[2];
+    };
+
+    auto issue = [&](int it, Stage& st) {
+        const int bi0 = (t0 + it * kStage) / kBlock;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int bi = min(bi0 + t, last_blk);          // never read past the table
+            const int64_t phys = bt[bi];
+            const int64_t slab = (phys * p.Hkv + hk) * (int64_t)(kBlock * D);   // elements
+            if constexpr (FP8) {
+                const unsigned char* kb = reinterpret_cast<const unsigned char*>(p.k_cache) + slab;
+                const unsigned char* vb = reinterpret_cast<const unsigned char*>(p.v_cache) + slab;
+#pragma unroll
+                for (int j = 0; j < KL; ++j)
+                    st.k[t][j] = *reinterpret_cast<const u32x4*>(kb + r * D + 64 * j + 16 * kg);
+#pragma unroll
+                for (int j = 0; j < VL; ++j)
+                    st.v[t][j] = *reinterpret_cast<const u32x4*>(vb + (j * 64 + lane) * 16);
+                st.ks[t] = p.k_scale[phys * p.Hkv + hk];
+                st.vs[t] = p.v_scale[phys * p.Hkv + hk];
+            } else {
+                const __bf16* kb = reinterpret_cast<const __bf16*>(p.k_cache) + slab;
+                const __bf16* vb = reinterpret_cast<const __bf16*>(p.v_cache) + slab;
+#pragma unroll
+                for (int s = 0; s < KL; ++s)
+                    st.k[t][s] = *reinterpret_cast<const u32x4*>(kb + r * D + 32 * s + 8 * kg);
+#pragma unroll
+                for (int j = 0; j < VL; ++j)
+                    st.v[t][j] = *reinterpret_cast<const u32x4*>(vb + (j * 64 + lane) * 8);
+                st.ks[t] = 1.0f;
+                st.vs[t] = 1.0f;
+            }
+        }
+    };
+
+    float m_run = -INFINITY;      // running max (log2 domain) of this lane's query column
+    float l_run = 0.0f;           // this lane's share of the running sum
+    f32x4 o[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto compute = [&](int it, Stage& st) {
+        const int kbase = t0 + it * kStage;
+        const bool tail = kbase + kStage > t1;
+
+        // ---- V: registers -> wavefront-private LDS tile (bf16, row = key) --
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int j = 0; j < VL; ++j) {
+                if constexpr (FP8) {
+                    const int e = (j * 64 + lane) * 16;     // element index in the block slab
+                    const int row = e / D, col = e % D;
+                    u32x4 raw = st.v[t][j];
+                    if (tail && kbase + 16 * t + row >= t1) raw = u32x4{0u, 0u, 0u, 0u};
+                    u32x2 a = fp8x4_to_bf16x4(raw[0]), bq = fp8x4_to_bf16x4(raw[1]);
+                    u32x2 c = fp8x4_to_bf16x4(raw[2]), dq = fp8x4_to_bf16x4(raw[3]);
+                    unsigned char* dst = wsm + (16 * t + row) * kVRow + col * 2;
+                    *reinterpret_cast<u32x4*>(dst) = u32x4{a[0], a[1], bq[0], bq[1]};
+                    *reinterpret_cast<u32x4*>(dst + 16) = u32x4{c[0], c[1], dq[0], dq[1]};
+                } else {
+                    const int e = (j * 64 + lane) * 8;
+                    const int row = e / D, col = e % D;
+                    u32x4 raw = st.v[t][j];
+                    if (tail && kbase + 16 * t + row >= t1) raw = u32x4{0u, 0u, 0u, 0u};
+                    *reinterpret_cast<u32x4*>(wsm + (16 * t + row) * kVRow + col * 2) = raw;
+                }
+            }
+        }
+
+        // ---- S^T = K . Q^T ---------------------------------------------------
+        f32x4 s_acc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            s_acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if constexpr (FP8) {
+#pragma unroll
+                for (int j = 0; j < KL; ++j) {
+                    u32x4 raw = st.k[t][j];
+                    u32x2 a = fp8x4_to_bf16x4(raw[0]), bq = fp8x4_to_bf16x4(raw[1]);
+                    u32x2 c = fp8x4_to_bf16x4(raw[2]), dq = fp8x4_to_bf16x4(raw[3]);
+                    s_acc[t] = mfma16(as_bf16x8(u32x4{a[0], a[1], bq[0], bq[1]}), qf[2 * j], s_acc[t]);
+                    s_acc[t] = mfma16(as_bf16x8(u32x4{c[0], c[1], dq[0], dq[1]}), qf[2 * j + 1], s_acc[t]);
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < NS; ++s) s_acc[t] = mfma16(as_bf16x8(st.k[t][s]), qf[s], s_acc[t]);
+            }
+        }
+
+        // ---- online softmax (lane: query column r, keys 16t + 4kg + i) -------
+        float x[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const float sc = p.scale_log2 * st.ks[t];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float v = s_acc[t][i] * sc;
+                if (tail && kbase + 16 * t + 4 * kg + i >= t1) v = -INFINITY;
+                x[4 * t + i] = v;
+                mx = fmaxf(mx, v);
+            }
+        }
+        mx = xor_max_16_32(mx);
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            x[i] = fast_exp2(x[i] - m_new);
+            psum += x[i];
+        }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int i = 0; i < NT; ++i) o[i] *= alpha;
+        u32x4 pp;
+        pp[0] = pack_bf16(x[0] * st.vs[0], x[1] * st.vs[0]);
+        pp[1] = pack_bf16(x[2] * st.vs[0], x[3] * st.vs[0]);
+        pp[2] = pack_bf16(x[4] * st.vs[1], x[5] * st.vs[1]);
+        pp[3] = pack_bf16(x[6] * st.vs[1], x[7] * st.vs[1]);
+        const bf16x8 pf = as_bf16x8(pp);
+
+        // ---- O^T += V^T . P^T -------------------------------------------------
+        // source lane s of group kg addresses key row 4kg + s/4, columns 16dt + 4(s%4)..+3
+        const unsigned char* vsrc = wsm + (4 * kg + (r >> 2)) * kVRow + (r & 3) * 8;
+#pragma unroll
+        for (int dt = 0; dt < NT; ++dt) {
+            i16x4 lo = lds_read_tr16(vsrc + dt * 32);
+            i16x4 hi = lds_read_tr16(vsrc + 16 * kVRow + dt * 32);
+            o[dt] = mfma16(join_bf16x8(lo, hi), pf, o[dt]);
+        }
+    };
+
+    {
+        Stage sa, sb;
+        if (n_iter > 0) issue(0, sa);
+        for (int it = 0; it < n_iter; it += 2) {
+            if (it + 1 < n_iter) issue(it + 1, sb);
+            compute(it, sa);
+            if (it + 1 < n_iter) {
+                if (it + 2 < n_iter) issue(it + 2, sa);
+                compute(it + 1, sb);
+            }
+        }
+    }
+
+    // ---- merge the four wavefronts ------------------------------------------
+    l_run = xor_sum_16_32(l_run);
+    {
+        float* part = reinterpret_cast<float*>(wsm);
+#pragma unroll
+        for (int dt = 0; dt < NT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part[r * D + 16 * dt + 4 * kg + i] = o[dt][i];
+        if (kg == 0) {
+            part[16 * D + r] = m_run;
+            part[16 * D + 16 + r] = l_run;
+        }
+    }
+    __syncthreads();
+
+    const int n_chunks = (ctx + kChunk - 1) / kChunk;
+    for (int idx = threadIdx.x; idx < G * D; idx += kDecodeWaves * 64) {
+        const int qi = idx / D, d = idx % D;
+        float mw[kDecodeWaves];
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kDecodeWaves; ++w) {
+            mw[w] = reinterpret_cast<const float*>(smem + w * kWaveBytes)[16 * D + qi];
+            M = fmaxf(M, mw[w]);
+        }
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < kDecodeWaves; ++w) {
+            const float* part = reinterpret_cast<const float*>(smem + w * kWaveBytes);
+            const float f = fast_exp2(mw[w] - M);       // a wavefront without keys has m = -inf -> 0
+            num += f * part[qi * D + d];
+            den += f * part[16 * D + 16 + qi];
+        }
+        const int64_t row = (int64_t)b * p.Hq + (int64_t)hk * G + qi;
+        if (n_chunks == 1) {
+            p.out[row * D + d] = (__bf16)(num / den);
+        } else {
+            const int64_t slot = row * p.max_chunks + chunk;
+            p.ws_o[slot * D + d] = num;
+            if (d == 0) {
+                p.ws_m[slot] = M;
+                p.ws_l[slot] = den;
+            }
+        }
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(D) void paged_decode_combine_kernel(DecodeParams p) {
+    const int row = blockIdx.x;                  // b * Hq + h
+    const int b = row / p.Hq;
+    const int ctx = min(p.context_lens[b], p.max_ctx);
+    const int n_chunks = (ctx + kChunk - 1) / kChunk;
+    if (n_chunks <= 1) return;                   // written by the split pass (or empty)
+    const int d = threadIdx.x;
+    const int64_t base = (int64_t)row * p.max_chunks;
+    float M = -INFINITY;
+    for (int c = 0; c < n_chunks; ++c) M = fmaxf(M, p.ws_m[base + c]);
+    float num = 0.f, den = 0.f;
+    for (int c = 0; c < n_chunks; ++c) {
+        const float f = fast_exp2(p.ws_m[base + c] - M);
+        num += f * p.ws_o[(base + c) * D + d];
+        den += f * p.ws_l[base + c];
+    }
+    p.out[(int64_t)row * D + d] = (__bf16)(num / den);
+}
+
+template <int D, bool FP8>
+static int launch_decode(const DecodeParams& p, hipStream_t stream) {
+    dim3 grid(p.max_chunks, p.Hkv, p.B);
+    hipLaunchKernelGGL((paged_decode_split_kernel<D, FP8>), grid, dim3(kDecodeWaves * 64), 0, stream, p);
+    if (p.max_chunks > 1)
+        hipLaunchKernelGGL((paged_decode_combine_kernel<D>), dim3(p.B * p.Hq), dim3(D), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+extern "C" int mi355_paged_decode_chunk_tokens(void) { return kChunk; }
+
+extern "C" size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx) {
+    if (B <= 0 || Hq <= 0 || D <= 0 || max_ctx <= 0) return 0;
+    const size_t chunks = ((size_t)max_ctx + kChunk - 1) / kChunk;
+    const size_t rows = (size_t)B * Hq * chunks;
+    return align_up(rows * D * 4, 256) + 2 * align_up(rows * 4, 256);
+}
+
+extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                      const int32_t* block_tables, int64_t bt_row_stride,
+                                      const int32_t* context_lens, const float* k_scale,
+                                      const float* v_scale, void* workspace, size_t workspace_bytes, int B,
+                                      int Hq, int Hkv, int D, int block_size, int max_ctx,
+                                      float softmax_scale, int kv_dtype, void* stream) {
+    if (!q || !k_cache || !v_cache || !out || !block_tables || !context_lens)
+        return set_error(MI355_EINVAL, "paged_decode: null pointer argument");
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || max_ctx <= 0)
+        return set_error(MI355_EINVAL, "paged_decode: B, Hq, Hkv and max_ctx must be positive");
+    if (Hq % Hkv != 0 || Hq / Hkv > 16)
+        return set_error(MI355_EINVAL, "paged_decode: Hq must be a multiple of Hkv with Hq/Hkv <= 16");
+    if (block_size != kBlock) return set_error(MI355_EINVAL, "paged_decode: block_size must be 16");
+    if (Hkv > 65535 || B > 65535) return set_error(MI355_EINVAL, "paged_decode: Hkv and B must be <= 65535");
+    if (kv_dtype != MI355_BF16 && kv_dtype != MI355_FP8_E4M3)
+        return set_error(MI355_EDTYPE, "paged_decode: kv_dtype must be MI355_BF16 or MI355_FP8_E4M3");
+    const bool fp8 = kv_dtype == MI355_FP8_E4M3;
+    if (fp8 && (!k_scale || !v_scale))
+        return set_error(MI355_EINVAL, "paged_decode: fp8 KV cache needs k_scale and v_scale");
+    if (!(D == 128 || D == 64 || (D == 32 && !fp8)))
+        return set_error(MI355_EINVAL, "paged_decode: head_dim must be 64 or 128 (or 32 with a bf16 cache)");
+    const size_t need = mi355_paged_decode_workspace_bytes(B, Hq, D, max_ctx);
+    const int max_chunks = (max_ctx + kChunk - 1) / kChunk;
+    if (max_chunks > 1 && (!workspace || workspace_bytes < need))
+        return set_error(MI355_EWORKSPACE, "paged_decode: workspace smaller than mi355_paged_decode_workspace_bytes()");
+
+    DecodeParams p;
+    p.q = (const __bf16*)q;
+    p.k_cache = k_cache;
+    p.v_cache = v_cache;
+    p.out = (__bf16*)out;
+    p.block_tables = block_tables;
+    p.bt_row_stride = bt_row_stride;
+    p.context_lens = context_lens;
+    p.k_scale = k_scale;
+    p.v_scale = v_scale;
+    const size_t rows = (size_t)B * Hq * max_chunks;
+    char* ws = (char*)workspace;
+    p.ws_o = (float*)ws;
+    p.ws_m = (float*)(ws + align_up(rows * D * 4, 256));
+    p.ws_l = (float*)(ws + align_up(rows * D * 4, 256) + align_up(rows * 4, 256));
+    p.B = B;
+    p.Hq = Hq;
+    p.Hkv = Hkv;
+    p.max_chunks = max_chunks;
+    p.max_ctx = max_ctx;
+    p.scale_log2 = softmax_scale * kLog2e;
+
+    hipStream_t s = (hipStream_t)stream;
+    int rc;
+    if (fp8) {
+        rc = D == 128 ? launch_decode<128, true>(p, s) : launch_decode<64, true>(p, s);
+    } else {
+        rc = D == 128 ? launch_decode<128, false>(p, s)
+                      : (D == 64 ? launch_decode<64, false>(p, s) : launch_decode<32, false>(p, s));
+    }
+    if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}

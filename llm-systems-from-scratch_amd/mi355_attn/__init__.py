@@ -1,0 +1,21 @@
+"""MI355X-native attention hot path: HIP kernels for gfx950 behind the reference's Python API.
+
+Drop-in surface (same names, argument meaning and tensor conventions as
+llm-core/llm_core/model.py:308-325 and the SDPA slot at model.py:382):
+
+    scaled_dot_product_attention(Q, K, V, mask=None)
+    flash_attn_prefill(q, k, v, causal=True)            # f(Q, K, V, is_causal=True) slot
+    flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, ...)
+    paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, ...)
+
+Every function runs on the HIP library; there is no CPU or PyTorch fallback.
+"""
+from .ops import (  # noqa: F401
+    flash_attn_prefill,
+    flash_attn_varlen_prefill,
+    paged_attention_decode,
+    paged_decode_workspace,
+    scaled_dot_product_attention,
+    sdpa_slot,
+)
+from ._lib import LIB_PATH, LibraryMissing, load  # noqa: F401

@@ -1,0 +1,67 @@
+"""ctypes binding of libmi355attn.so (declarations mirror include/mi355_attn.h)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi355attn.so")
+
+MI355_BF16 = 0
+MI355_FP8_E4M3 = 1
+MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2
+
+_i64x3 = C.c_int64 * 3
+_lib = None
+
+EXPORTS = (
+    "mi355_prefill_fwd",
+    "mi355_paged_decode_fwd",
+    "mi355_paged_decode_workspace_bytes",
+    "mi355_paged_decode_chunk_tokens",
+    "mi355_last_error",
+    "mi355_version",
+)
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def load():
+    """Loads the HIP library once.  There is no fallback: a missing library is an error."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise LibraryMissing(
+            f"{LIB_PATH} is not built; run `python llm-systems-from-scratch_amd/build.py` "
+            "(needs hipcc, cross-compiles for gfx950 without a GPU)")
+    lib = C.CDLL(LIB_PATH)
+    vp, i32, i64, f32, sz = C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_size_t
+    lib.mi355_prefill_fwd.restype = i32
+    lib.mi355_prefill_fwd.argtypes = [vp, vp, vp, vp, _i64x3, _i64x3, _i64x3, _i64x3, vp, vp, vp, _i64x3,
+                                      i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
+    lib.mi355_paged_decode_fwd.restype = i32
+    lib.mi355_paged_decode_fwd.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, sz,
+                                           i32, i32, i32, i32, i32, i32, f32, i32, vp]
+    lib.mi355_paged_decode_workspace_bytes.restype = sz
+    lib.mi355_paged_decode_workspace_bytes.argtypes = [i32, i32, i32, i32]
+    lib.mi355_paged_decode_chunk_tokens.restype = i32
+    lib.mi355_paged_decode_chunk_tokens.argtypes = []
+    lib.mi355_last_error.restype = C.c_char_p
+    lib.mi355_version.restype = C.c_char_p
+    _lib = lib
+    return lib
+
+
+def strides3(values):
+    return _i64x3(*[int(v) for v in values])
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = load().mi355_last_error().decode()
+        if rc < 0:
+            raise ValueError(f"{what}: {msg} (code {rc})")
+        raise RuntimeError(f"{what}: HIP error {rc}: {msg}")

@@ -1,0 +1,228 @@
+"""Host-side operators: argument checking, output allocation, C-ABI calls.
+
+Tensor conventions follow the reference attention module
+(llm-core/llm_core/model.py:366-388): Q/K/V are (batch, heads, seq, d_head) with
+arbitrary batch/head/seq strides (the reference's V is a strided view of the
+(batch, seq, heads*d_head) projection) and a unit innermost stride.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+_BLOCK = 16
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require_gpu_bf16(name, t):
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got {t.device}); this library has no CPU path")
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be bfloat16 (got {t.dtype})")
+
+
+def _rows16(name, t):
+    """Return `t` with unit innermost stride and 16-byte aligned rows (copy only if needed)."""
+    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+    return t if ok else t.contiguous()
+
+
+def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode):
+    lib = _lib.load()
+    if cu_q is None:
+        qs, ks, vs, os_ = (x.stride()[:3] for x in (q, k, v, out))
+    else:   # packed (T, H, D): [batch (unused), head, row]
+        qs, ks, vs, os_ = ((0, x.stride(1), x.stride(0)) for x in (q, k, v, out))
+    ms = (0, 0, 0) if mask is None else mask.stride()[:3]
+    rc = lib.mi355_prefill_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+        _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
+        None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(),
+        None if mask is None else mask.data_ptr(), _lib.strides3(ms),
+        B, Hq, Hkv, Sq, Sk, D, float(scale), mode, _lib.MI355_BF16, _stream())
+    _lib.check(rc, "mi355_prefill_fwd")
+
+
+def _dense(q, k, v, mask, mode, softmax_scale):
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        _require_gpu_bf16(n, t)
+        if t.dim() != 4:
+            raise ValueError(f"{n} must be (batch, heads, seq, d_head), got {tuple(t.shape)}")
+    B, Hq, Sq, D = q.shape
+    Bk, Hkv, Sk, Dk = k.shape
+    if (Bk, Dk) != (B, D) or tuple(v.shape) != (B, Hkv, Sk, D):
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if Hq % Hkv:
+        raise ValueError("query heads must be a multiple of kv heads")
+    q, k, v = _rows16("q", q), _rows16("k", k), _rows16("v", v)
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    # (B, S, H, D) memory returned as its (B, H, S, D) view: merging heads afterwards
+    # (model.py:388) is then a free reshape instead of a copy.
+    out = torch.empty(B, Sq, Hq, D, dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
+    if B == 0 or Sq == 0:
+        return out
+    if Sk == 0:
+        raise ValueError("attention over zero keys is undefined")
+    _prefill(q, k, v, out, None, None, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode)
+    return out
+
+
+def flash_attn_prefill(q, k, v, *, causal=True, softmax_scale=None):
+    """Prefill forward.  q (B,Hq,Sq,D); k, v (B,Hkv,Sk,D) bf16 -> (B,Hq,Sq,D) bf16.
+
+    Fills the slot of torch.nn.functional.scaled_dot_product_attention(Q, K, V,
+    is_causal=True) at llm-core/llm_core/model.py:382.  With Sk > Sq the causal
+    diagonal is bottom-right aligned (the queries are the last Sq positions).
+    """
+    return _dense(q, k, v, None, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, softmax_scale)
+
+
+def sdpa_slot(Q, K, V, is_causal=True):
+    """Callable with the exact call shape used at llm-core/llm_core/model.py:382."""
+    return flash_attn_prefill(Q, K, V, causal=is_causal)
+
+
+def scaled_dot_product_attention(Q, K, V, mask=None):
+    """Same signature and semantics as llm-core/llm_core/model.py:308-325.
+
+    Q (..., queries, d_k), K (..., keys, d_k), V (..., keys, d_v); `mask` is a
+    boolean keep-mask (True = attend) broadcastable to (..., queries, keys); the
+    scale is 1/sqrt(d_k).  A query row whose keys are all masked yields NaN, as
+    the reference softmax (llm-core/llm_core/nn_functional.py:8-11) does.
+    Restriction of the HIP path: bf16 tensors, d_v == d_k in {32, 64, 128}.
+    """
+    if Q.dim() < 2 or K.dim() != Q.dim() or V.dim() != Q.dim():
+        raise ValueError("Q, K and V need the same number of dimensions (>= 2)")
+    lead = torch.broadcast_shapes(Q.shape[:-2], K.shape[:-2], V.shape[:-2])
+    nq, nk, d = Q.shape[-2], K.shape[-2], Q.shape[-1]
+    if mask is not None:
+        if mask.dtype != torch.bool:
+            raise TypeError("mask must be a boolean keep-mask")
+        lead = torch.broadcast_shapes(lead, mask.shape[:-2])
+
+    def as4(t, rows):
+        t = t.expand(*lead, rows, t.shape[-1])
+        if t.dim() == 4:
+            return t
+        if t.dim() < 4:
+            return t.reshape((1,) * (4 - t.dim()) + tuple(t.shape))
+        return t.reshape(-1, *t.shape[-3:])
+
+    q4, k4, v4 = as4(Q, nq), as4(K, nk), as4(V, nk)
+    m4 = None
+    mode = _lib.MASK_NONE
+    if mask is not None:
+        m4 = as4(mask.expand(*mask.shape[:-2], nq, nk), nq).view(torch.uint8)
+        if m4.stride(-1) != 1:
+            m4 = m4.contiguous()
+        mode = _lib.MASK_BOOL
+    out = _dense(q4, k4, v4, m4, mode, None)
+    return out.reshape(*lead, nq, d)
+
+
+def flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, *,
+                              causal=True, softmax_scale=None):
+    """Packed ("varlen") prefill.  q (Tq,Hq,D); k, v (Tk,Hkv,D) bf16; cu_seqlens int32 (B+1,), cu[0]=0.
+
+    Sequence b owns rows [cu[b], cu[b+1]).  Returns (Tq,Hq,D) bf16.
+    """
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        _require_gpu_bf16(n, t)
+        if t.dim() != 3:
+            raise ValueError(f"{n} must be (tokens, heads, d_head), got {tuple(t.shape)}")
+    for n, c in (("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
+        if c.dtype != torch.int32 or not c.is_cuda or c.dim() != 1 or not c.is_contiguous():
+            raise TypeError(f"{n} must be a contiguous 1-D int32 GPU tensor")
+    if cu_seqlens_q.numel() != cu_seqlens_k.numel() or cu_seqlens_q.numel() < 2:
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must both have batch+1 entries")
+    Tq, Hq, D = q.shape
+    Tk, Hkv, Dk = k.shape
+    if Dk != D or tuple(v.shape) != (Tk, Hkv, D) or Hq % Hkv:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    q, k, v = _rows16("q", q), _rows16("k", k), _rows16("v", v)
+    B = cu_seqlens_q.numel() - 1
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    out = torch.empty(Tq, Hq, D, dtype=q.dtype, device=q.device)
+    if Tq == 0 or max_seqlen_q == 0:
+        return out
+    _prefill(q, k, v, out, cu_seqlens_q, cu_seqlens_k, None, B, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k),
+             D, scale, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE)
+    return out
+
+
+def paged_decode_workspace(batch, n_q_heads, head_dim, max_context, device):
+    """Scratch tensor for paged_attention_decode (reusable across calls of the same or smaller shape)."""
+    n = _lib.load().mi355_paged_decode_workspace_bytes(batch, n_q_heads, head_dim, max_context)
+    return torch.empty(max(int(n), 16), dtype=torch.uint8, device=device)
+
+
+def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, softmax_scale=None,
+                           k_scale=None, v_scale=None, max_context=None, workspace=None, out=None):
+    """Paged-KV decode attention, one query token per sequence.
+
+    q (B,Hq,D) bf16; k_cache, v_cache (num_blocks,Hkv,16,D) bf16, or fp8-e4m3
+    (torch.float8_e4m3fn / uint8 bit patterns) when k_scale and v_scale
+    (num_blocks,Hkv) fp32 are given; block_tables (B,max_blocks) int32;
+    context_lens (B,) int32 >= 1.  `max_context` bounds context_lens (default:
+    block_tables.shape[1]*16) so no device->host sync is needed.  Returns (B,Hq,D) bf16.
+    """
+    _require_gpu_bf16("q", q)
+    if q.dim() != 3:
+        raise ValueError(f"q must be (batch, heads, d_head), got {tuple(q.shape)}")
+    B, Hq, D = q.shape
+    fp8 = k_scale is not None or v_scale is not None
+    if fp8:
+        if k_scale is None or v_scale is None:
+            raise ValueError("k_scale and v_scale must be given together")
+        for n, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+            if c.dtype not in (torch.uint8, torch.float8_e4m3fn):
+                raise TypeError(f"{n} must be float8_e4m3fn or uint8 when scales are given (got {c.dtype})")
+    else:
+        for n, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+            if c.dtype != torch.bfloat16:
+                raise TypeError(f"{n} must be bfloat16 (got {c.dtype}); pass k_scale/v_scale for an fp8 cache")
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
+        raise ValueError("k_cache and v_cache must both be (num_blocks, kv_heads, 16, d_head)")
+    nb, Hkv, bs, Dc = k_cache.shape
+    if bs != _BLOCK or Dc != D:
+        raise ValueError(f"cache must be (num_blocks, kv_heads, {_BLOCK}, {D}), got {tuple(k_cache.shape)}")
+    for n, c in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache)):
+        if not c.is_contiguous() or not c.is_cuda:
+            raise ValueError(f"{n} must be a contiguous GPU tensor")
+    if block_tables.dtype != torch.int32 or context_lens.dtype != torch.int32:
+        raise TypeError("block_tables and context_lens must be int32")
+    if block_tables.dim() != 2 or block_tables.shape[0] != B or block_tables.stride(1) != 1:
+        raise ValueError("block_tables must be (batch, max_blocks) with unit column stride")
+    if context_lens.shape != (B,) or not context_lens.is_contiguous():
+        raise ValueError("context_lens must be a contiguous (batch,) tensor")
+    if fp8:
+        for n, s in (("k_scale", k_scale), ("v_scale", v_scale)):
+            if s.dtype != torch.float32 or tuple(s.shape) != (nb, Hkv) or not s.is_contiguous():
+                raise ValueError(f"{n} must be a contiguous float32 (num_blocks, kv_heads) tensor")
+    if max_context is None:
+        max_context = block_tables.shape[1] * _BLOCK
+    if max_context > block_tables.shape[1] * _BLOCK:
+        raise ValueError("max_context exceeds what block_tables can address")
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    if out is None:
+        out = torch.empty_like(q)
+    if B == 0:
+        return out
+    lib = _lib.load()
+    if workspace is None:
+        workspace = paged_decode_workspace(B, Hq, D, max_context, q.device)
+    rc = lib.mi355_paged_decode_fwd(
+        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+        block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
+        k_scale.data_ptr() if fp8 else None, v_scale.data_ptr() if fp8 else None,
+        workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+        B, Hq, Hkv, D, bs, int(max_context), float(scale),
+        _lib.MI355_FP8_E4M3 if fp8 else _lib.MI355_BF16, _stream())
+    _lib.check(rc, "mi355_paged_decode_fwd")
+    return out
