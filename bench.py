@@ -1,0 +1,270 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A "step" is one pass of paged-KV decode attention (split-K pass + combine) over the
+whole batch of configs[3]: bf16 KV cache, batch 128, 32 query / 8 kv heads, head_dim
+128, block 16, ragged context lengths ~ U[512, 16384] (seeded), physical blocks a
+random permutation of a pool sized 1.1x.  Inputs are resident in HBM before timing.
+`value` is algorithmic bytes / wall time per step.  The same JSON line also carries
+the prefill measurement at configs[2] (bf16, packed varlen, B8, 32/8 heads, D128,
+S4096, causal) and the fp8-KV decode at configs[4], each with its own roofline.
+
+The CPU baseline is the oracle (a restatement of the reference's PyTorch attention)
+timed on the host cores over a bounded sample of the same inputs; its outputs also
+check the GPU results of that sample.
+
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--seed S] [--only decode|prefill|fp8]
+                       [--no-cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "llm-systems-from-scratch_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+METRIC = "paged-decode attn HBM GB/s (% of 8 TB/s) + prefill attn TFLOP/s (% MFMA peak)"
+
+
+def _traffic(key):
+    """HBM bytes per launch measured with rocprofv3 --pmc (kept as data under profiles/)."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+
+
+def timed(fn, steps, warmup):
+    """Returns (wall ms/step, device ms/step): K launches between two syncs, HIP events on the launch stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+
+def bench_decode(cfg, args, with_cpu):
+    import torch
+    import mi355_attn
+    from mi355_attn import workloads
+
+    case = workloads.decode_config(cfg, seed=args.seed)
+    B, Hq, D = case.q.shape
+    ws = mi355_attn.paged_decode_workspace(B, Hq, D, case.max_context, case.q.device)
+    out = torch.empty_like(case.q)
+
+    def step():
+        mi355_attn.paged_attention_decode(case.q, case.k_cache, case.v_cache, case.block_tables, case.context_lens,
+                                          k_scale=case.k_scale, v_scale=case.v_scale, max_context=case.max_context,
+                                          workspace=ws, out=out)
+
+    wall_ms, dev_ms = timed(step, args.steps, args.warmup)
+    nbytes = case.algorithmic_bytes()
+    res = {
+        "value": nbytes / wall_ms / 1e6,
+        "unit": "GB/s",
+        "ms_per_step": wall_ms,
+        "tokens": case.tokens,
+        "algorithmic_bytes": nbytes,
+        "roofline": {
+            "bound": "hbm", "kernel": "paged_decode_split_kernel (+ combine, same launch sequence)",
+            "achieved": nbytes / dev_ms / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS, "device_ms": dev_ms,
+            "traffic": _traffic(f"decode_cfg{cfg}"),
+        },
+    }
+    if with_cpu:
+        res["cpu_baseline"], res["parity"] = cpu_decode(case, out, cfg)
+    return res
+
+
+def cpu_decode(case, gpu_out, cfg, n_seq=48):
+    """Oracle on the host cores over the first n_seq sequences; also checks the GPU result of those."""
+    import torch
+    from oracle import attention_oracle as orc
+
+    n_seq = min(n_seq, case.q.shape[0])
+    ctx = case.context_lens_host[:n_seq]
+    nblk = (ctx + 15) // 16
+    ids = torch.cat([case.block_tables[b, :int(nblk[b])] for b in range(n_seq)]).long()
+    kc = case.k_cache[ids].cpu()
+    vc = case.v_cache[ids].cpu()
+    ks = case.k_scale[ids].cpu() if case.k_scale is not None else None
+    vs = case.v_scale[ids].cpu() if case.v_scale is not None else None
+    bt = torch.zeros(n_seq, int(nblk.max()), dtype=torch.int32)
+    off = 0
+    for b in range(n_seq):
+        bt[b, :int(nblk[b])] = torch.arange(off, off + int(nblk[b]), dtype=torch.int32)
+        off += int(nblk[b])
+    q = case.q[:n_seq].cpu()
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    t0 = time.perf_counter()
+    ref = orc.paged_decode_reference(q, kc, vc, bt, ctx, k_scale=ks, v_scale=vs)
+    dt = time.perf_counter() - t0
+    per_token = 2 * kc.shape[1] * kc.shape[3] * kc.element_size() + (8 * kc.shape[1] / 16 if ks is not None else 0)
+    sample_bytes = int(ctx.sum()) * per_token
+    err = (gpu_out[:n_seq].float().cpu() - ref).abs()
+    bound = 2e-2 + 1e-2 * ref.abs()
+    base = {"value": sample_bytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "seconds": dt,
+            "sample": f"configs[{cfg}] first {n_seq} of {case.q.shape[0]} sequences ({int(ctx.sum())} tokens), "
+                      "oracle paged_decode_reference, torch CPU fp32"}
+    parity = {"checked_sequences": n_seq, "max_abs_err": float(err.max()),
+              "within_2e-2_abs_1e-2_rel": bool((err <= bound).all())}
+    return base, parity
+
+
+def bench_prefill(cfg, args, with_cpu):
+    import torch
+    import mi355_attn
+    from mi355_attn import workloads
+
+    case = workloads.prefill_config(cfg, seed=args.seed)
+    holder = {}
+
+    if case.cu_seqlens is not None:
+        def step():
+            holder["out"] = mi355_attn.flash_attn_varlen_prefill(case.q, case.k, case.v, case.cu_seqlens,
+                                                                 case.cu_seqlens, case.seqlen, case.seqlen, causal=True)
+    else:
+        def step():
+            holder["out"] = mi355_attn.flash_attn_prefill(case.q, case.k, case.v, causal=True)
+
+    wall_ms, dev_ms = timed(step, args.steps, args.warmup)
+    flops = case.flops()
+    res = {
+        "value": flops / wall_ms / 1e9,
+        "unit": "TFLOP/s",
+        "ms_per_step": wall_ms,
+        "algorithmic_flops": flops,
+        "roofline": {
+            "bound": "mfma", "kernel": "prefill_fwd_kernel",
+            "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms,
+            "traffic": _traffic(f"prefill_cfg{cfg}"),
+        },
+    }
+    if with_cpu:
+        res["cpu_baseline"], res["parity"] = cpu_prefill(case, holder["out"], cfg)
+    return res
+
+
+def cpu_prefill(case, gpu_out, cfg, n_heads=8):
+    import torch
+    from oracle import attention_oracle as orc
+
+    S = case.seqlen
+    if case.cu_seqlens is not None:          # packed (T, H, D): sequence 0, first n_heads query heads
+        Hq, Hkv = case.q.shape[1], case.k.shape[1]
+        n_heads = min(n_heads, Hq)
+        n_kv = max(1, n_heads * Hkv // Hq)
+        q = case.q[:S, :n_heads].transpose(0, 1)[None].cpu()
+        k = case.k[:S, :n_kv].transpose(0, 1)[None].cpu()
+        v = case.v[:S, :n_kv].transpose(0, 1)[None].cpu()
+        got = gpu_out[:S, :n_heads].transpose(0, 1)[None].float().cpu()
+    else:
+        n_heads = min(n_heads, case.q.shape[1])
+        q, k, v = (t[:1, :n_heads].cpu() for t in (case.q, case.k, case.v))
+        got = gpu_out[:1, :n_heads].float().cpu()
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    t0 = time.perf_counter()
+    ref = orc.prefill_reference(q, k, v, causal=True, head_chunk=4)
+    dt = time.perf_counter() - t0
+    flops = 4 * n_heads * q.shape[-1] * S * S // 2
+    err = (got - ref).abs()
+    bound = 2e-2 + 1e-2 * ref.abs()
+    base = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "seconds": dt,
+            "sample": f"configs[{cfg}] sequence 0, query heads 0..{n_heads - 1} (S={S}), oracle prefill_reference, "
+                      "torch CPU fp32, causal-convention FLOPs"}
+    parity = {"checked_heads": n_heads, "max_abs_err": float(err.max()),
+              "within_2e-2_abs_1e-2_rel": bool((err <= bound).all())}
+    return base, parity
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--only", choices=["decode", "prefill", "fp8"], default=None)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path needs no exchange between GPUs; "
+              "see DESIGN.md for how it would shard). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import mi355_attn
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    mi355_attn.load()
+    torch.cuda.set_device(0)
+    with_cpu = not args.no_cpu
+
+    line = {
+        "metric": METRIC, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic (seeded)",
+    }
+    dec = None
+    if args.only in (None, "decode"):
+        dec = bench_decode(3, args, with_cpu)
+        line.update({
+            "value": dec["value"], "unit": "GB/s", "ms_per_step": dec["ms_per_step"], "dtype": "bf16",
+            "config": {"workload": "configs[3]: paged decode attention, bf16 KV cache, batch 128, 32 q / 8 kv heads, "
+                                   "head_dim 128, block 16, ctx ~ U[512,16384], pool 1.1x, seed %d" % args.seed,
+                       "tokens": dec["tokens"], "algorithmic_bytes": dec["algorithmic_bytes"]},
+            "roofline": dec["roofline"],
+        })
+        if with_cpu:
+            line["cpu_baseline"] = dec["cpu_baseline"]
+            line["parity"] = dec["parity"]
+    if args.only in (None, "prefill"):
+        pre = bench_prefill(2, args, with_cpu)
+        pre["config"] = {"workload": "configs[2]: causal prefill forward, bf16, packed varlen, batch 8, 32 q / 8 kv "
+                                     "heads, head_dim 128, seq 4096, seed %d" % args.seed}
+        pre["dtype"] = "bf16"
+        line["prefill"] = pre
+        if dec is None and args.only == "prefill":
+            line.update({"value": pre["value"], "unit": "TFLOP/s", "ms_per_step": pre["ms_per_step"], "dtype": "bf16",
+                         "config": pre["config"], "roofline": pre["roofline"]})
+            if with_cpu:
+                line["cpu_baseline"] = pre["cpu_baseline"]
+    if args.only in (None, "fp8"):
+        f8 = bench_decode(4, args, with_cpu)
+        f8["config"] = {"workload": "configs[4]: paged decode attention, fp8-e4m3 KV cache + per-(block, kv head) fp32 "
+                                    "scales, batch 256, 64 q / 8 kv heads, head_dim 128, block 16, ctx log-uniform "
+                                    "[128,32768], seed %d" % args.seed}
+        f8["dtype"] = "fp8 KV / bf16 math"
+        line["decode_fp8"] = f8
+        if args.only == "fp8":
+            line.update({"value": f8["value"], "unit": "GB/s", "ms_per_step": f8["ms_per_step"],
+                         "dtype": f8["dtype"], "config": f8["config"], "roofline": f8["roofline"]})
+            if with_cpu:
+                line["cpu_baseline"] = f8["cpu_baseline"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
