@@ -208,6 +208,8 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", choices=["decode", "prefill", "fp8"], default=None)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="only run the 1 GiB plain copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path needs no exchange between GPUs; "
@@ -222,6 +224,17 @@ def main():
     mi355_attn.load()
     torch.cuda.set_device(0)
     with_cpu = not args.no_cpu
+    if args.calibrate:
+        from mi355_attn import _lib
+        n = 1 << 30
+        a = torch.full((n,), 1, dtype=torch.uint8, device="cuda:0")
+        b = torch.empty_like(a)
+        for _ in range(max(1, args.steps)):
+            _lib.check(_lib.load().mi355_calib_copy(a.data_ptr(), b.data_ptr(), n,
+                                                    torch.cuda.current_stream().cuda_stream), "mi355_calib_copy")
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "mi355_calib_copy", "bytes_read": n, "bytes_written": n}))
+        return
 
     line = {
         "metric": METRIC, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -106,6 +106,13 @@ size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx);
 /* Tokens of one sequence handled by one workgroup of the split-K pass. */
 int mi355_paged_decode_chunk_tokens(void);
 
+/*
+ * Plain device-to-device copy of `bytes` bytes (16-byte aligned).  Measurement aid
+ * with no counterpart in the reference: a copy of known size whose FETCH_SIZE /
+ * WRITE_SIZE counter readings calibrate the HBM-traffic figures of the kernels above.
+ */
+int mi355_calib_copy(const void* src, void* dst, size_t bytes, void* stream);
+
 const char* mi355_last_error(void);
 const char* mi355_version(void);
 

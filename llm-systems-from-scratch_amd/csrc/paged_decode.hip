@@ -68,9 +68,13 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
 
     __shared__ __attribute__((aligned(16))) unsigned char smem[kDecodeWaves * kWaveBytes];
 
-    const int chunk = blockIdx.x;
-    const int hk = blockIdx.y;
-    const int b = blockIdx.z;
+    // 1-D grid, kv head fastest, then sequence, chunk slowest.  Workgroup ids are dealt
+    // round-robin to the 8 XCDs, so the low bits of the id must not select the chunk:
+    // with ragged lengths late chunks are mostly empty and the XCDs that own them would idle.
+    const int wg = blockIdx.x;
+    const int hk = wg % p.Hkv;
+    const int b = (wg / p.Hkv) % p.B;
+    const int chunk = wg / (p.Hkv * p.B);
     const int ctx = min(p.context_lens[b], p.max_ctx);     // a length beyond the promised bound is truncated, never chased
     const int chunk_start = chunk * kChunk;
     if (chunk_start >= ctx) return;
@@ -105,41 +109,55 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
     const int last_blk = (ctx - 1) / kBlock;
     const int32_t* bt = p.block_tables + (int64_t)b * p.bt_row_stride;
 
-    struct Stage {
-        u32x4 k[2][KL];
-        u32x4 v[2][VL];
-        float ks[2], vs[2];
-    };
+    // Block ids (and fp8 scales) of this wavefront's token range, one block per lane, fetched
+    // once: lane l holds logical block t0/16 + l, clamped to the sequence's last block so that
+    // every id is a real block.  The step loop reads them with v_readlane, so no dependent
+    // table load sits between two steps.
+    const int my_phys = bt[min(t0 / kBlock + lane, last_blk)];
+    float my_ks = 1.0f, my_vs = 1.0f;
+    if constexpr (FP8) {
+        my_ks = p.k_scale[(int64_t)my_phys * p.Hkv + hk];
+        my_vs = p.v_scale[(int64_t)my_phys * p.Hkv + hk];
+    }
 
-    auto issue = [&](int it, Stage& st) {
-        const int bi0 = (t0 + it * kStage) / kBlock;
+    u32x4 kreg[2][KL];
+    u32x4 vreg[2][VL];
+
+    auto slab_of = [&](int blk) -> int64_t {     // element offset of (block, kv head) in the cache
+        const int64_t phys = __builtin_amdgcn_readlane(my_phys, blk);
+        return (phys * p.Hkv + hk) * (int64_t)(kBlock * D);
+    };
+    auto load_k = [&](int it) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int bi = min(bi0 + t, last_blk);          // never read past the table
-            const int64_t phys = bt[bi];
-            const int64_t slab = (phys * p.Hkv + hk) * (int64_t)(kBlock * D);   // elements
+            const int64_t slab = slab_of(2 * it + t);
             if constexpr (FP8) {
                 const unsigned char* kb = reinterpret_cast<const unsigned char*>(p.k_cache) + slab;
-                const unsigned char* vb = reinterpret_cast<const unsigned char*>(p.v_cache) + slab;
 #pragma unroll
                 for (int j = 0; j < KL; ++j)
-                    st.k[t][j] = *reinterpret_cast<const u32x4*>(kb + r * D + 64 * j + 16 * kg);
-#pragma unroll
-                for (int j = 0; j < VL; ++j)
-                    st.v[t][j] = *reinterpret_cast<const u32x4*>(vb + (j * 64 + lane) * 16);
-                st.ks[t] = p.k_scale[phys * p.Hkv + hk];
-                st.vs[t] = p.v_scale[phys * p.Hkv + hk];
+                    kreg[t][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb + r * D + 64 * j + 16 * kg));
             } else {
                 const __bf16* kb = reinterpret_cast<const __bf16*>(p.k_cache) + slab;
-                const __bf16* vb = reinterpret_cast<const __bf16*>(p.v_cache) + slab;
 #pragma unroll
                 for (int s = 0; s < KL; ++s)
-                    st.k[t][s] = *reinterpret_cast<const u32x4*>(kb + r * D + 32 * s + 8 * kg);
+                    kreg[t][s] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb + r * D + 32 * s + 8 * kg));
+            }
+        }
+    };
+    auto load_v = [&](int it) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int64_t slab = slab_of(2 * it + t);
+            if constexpr (FP8) {
+                const unsigned char* vb = reinterpret_cast<const unsigned char*>(p.v_cache) + slab;
 #pragma unroll
                 for (int j = 0; j < VL; ++j)
-                    st.v[t][j] = *reinterpret_cast<const u32x4*>(vb + (j * 64 + lane) * 8);
-                st.ks[t] = 1.0f;
-                st.vs[t] = 1.0f;
+                    vreg[t][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vb + (j * 64 + lane) * 16));
+            } else {
+                const __bf16* vb = reinterpret_cast<const __bf16*>(p.v_cache) + slab;
+#pragma unroll
+                for (int j = 0; j < VL; ++j)
+                    vreg[t][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vb + (j * 64 + lane) * 8));
             }
         }
     };
@@ -150,7 +168,16 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
 #pragma unroll
     for (int i = 0; i < NT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto compute = [&](int it, Stage& st) {
+    // Software pipeline without double buffering: the registers of step `it` are refilled for
+    // step it+1 as soon as they have been consumed (V after its copy to LDS, K after K.Q^T), so
+    // the next step's loads fly during this step's softmax and P.V.  The last step "prefetches"
+    // itself again (cache hits, never used): an unconditional prefetch keeps the loop free of
+    // branches, so the wait counts stay exact.
+    if (n_iter > 0) {
+        load_v(0);
+        load_k(0);
+    }
+    for (int it = 0; it < n_iter; ++it) {
         const int kbase = t0 + it * kStage;
         const bool tail = kbase + kStage > t1;
 
@@ -162,7 +189,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
                 if constexpr (FP8) {
                     const int e = (j * 64 + lane) * 16;     // element index in the block slab
                     const int row = e / D, col = e % D;
-                    u32x4 raw = st.v[t][j];
+                    u32x4 raw = vreg[t][j];
                     if (tail && kbase + 16 * t + row >= t1) raw = u32x4{0u, 0u, 0u, 0u};
                     u32x2 a = fp8x4_to_bf16x4(raw[0]), bq = fp8x4_to_bf16x4(raw[1]);
                     u32x2 c = fp8x4_to_bf16x4(raw[2]), dq = fp8x4_to_bf16x4(raw[3]);
@@ -172,12 +199,13 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
                 } else {
                     const int e = (j * 64 + lane) * 8;
                     const int row = e / D, col = e % D;
-                    u32x4 raw = st.v[t][j];
+                    u32x4 raw = vreg[t][j];
                     if (tail && kbase + 16 * t + row >= t1) raw = u32x4{0u, 0u, 0u, 0u};
                     *reinterpret_cast<u32x4*>(wsm + (16 * t + row) * kVRow + col * 2) = raw;
                 }
             }
         }
+        load_v(min(it + 1, n_iter - 1));
 
         // ---- S^T = K . Q^T ---------------------------------------------------
         f32x4 s_acc[2];
@@ -187,7 +215,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
             if constexpr (FP8) {
 #pragma unroll
                 for (int j = 0; j < KL; ++j) {
-                    u32x4 raw = st.k[t][j];
+                    u32x4 raw = kreg[t][j];
                     u32x2 a = fp8x4_to_bf16x4(raw[0]), bq = fp8x4_to_bf16x4(raw[1]);
                     u32x2 c = fp8x4_to_bf16x4(raw[2]), dq = fp8x4_to_bf16x4(raw[3]);
                     s_acc[t] = mfma16(as_bf16x8(u32x4{a[0], a[1], bq[0], bq[1]}), qf[2 * j], s_acc[t]);
@@ -195,16 +223,25 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
                 }
             } else {
 #pragma unroll
-                for (int s = 0; s < NS; ++s) s_acc[t] = mfma16(as_bf16x8(st.k[t][s]), qf[s], s_acc[t]);
+                for (int s = 0; s < NS; ++s) s_acc[t] = mfma16(as_bf16x8(kreg[t][s]), qf[s], s_acc[t]);
             }
         }
+        load_k(min(it + 1, n_iter - 1));
 
         // ---- online softmax (lane: query column r, keys 16t + 4kg + i) -------
+        float ks2[2] = {1.0f, 1.0f}, vs2[2] = {1.0f, 1.0f};
+        if constexpr (FP8) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                ks2[t] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_ks), 2 * it + t));
+                vs2[t] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_vs), 2 * it + t));
+            }
+        }
         float x[8];
         float mx = -INFINITY;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const float sc = p.scale_log2 * st.ks[t];
+            const float sc = p.scale_log2 * ks2[t];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float v = s_acc[t][i] * sc;
@@ -227,10 +264,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
 #pragma unroll
         for (int i = 0; i < NT; ++i) o[i] *= alpha;
         u32x4 pp;
-        pp[0] = pack_bf16(x[0] * st.vs[0], x[1] * st.vs[0]);
-        pp[1] = pack_bf16(x[2] * st.vs[0], x[3] * st.vs[0]);
-        pp[2] = pack_bf16(x[4] * st.vs[1], x[5] * st.vs[1]);
-        pp[3] = pack_bf16(x[6] * st.vs[1], x[7] * st.vs[1]);
+        pp[0] = pack_bf16(x[0] * vs2[0], x[1] * vs2[0]);
+        pp[1] = pack_bf16(x[2] * vs2[0], x[3] * vs2[0]);
+        pp[2] = pack_bf16(x[4] * vs2[1], x[5] * vs2[1]);
+        pp[3] = pack_bf16(x[6] * vs2[1], x[7] * vs2[1]);
         const bf16x8 pf = as_bf16x8(pp);
 
         // ---- O^T += V^T . P^T -------------------------------------------------
@@ -242,19 +279,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
             i16x4 hi = lds_read_tr16(vsrc + 16 * kVRow + dt * 32);
             o[dt] = mfma16(join_bf16x8(lo, hi), pf, o[dt]);
         }
-    };
-
-    {
-        Stage sa, sb;
-        if (n_iter > 0) issue(0, sa);
-        for (int it = 0; it < n_iter; it += 2) {
-            if (it + 1 < n_iter) issue(it + 1, sb);
-            compute(it, sa);
-            if (it + 1 < n_iter) {
-                if (it + 2 < n_iter) issue(it + 2, sa);
-                compute(it + 1, sb);
-            }
-        }
+        // Compiler barrier: without a may-write instruction after the prefetch loads, the
+        // optimiser turns "phi of loads" into "load of phi" and the loads land at the top of
+        // the NEXT iteration, i.e. the prefetch is undone.
+        asm volatile("" ::: "memory");
     }
 
     // ---- merge the four wavefronts ------------------------------------------
@@ -326,7 +354,7 @@ __global__ __launch_bounds__(D) void paged_decode_combine_kernel(DecodeParams p)
 
 template <int D, bool FP8>
 static int launch_decode(const DecodeParams& p, hipStream_t stream) {
-    dim3 grid(p.max_chunks, p.Hkv, p.B);
+    dim3 grid((unsigned)p.max_chunks * p.Hkv * p.B);
     hipLaunchKernelGGL((paged_decode_split_kernel<D, FP8>), grid, dim3(kDecodeWaves * 64), 0, stream, p);
     if (p.max_chunks > 1)
         hipLaunchKernelGGL((paged_decode_combine_kernel<D>), dim3(p.B * p.Hq), dim3(D), 0, stream, p);
@@ -361,7 +389,8 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
     if (Hq % Hkv != 0 || Hq / Hkv > 16)
         return set_error(MI355_EINVAL, "paged_decode: Hq must be a multiple of Hkv with Hq/Hkv <= 16");
     if (block_size != kBlock) return set_error(MI355_EINVAL, "paged_decode: block_size must be 16");
-    if (Hkv > 65535 || B > 65535) return set_error(MI355_EINVAL, "paged_decode: Hkv and B must be <= 65535");
+    if ((int64_t)((max_ctx + kChunk - 1) / kChunk) * Hkv * B > 0x7fffffffLL)
+        return set_error(MI355_EINVAL, "paged_decode: chunks * Hkv * B exceeds the grid limit");
     if (kv_dtype != MI355_BF16 && kv_dtype != MI355_FP8_E4M3)
         return set_error(MI355_EDTYPE, "paged_decode: kv_dtype must be MI355_BF16 or MI355_FP8_E4M3");
     const bool fp8 = kv_dtype == MI355_FP8_E4M3;

@@ -19,6 +19,7 @@ EXPORTS = (
     "mi355_paged_decode_fwd",
     "mi355_paged_decode_workspace_bytes",
     "mi355_paged_decode_chunk_tokens",
+    "mi355_calib_copy",
     "mi355_last_error",
     "mi355_version",
 )
@@ -49,6 +50,8 @@ def load():
     lib.mi355_paged_decode_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.mi355_paged_decode_chunk_tokens.restype = i32
     lib.mi355_paged_decode_chunk_tokens.argtypes = []
+    lib.mi355_calib_copy.restype = i32
+    lib.mi355_calib_copy.argtypes = [vp, vp, sz, vp]
     lib.mi355_last_error.restype = C.c_char_p
     lib.mi355_version.restype = C.c_char_p
     _lib = lib
