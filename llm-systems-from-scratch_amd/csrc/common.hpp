@@ -103,4 +103,20 @@ __device__ __forceinline__ float xor32_sum(float v) {
     return a + b;
 }
 
+// ---- direct global -> LDS loads ---------------------------------------------
+// global_load_lds_dwordx4: every lane supplies its own 16-byte global address; the
+// wavefront's 64 x 16 bytes land at lds_base + 16*lane (lds_base is wave-uniform).
+// The compiler does NOT track these loads when it places wait counts for later LDS
+// reads, so every consumer must be preceded by wait_vmcnt<N>() (N = number of
+// younger vector-memory instructions of this wavefront allowed to stay in flight).
+__device__ __forceinline__ void load_to_lds_16(const void* gptr, void* lds_base) {
+    __builtin_amdgcn_global_load_lds(gptr, (MI355_LDS void*)lds_base, 16, 0, 0);
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+
 }  // namespace mi355

@@ -1,8 +1,8 @@
 // FlashAttention-style prefill forward for gfx950 (bf16, MFMA 32x32x16).
 //
 // One workgroup = 4 wavefronts = one tile of 128 queries of one (batch, head);
-// each wavefront owns 32 query rows.  K/V tiles of 64 keys are staged in LDS and
-// shared by the four wavefronts.  Per wavefront and KV tile:
+// each wavefront owns 32 query rows.  K/V tiles of 64 keys are double-buffered in
+// LDS and shared by the four wavefronts.  Per wavefront and KV tile:
 //
 //   S^T (64 keys x 32 queries) = K . Q^T     K fragments: ds_read_b128 from LDS,
 //                                            Q^T fragments live in registers
@@ -16,6 +16,13 @@
 // Working on the transposed problem is what makes the S accumulator layout equal
 // to the B-operand layout of the second MFMA (up to a key permutation that the
 // V^T read mirrors).
+//
+// Tiles travel global -> LDS with global_load_lds_dwordx4 (no staging registers).
+// Such a load writes 1 KiB of consecutive LDS per wavefront, so rows cannot be
+// padded; bank conflicts are avoided by an XOR swizzle instead: the 16-byte chunk
+// c of row r is stored in slot c ^ swz(r), applied on the global-address side.
+#include <type_traits>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -41,28 +48,30 @@ struct PrefillParams {
     int n_qtiles;
 };
 
+// XOR pattern applied to the 16-byte chunk index of LDS row `row` (rows hold D bf16).
+// Chosen so that (a) 16 lanes reading one logical chunk of 16 consecutive rows and
+// (b) a transposed read touching 4 consecutive rows x 32 bytes both spread over
+// distinct banks (LDS banks repeat every 256 bytes).
 template <int D>
-struct PrefillLds {
-    static constexpr int kKRow = D * 2 + 16;      // bytes per K row: 16-lane b128 reads hit 16 distinct 16B bank groups
-    static constexpr int kVRow = D * 2 + 64;      // bytes per V row: 4 rows x 64B of a transposed read cover all banks
-    static constexpr int kKBytes = kBN * kKRow;
-    static constexpr int kVBytes = kBN * kVRow;
-};
+__device__ __forceinline__ int swz(int row) {
+    if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+    else if constexpr (D == 64) return (((row >> 1) & 3) << 1) | ((row >> 3) & 1);
+    else return (row >> 2) & 3;
+}
 
 template <int D>
 __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillParams p) {
-    constexpr int NS = D / 16;              // MFMA k-steps of K.Q^T
-    constexpr int NDT = D / 32;             // 32-row tiles of O^T
-    constexpr int kKRow = PrefillLds<D>::kKRow;
-    constexpr int kVRow = PrefillLds<D>::kVRow;
-    constexpr int CPR = D / 8;              // 16-byte chunks per row
-    constexpr int NLD = kBN * CPR / (kPfWaves * 64);   // 16-byte staging loads per thread per tile
+    constexpr int NS = D / 16;                    // MFMA k-steps of K.Q^T
+    constexpr int NDT = D / 32;                   // 32-row tiles of O^T
+    constexpr int CPR = D / 8;                    // 16-byte chunks per row
+    constexpr int kRow = D * 2;                   // bytes per LDS row
+    constexpr int kTile = kBN * kRow;             // bytes per K (or V) tile
+    constexpr int NI = kBN * CPR / 64 / kPfWaves; // direct-to-LDS instructions per wavefront per tile and tensor
 
-    __shared__ __attribute__((aligned(16))) unsigned char k_lds[PrefillLds<D>::kKBytes];
-    __shared__ __attribute__((aligned(16))) unsigned char v_lds[PrefillLds<D>::kVBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kTile];
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kTile];
 
-    // heavy (late) query tiles first: causal work grows with the tile index
-    const int qtile = p.n_qtiles - 1 - (int)blockIdx.x;
+    const int pair = blockIdx.x;
     const int h = blockIdx.y;
     const int b = blockIdx.z;
     const int hk = h / (p.Hq / p.Hkv);
@@ -86,8 +95,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
         vb = p.v + (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
         ob = p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[1];
     }
-    const int q0 = qtile * kBM;
-    if (q0 >= sq) return;
+    // Causal work grows with the query-tile index, so a workgroup takes the tiles
+    // (nq-1-pair) and (pair): every workgroup of a sequence then carries the same load.
+    const int nq = (sq + kBM - 1) / kBM;
+    if (sk <= 0 || 2 * pair >= nq) return;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -98,170 +109,212 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
     const bool causal = p.mask_mode == MI355_MASK_CAUSAL;
     const bool boolmask = p.mask_mode == MI355_MASK_BOOL;
     const int coff = sk - sq;                          // bottom-right aligned causal diagonal
-    const int qw0 = q0 + 32 * wave;                    // first query of this wavefront
-    const int qi = qw0 + n;                            // this lane's query
-    const bool q_ok = qi < sq;
 
-    int kv_end = sk;
-    if (causal) kv_end = max(0, min(sk, min(sq, q0 + kBM) + coff));
-    const int n_tiles = (kv_end + kBN - 1) / kBN;
-
-    // ---- Q^T fragments: step s covers d = 16s + 8kg + j ----------------------
-    bf16x8 qf[NS];
+    // ---- tile loader: wavefront w, instruction j covers LDS chunks (w*NI + j)*64 .. +63 -----
+    // lane -> (row, slot); it fetches global chunk slot ^ swz(row) of that row.  The per-lane
+    // part of the address is a constant byte offset; the tile's first row is a scalar base.
+    int ld_row[NI], ld_col[NI];
+    uint32_t k_voff[NI], v_voff[NI];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        u32x4 t = {0u, 0u, 0u, 0u};
-        if (q_ok) t = *reinterpret_cast<const u32x4*>(qb + (int64_t)qi * p.qs[2] + 16 * s + 8 * kg);
-        qf[s] = as_bf16x8(t);
+    for (int j = 0; j < NI; ++j) {
+        const int idx = (wave * NI + j) * 64 + lane;
+        ld_row[j] = idx / CPR;
+        ld_col[j] = ((idx % CPR) ^ swz<D>(idx / CPR)) * 16;      // byte offset inside the row
+        k_voff[j] = (uint32_t)(ld_row[j] * (int)p.ks[2] * 2 + ld_col[j]);
+        v_voff[j] = (uint32_t)(ld_row[j] * (int)p.vs[2] * 2 + ld_col[j]);
     }
-
-    f32x16 o[NDT];
+    auto issue_tile = [&](int tile, int buf) {
+        const unsigned char* kbase = reinterpret_cast<const unsigned char*>(kb + (int64_t)tile * kBN * p.ks[2]);
+        const unsigned char* vbase = reinterpret_cast<const unsigned char*>(vb + (int64_t)tile * kBN * p.vs[2]);
+        unsigned char* kdst = k_lds + buf * kTile + wave * NI * 1024;
+        unsigned char* vdst = v_lds + buf * kTile + wave * NI * 1024;
+        if (tile * kBN + kBN <= sk) {
 #pragma unroll
-    for (int i = 0; i < NDT; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) o[i][j] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-
-    const uint8_t* mrow = nullptr;
-    if (boolmask) mrow = p.mask + (int64_t)b * p.ms[0] + (int64_t)h * p.ms[1] + (int64_t)qi * p.ms[2];
-
-    // ---- staging registers ---------------------------------------------------
-    u32x4 kst[NLD], vst[NLD];
-    auto fetch = [&](int tile) {
-#pragma unroll
-        for (int j = 0; j < NLD; ++j) {
-            const int c = tid + j * (kPfWaves * 64);
-            const int row = c / CPR, cc = c % CPR;
-            const int key = tile * kBN + row;
-            u32x4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
-            if (key < sk) {
-                kk = *reinterpret_cast<const u32x4*>(kb + (int64_t)key * p.ks[2] + cc * 8);
-                vv = *reinterpret_cast<const u32x4*>(vb + (int64_t)key * p.vs[2] + cc * 8);
+            for (int j = 0; j < NI; ++j) {
+                load_to_lds_16(kbase + k_voff[j], kdst + j * 1024);
+                load_to_lds_16(vbase + v_voff[j], vdst + j * 1024);
             }
-            kst[j] = kk;
-            vst[j] = vv;
-        }
-    };
-    auto stash = [&]() {
+        } else {
+            // last, partial tile: rows past the end re-read the last row (finite; their scores are masked)
+            const int last = sk - 1 - tile * kBN;
 #pragma unroll
-        for (int j = 0; j < NLD; ++j) {
-            const int c = tid + j * (kPfWaves * 64);
-            const int row = c / CPR, cc = c % CPR;
-            *reinterpret_cast<u32x4*>(k_lds + row * kKRow + cc * 16) = kst[j];
-            *reinterpret_cast<u32x4*>(v_lds + row * kVRow + cc * 16) = vst[j];
+            for (int j = 0; j < NI; ++j) {
+                const int row = min(ld_row[j], last);
+                load_to_lds_16(kbase + (uint32_t)(row * (int)p.ks[2] * 2 + ld_col[j]), kdst + j * 1024);
+                load_to_lds_16(vbase + (uint32_t)(row * (int)p.vs[2] * 2 + ld_col[j]), vdst + j * 1024);
+            }
         }
     };
 
-    if (n_tiles > 0) fetch(0);
-
-    for (int tile = 0; tile < n_tiles; ++tile) {
-        __syncthreads();                 // everyone is done reading the previous tile
-        stash();
-        __syncthreads();
-        if (tile + 1 < n_tiles) fetch(tile + 1);
-
-        const int k0 = tile * kBN;
-        // wavefront-level skip: every key of the tile is above this wavefront's diagonal
-        if (causal && k0 > qw0 + 31 + coff) continue;
-
-        // ---- S^T = K . Q^T -----------------------------------------------------
-        f32x16 s_acc[2];
+    // ---- per-lane LDS read offsets (tile- and buffer-independent parts) ------
+    // K fragment of step s, key row 32t + n: logical chunk 2s + kg -> slot (2s + kg) ^ swz(n)
+    // (swz depends on the row only through bits that 32t does not touch).
+    int k_off[NS];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+    for (int s = 0; s < NS; ++s) k_off[s] = n * kRow + (((2 * s + kg) ^ swz<D>(n)) << 4);
+    // V^T fragment of O^T tile dt: source lane s16 of 16-lane group g16 addresses key row
+    // 4*(g16>>1) + (s16>>2) (+8 for the upper half), d = 32dt + 16*(g16&1) + 4*(s16&3) .. +3
+    const int g16 = lane >> 4, s16 = lane & 15;
+    int v_off[2][NDT];
 #pragma unroll
-            for (int j = 0; j < 16; ++j) s_acc[t][j] = 0.f;
-            const unsigned char* kp = k_lds + (32 * t + n) * kKRow + kg * 16;
+    for (int e = 0; e < 2; ++e) {
+        const int row = 4 * (g16 >> 1) + (s16 >> 2) + 8 * e;
 #pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                const u32x4 kf = *reinterpret_cast<const u32x4*>(kp + s * 32);
-                s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s_acc[t]);
-            }
+        for (int dt = 0; dt < NDT; ++dt) {
+            const int d = 32 * dt + 16 * (g16 & 1) + 4 * (s16 & 3);
+            v_off[e][dt] = row * kRow + ((((d >> 3)) ^ swz<D>(row)) << 4) + (d & 7) * 2;
+        }
+    }
+    const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
+
+    for (int half = 0; half < 2; ++half) {
+        const int qtile = half == 0 ? nq - 1 - pair : pair;
+        if (half == 1 && qtile == nq - 1 - pair) break;         // odd tile count: the middle tile has no partner
+        const int q0 = qtile * kBM;
+        const int qw0 = q0 + 32 * wave;                    // first query of this wavefront
+        const int qi = qw0 + n;                            // this lane's query
+        const bool q_ok = qi < sq;
+
+        int kv_end = sk;
+        if (causal) kv_end = max(0, min(sk, min(sq, q0 + kBM) + coff));
+        const int n_tiles = (kv_end + kBN - 1) / kBN;
+
+        // ---- Q^T fragments: step s covers d = 16s + 8kg + j ----------------------
+        bf16x8 qf[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            u32x4 t = {0u, 0u, 0u, 0u};
+            if (q_ok) t = *reinterpret_cast<const u32x4*>(qb + (int64_t)qi * p.qs[2] + 16 * s + 8 * kg);
+            qf[s] = as_bf16x8(t);
         }
 
-        // ---- scale, mask, online softmax ----------------------------------------
-        // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
-        const bool need_mask = (causal && k0 + kBN - 1 > qw0 + coff) || (k0 + kBN > sk) || boolmask;
-        float mx = -INFINITY;
+        f32x16 o[NDT];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int i = 0; i < NDT; ++i)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float x = s_acc[t][i] * p.scale_log2;
-                if (need_mask) {
-                    const int key = k0 + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3);
-                    bool keep = key < sk;
-                    if (causal) keep = keep && (key <= qi + coff);
-                    if (boolmask) keep = keep && q_ok && (mrow[key < sk ? key : 0] != 0);
-                    if (!keep) x = -INFINITY;
+            for (int j = 0; j < 16; ++j) o[i][j] = 0.f;
+        float m_run = -INFINITY, l_run = 0.f;     // m_run: running max of the RAW scores (scale applied in the exponent)
+
+        const uint8_t* mrow = nullptr;
+        if (boolmask) mrow = p.mask + (int64_t)b * p.ms[0] + (int64_t)h * p.ms[1] + (int64_t)qi * p.ms[2];
+
+        // one KV tile; BUF (the LDS buffer holding it) is a compile-time constant so that every
+        // LDS read is "per-lane register + immediate offset"
+        auto step = [&](auto buf_c, int tile) {
+            constexpr int BUF = decltype(buf_c)::value;
+            wait_vmcnt<0>();                 // this wavefront's share of tile `tile` has landed
+            __syncthreads();                 // ... and everybody's; also: all are done reading the other buffer
+            if (tile + 1 < n_tiles) issue_tile(tile + 1, BUF ^ 1);
+
+            const int k0 = tile * kBN;
+            // wavefront-level skip: every key of the tile is above this wavefront's diagonal
+            if (causal && k0 > qw0 + 31 + coff) return;
+
+            const unsigned char* kt = k_lds + BUF * kTile;
+            const unsigned char* vt = v_lds + BUF * kTile;
+
+            // ---- S^T = K . Q^T -----------------------------------------------------
+            f32x16 s_acc[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) s_acc[t][j] = 0.f;
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    const u32x4 kf = *reinterpret_cast<const u32x4*>(kt + t * 32 * kRow + k_off[s]);
+                    s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s_acc[t]);
                 }
-                s_acc[t][i] = x;
-                mx = fmaxf(mx, x);
             }
-        }
-        mx = xor32_max(mx);
-        const float m_new = fmaxf(m_run, mx);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;    // row with no key yet: keep p = 0, not NaN
-        const float alpha = fast_exp2(m_run - m_use);
-        m_run = m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float e = fast_exp2(s_acc[t][i] - m_use);
-                s_acc[t][i] = e;
-                psum += e;
-            }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
 
-        // ---- O^T += V^T . P^T ------------------------------------------------------
-        // 16-key slice u: P^T fragment = accumulator registers 8(u%2).. of tile u/2, i.e.
-        // keys 16u + 4kg + (0..3) and 16u + 8 + 4kg + (0..3); the V^T read mirrors it.
-        const int g16 = lane >> 4, s16 = lane & 15;
-        const unsigned char* vp = v_lds + (4 * (g16 >> 1) + (s16 >> 2)) * kVRow + (16 * (g16 & 1) + 4 * (s16 & 3)) * 2;
+            // ---- mask, online softmax -------------------------------------------------
+            // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
+            const bool need_mask = (causal && k0 + kBN - 1 > qw0 + coff) || (k0 + kBN > sk) || boolmask;
+            if (need_mask) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int t = u >> 1, e0 = 8 * (u & 1);
-            u32x4 pw;
-            pw[0] = pack_bf16(s_acc[t][e0 + 0], s_acc[t][e0 + 1]);
-            pw[1] = pack_bf16(s_acc[t][e0 + 2], s_acc[t][e0 + 3]);
-            pw[2] = pack_bf16(s_acc[t][e0 + 4], s_acc[t][e0 + 5]);
-            pw[3] = pack_bf16(s_acc[t][e0 + 6], s_acc[t][e0 + 7]);
-            const bf16x8 pf = as_bf16x8(pw);
+                for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int dt = 0; dt < NDT; ++dt) {
-                const unsigned char* a = vp + (16 * u) * kVRow + dt * 64;
-                const i16x4 lo = lds_read_tr16(a);
-                const i16x4 hi = lds_read_tr16(a + 8 * kVRow);
-                o[dt] = mfma32(join_bf16x8(lo, hi), pf, o[dt]);
+                    for (int i = 0; i < 16; ++i) {
+                        const int key = k0 + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3);
+                        bool keep = key < sk;
+                        if (causal) keep = keep && (key <= qi + coff);
+                        if (boolmask) keep = keep && q_ok && (mrow[key < sk ? key : 0] != 0);
+                        if (!keep) s_acc[t][i] = -INFINITY;
+                    }
             }
-        }
-    }
+            float mx = s_acc[0][0];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[t][i]);
+            mx = xor32_max(mx);
+            const float m_new = fmaxf(m_run, mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;    // row with no key yet: keep p = 0, not NaN
+            const float alpha = fast_exp2((m_run - m_use) * p.scale_log2);
+            const float neg_ms = -m_use * p.scale_log2;
+            m_run = m_new;
+            // the running max settles after a few tiles; skip the rescale when no lane moved
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+                l_run *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+            }
 
-    // ---- normalise and store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4 ---
-    l_run = xor32_sum(l_run);
-    const float inv = 1.0f / l_run;          // l == 0 (no key kept) -> NaN row, like the reference softmax
-    if (q_ok) {
-        __bf16* orow = ob + (int64_t)qi * p.os[2];
+            // ---- O^T += V^T . P^T ------------------------------------------------------
+            // 16-key slice u: P^T fragment = accumulator registers 8(u%2).. of tile u/2, i.e.
+            // keys 16u + 4kg + (0..3) and 16u + 8 + 4kg + (0..3); the V^T read mirrors it.
+            // The row sum adds the bf16-rounded weights, i.e. exactly what multiplies V.
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
+            for (int u = 0; u < 4; ++u) {
+                const int t = u >> 1, e0 = 8 * (u & 1);
+                u32x4 pw;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 w;
-                w[0] = pack_bf16(o[dt][4 * g + 0] * inv, o[dt][4 * g + 1] * inv);
-                w[1] = pack_bf16(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
-                *reinterpret_cast<u32x2*>(orow + 32 * dt + 8 * g + 4 * kg) = w;
+                for (int w = 0; w < 4; ++w) {
+                    const float a0 = fast_exp2(fmaf(s_acc[t][e0 + 2 * w], p.scale_log2, neg_ms));
+                    const float a1 = fast_exp2(fmaf(s_acc[t][e0 + 2 * w + 1], p.scale_log2, neg_ms));
+                    pw[w] = pack_bf16(a0, a1);
+                    const uint32_t pwv = pw[w];
+                    l_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pwv), ones2, l_run, false);
+                }
+                const bf16x8 pf = as_bf16x8(pw);
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    const i16x4 lo = lds_read_tr16(vt + 16 * u * kRow + v_off[0][dt]);
+                    const i16x4 hi = lds_read_tr16(vt + 16 * u * kRow + v_off[1][dt]);
+                    o[dt] = mfma32(join_bf16x8(lo, hi), pf, o[dt]);
+                }
             }
+        };
+
+        __syncthreads();                     // the previous query tile's readers are done with the LDS buffers
+        if (n_tiles > 0) issue_tile(0, 0);
+        for (int tile = 0; tile < n_tiles; tile += 2) {
+            step(std::integral_constant<int, 0>{}, tile);
+            if (tile + 1 < n_tiles) step(std::integral_constant<int, 1>{}, tile + 1);
+        }
+
+        // ---- normalise and store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4 ---
+        l_run = xor32_sum(l_run);
+        const float inv = 1.0f / l_run;          // l == 0 (no key kept) -> NaN row, like the reference softmax
+        if (q_ok) {
+            __bf16* orow = ob + (int64_t)qi * p.os[2];
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    u32x2 w;
+                    w[0] = pack_bf16(o[dt][4 * g + 0] * inv, o[dt][4 * g + 1] * inv);
+                    w[1] = pack_bf16(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
+                    *reinterpret_cast<u32x2*>(orow + 32 * dt + 8 * g + 4 * kg) = w;
+                }
+        }
     }
 }
 
 template <int D>
 static int launch_prefill(const PrefillParams& p, hipStream_t stream) {
-    dim3 grid(p.n_qtiles, p.Hq, p.B);
+    dim3 grid((p.n_qtiles + 1) / 2, p.Hq, p.B);     // one workgroup per PAIR of query tiles
     hipLaunchKernelGGL((prefill_fwd_kernel<D>), grid, dim3(kPfWaves * 64), 0, stream, p);
     return (int)hipGetLastError();
 }
@@ -295,6 +348,8 @@ extern "C" int mi355_prefill_fwd(const void* q, const void* k, const void* v, vo
         if ((q_strides[i] | k_strides[i] | v_strides[i] | o_strides[i]) & 7)
             return set_error(MI355_EINVAL, "prefill: strides must be multiples of 8 elements (16-byte rows)");
     }
+    if (k_strides[2] <= 0 || v_strides[2] <= 0 || k_strides[2] >= (1 << 24) || v_strides[2] >= (1 << 24))
+        return set_error(MI355_EINVAL, "prefill: k/v row strides must be positive and below 2^24 elements");
     if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15)
         return set_error(MI355_EINVAL, "prefill: q, k, v and out must be 16-byte aligned");
 
