@@ -59,7 +59,7 @@ __device__ __forceinline__ int swz(int row) {
     else return (row >> 2) & 3;
 }
 
-template <int D>
+template <int D, int MODE>
 __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillParams p) {
     constexpr int NS = D / 16;                    // MFMA k-steps of K.Q^T
     constexpr int NDT = D / 32;                   // 32-row tiles of O^T
@@ -106,8 +106,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
     const int n = lane & 31;          // query column of S^T / O^T, key row of K, d row of V^T
     const int kg = lane >> 5;         // 0..1
 
-    const bool causal = p.mask_mode == MI355_MASK_CAUSAL;
-    const bool boolmask = p.mask_mode == MI355_MASK_BOOL;
+    constexpr bool causal = MODE == MI355_MASK_CAUSAL;
+    constexpr bool boolmask = MODE == MI355_MASK_BOOL;
     const int coff = sk - sq;                          // bottom-right aligned causal diagonal
 
     // ---- tile loader: wavefront w, instruction j covers LDS chunks (w*NI + j)*64 .. +63 -----
@@ -193,86 +193,88 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
         for (int i = 0; i < NDT; ++i)
 #pragma unroll
             for (int j = 0; j < 16; ++j) o[i][j] = 0.f;
-        float m_run = -INFINITY, l_run = 0.f;     // m_run: running max of the RAW scores (scale applied in the exponent)
+        // m_ref: exponent reference of this lane's query row, in RAW score units (>= row max - slack);
+        // neg_ref = -m_ref * scale_log2 is the additive term of the exponent
+        float m_ref = -INFINITY, neg_ref = 0.f, l_run = 0.f;
 
         const uint8_t* mrow = nullptr;
-        if (boolmask) mrow = p.mask + (int64_t)b * p.ms[0] + (int64_t)h * p.ms[1] + (int64_t)qi * p.ms[2];
+        if (boolmask)     // rows of padded query lanes alias the last real row (their results are never stored)
+            mrow = p.mask + (int64_t)b * p.ms[0] + (int64_t)h * p.ms[1] + (int64_t)min(qi, sq - 1) * p.ms[2];
 
-        // one KV tile; BUF (the LDS buffer holding it) is a compile-time constant so that every
-        // LDS read is "per-lane register + immediate offset"
-        auto step = [&](auto buf_c, int tile) {
-            constexpr int BUF = decltype(buf_c)::value;
+        // Leading tiles whose keys are all visible to every query of this wavefront need no
+        // mask code at all; only the tiles on the diagonal / at the ragged end take the masked path.
+        int n_plain = sk / kBN;
+        if (causal) n_plain = min(n_plain, max(0, qw0 + coff + 1) / kBN);
+        if (boolmask) n_plain = 0;
+        n_plain = min(n_plain, n_tiles);
+
+        f32x16 s_acc[2];
+        float mx = 0.f;
+        const auto flip = [&]() {            // the per-lane read offsets carry the LDS buffer bit
+#pragma unroll
+            for (int s = 0; s < NS; ++s) k_off[s] ^= kTile;
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) v_off[e][dt] ^= kTile;
+        };
+
+        // First half of a KV tile: wait for it, start the next one, S^T = K . Q^T, mask, row max.
+        // Returns false when the whole tile lies above this wavefront's diagonal (nothing to add).
+        auto head = [&](auto masked_c, int tile) -> bool {
+            constexpr bool MASKED = decltype(masked_c)::value;
             wait_vmcnt<0>();                 // this wavefront's share of tile `tile` has landed
             __syncthreads();                 // ... and everybody's; also: all are done reading the other buffer
-            if (tile + 1 < n_tiles) issue_tile(tile + 1, BUF ^ 1);
+            if (tile + 1 < n_tiles) issue_tile(tile + 1, (tile + 1) & 1);
 
             const int k0 = tile * kBN;
-            // wavefront-level skip: every key of the tile is above this wavefront's diagonal
-            if (causal && k0 > qw0 + 31 + coff) return;
-
-            const unsigned char* kt = k_lds + BUF * kTile;
-            const unsigned char* vt = v_lds + BUF * kTile;
-
-            // ---- S^T = K . Q^T -----------------------------------------------------
-            f32x16 s_acc[2];
+            if (causal && MASKED && k0 > qw0 + 31 + coff) return false;
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) s_acc[t][j] = 0.f;
 #pragma unroll
                 for (int s = 0; s < NS; ++s) {
-                    const u32x4 kf = *reinterpret_cast<const u32x4*>(kt + t * 32 * kRow + k_off[s]);
+                    const u32x4 kf = *reinterpret_cast<const u32x4*>(k_lds + t * 32 * kRow + k_off[s]);
                     s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s_acc[t]);
                 }
             }
-
-            // ---- mask, online softmax -------------------------------------------------
             // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
-            const bool need_mask = (causal && k0 + kBN - 1 > qw0 + coff) || (k0 + kBN > sk) || boolmask;
-            if (need_mask) {
+            if constexpr (MASKED) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int key = k0 + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3);
                         bool keep = key < sk;
-                        if (causal) keep = keep && (key <= qi + coff);
-                        if (boolmask) keep = keep && q_ok && (mrow[key < sk ? key : 0] != 0);
-                        if (!keep) s_acc[t][i] = -INFINITY;
+                        if constexpr (causal) keep = keep & (key <= qi + coff);
+                        // unconditional, clamped byte load: no divergent control flow around the select
+                        if constexpr (boolmask) keep = keep & (mrow[min(key, sk - 1)] != 0);
+                        s_acc[t][i] = keep ? s_acc[t][i] : -INFINITY;
                     }
             }
-            float mx = s_acc[0][0];
+            mx = s_acc[0][0];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[t][i]);
             mx = xor32_max(mx);
-            const float m_new = fmaxf(m_run, mx);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;    // row with no key yet: keep p = 0, not NaN
-            const float alpha = fast_exp2((m_run - m_use) * p.scale_log2);
-            const float neg_ms = -m_use * p.scale_log2;
-            m_run = m_new;
-            // the running max settles after a few tiles; skip the rescale when no lane moved
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-                l_run *= alpha;
-#pragma unroll
-                for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-            }
+            return true;
+        };
 
-            // ---- O^T += V^T . P^T ------------------------------------------------------
-            // 16-key slice u: P^T fragment = accumulator registers 8(u%2).. of tile u/2, i.e.
-            // keys 16u + 4kg + (0..3) and 16u + 8 + 4kg + (0..3); the V^T read mirrors it.
-            // The row sum adds the bf16-rounded weights, i.e. exactly what multiplies V.
+        // Second half: P = 2^(S*scale - ref), row sums, O^T += V^T . P^T.
+        // 16-key slice u: P^T fragment = accumulator registers 8(u%2).. of tile u/2, i.e.
+        // keys 16u + 4kg + (0..3) and 16u + 8 + 4kg + (0..3); the V^T read mirrors it.
+        // The row sum adds the bf16-rounded weights, i.e. exactly what multiplies V.
+        auto accumulate = [&]() {
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int t = u >> 1, e0 = 8 * (u & 1);
                 u32x4 pw;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    const float a0 = fast_exp2(fmaf(s_acc[t][e0 + 2 * w], p.scale_log2, neg_ms));
-                    const float a1 = fast_exp2(fmaf(s_acc[t][e0 + 2 * w + 1], p.scale_log2, neg_ms));
+                    const float a0 = fast_exp2(fmaf(s_acc[t][e0 + 2 * w], p.scale_log2, neg_ref));
+                    const float a1 = fast_exp2(fmaf(s_acc[t][e0 + 2 * w + 1], p.scale_log2, neg_ref));
                     pw[w] = pack_bf16(a0, a1);
                     const uint32_t pwv = pw[w];
                     l_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pwv), ones2, l_run, false);
@@ -280,19 +282,56 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
                 const bf16x8 pf = as_bf16x8(pw);
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt) {
-                    const i16x4 lo = lds_read_tr16(vt + 16 * u * kRow + v_off[0][dt]);
-                    const i16x4 hi = lds_read_tr16(vt + 16 * u * kRow + v_off[1][dt]);
+                    const i16x4 lo = lds_read_tr16(v_lds + 16 * u * kRow + v_off[0][dt]);
+                    const i16x4 hi = lds_read_tr16(v_lds + 16 * u * kRow + v_off[1][dt]);
                     o[dt] = mfma32(join_bf16x8(lo, hi), pf, o[dt]);
                 }
             }
         };
 
+        // Lazy rescaling: the exponent reference m_ref only moves when some row's maximum
+        // outgrows it by more than 2^kSlack; until then weights are at most 2^kSlack (exact in
+        // the fp32 sums, harmless in bf16) and the O accumulators need no per-tile multiply.
+        // The fast loop below therefore only accumulates in place; a tile that needs the
+        // reference moved leaves it, rescales, and re-enters.
+        constexpr float kSlack = 8.0f;
+        auto run_tiles = [&](auto masked_c, int tile, const int tile_end) {
+            for (;;) {
+                bool pending = false;
+                while (tile < tile_end) {
+                    if (head(masked_c, tile)) {
+                        const bool grow = !((mx - m_ref) * p.scale_log2 <= kSlack);   // also true while m_ref = -inf
+                        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+                            pending = true;
+                            break;
+                        }
+                        accumulate();
+                    }
+                    flip();
+                    ++tile;
+                }
+                if (!pending) break;
+                const float m_new = fmaxf(m_ref, mx);
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;    // row with no key yet: keep p = 0, not NaN
+                const float alpha = fast_exp2((m_ref - m_use) * p.scale_log2);
+                m_ref = m_new;
+                neg_ref = -m_use * p.scale_log2;
+                l_run *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+                accumulate();
+                flip();
+                ++tile;
+            }
+        };
+
         __syncthreads();                     // the previous query tile's readers are done with the LDS buffers
         if (n_tiles > 0) issue_tile(0, 0);
-        for (int tile = 0; tile < n_tiles; tile += 2) {
-            step(std::integral_constant<int, 0>{}, tile);
-            if (tile + 1 < n_tiles) step(std::integral_constant<int, 1>{}, tile + 1);
-        }
+        run_tiles(std::false_type{}, 0, n_plain);
+        run_tiles(std::true_type{}, n_plain, n_tiles);
+        if (n_tiles & 1) flip();             // leave the offsets pointing at buffer 0 for the next query tile
 
         // ---- normalise and store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4 ---
         l_run = xor32_sum(l_run);
@@ -315,7 +354,13 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
 template <int D>
 static int launch_prefill(const PrefillParams& p, hipStream_t stream) {
     dim3 grid((p.n_qtiles + 1) / 2, p.Hq, p.B);     // one workgroup per PAIR of query tiles
-    hipLaunchKernelGGL((prefill_fwd_kernel<D>), grid, dim3(kPfWaves * 64), 0, stream, p);
+    dim3 block(kPfWaves * 64);
+    if (p.mask_mode == MI355_MASK_CAUSAL)
+        hipLaunchKernelGGL((prefill_fwd_kernel<D, MI355_MASK_CAUSAL>), grid, block, 0, stream, p);
+    else if (p.mask_mode == MI355_MASK_BOOL)
+        hipLaunchKernelGGL((prefill_fwd_kernel<D, MI355_MASK_BOOL>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((prefill_fwd_kernel<D, MI355_MASK_NONE>), grid, block, 0, stream, p);
     return (int)hipGetLastError();
 }
 
