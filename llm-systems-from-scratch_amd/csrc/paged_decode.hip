@@ -13,9 +13,13 @@
 //   O^T (d x queries) += V^T . P^T      V^T fragments come from a wavefront-private
 //                                       LDS tile through ds_read_b64_tr_b16
 //
-// K goes global -> registers directly in MFMA A-operand layout; V goes
-// global -> registers (fully coalesced 1 KiB per instruction) -> LDS -> transposed
-// read.  The next step's K/V loads are issued before the current step's math.
+// K and V both go global -> registers (fully coalesced, non-temporal, 1 KiB per
+// instruction) -> wavefront-private LDS tile; K fragments come back with
+// ds_read_b128 in MFMA A-operand layout, V^T fragments with the transposed read.
+// The next step's loads are issued as soon as the staging registers are free, so
+// they fly during the whole step.  (Direct global->LDS loads are not used: an LDS
+// read of a wavefront waits for every direct-to-LDS load it issued earlier, which
+// would serialise a wavefront-private pipeline.)
 // The four wavefronts merge their (m, l, O) in LDS; a sequence that fits one
 // chunk is normalised and written straight to `out`, otherwise the chunk's
 // partial goes to the workspace and the combine kernel finishes it:
@@ -48,22 +52,29 @@ struct DecodeParams {
     float scale_log2;
 };
 
-template <int D>
+template <int D, bool FP8>
 struct DecodeLds {
-    static constexpr int kVRow = D * 2 + 32;                 // bytes per staged V row (padded)
+    static constexpr int kVRow = D * 2 + 32;                 // bytes per staged V row (bf16, padded)
     static constexpr int kVBytes = kStage * kVRow;           // per-wavefront V tile
+    static constexpr int kKRow = FP8 ? D : D * 2;            // bytes per staged K row (raw cache bytes, swizzled)
+    static constexpr int kKBytes = kStage * kKRow;           // per-wavefront K tile
     static constexpr int kPartFloats = 16 * D + 32;          // per-wavefront (O, m, l)
-    static constexpr int kWaveBytes = kVBytes > kPartFloats * 4 ? kVBytes : kPartFloats * 4;
+    static constexpr int kTiles = kVBytes + kKBytes;
+    static constexpr int kWaveBytes = kTiles > kPartFloats * 4 ? kTiles : kPartFloats * 4;
 };
 
 template <int D, bool FP8>
 __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(DecodeParams p) {
     constexpr int NS = D / 32;                       // MFMA k-steps of K.Q^T
     constexpr int NT = D / 16;                       // 16-row tiles of O^T
-    constexpr int KL = FP8 ? (D / 64) : NS;          // 16-byte K loads per lane per block
-    constexpr int VL = FP8 ? (D / 64) : (D / 32);    // 16-byte V loads per lane per block
-    constexpr int kVRow = DecodeLds<D>::kVRow;
-    constexpr int kWaveBytes = DecodeLds<D>::kWaveBytes;
+    constexpr int VL = FP8 ? (D / 64) : (D / 32);    // 16-byte loads per lane per block (K and V alike)
+    constexpr int KL = VL;
+    constexpr int kVRow = DecodeLds<D, FP8>::kVRow;
+    constexpr int kVBytes = DecodeLds<D, FP8>::kVBytes;
+    constexpr int kKRow = DecodeLds<D, FP8>::kKRow;
+    constexpr int kKChunks = kKRow / 16;              // 16-byte chunks per staged K row
+    constexpr int kKRowsPer256 = 256 / kKRow > 0 ? 256 / kKRow : 1;
+    constexpr int kWaveBytes = DecodeLds<D, FP8>::kWaveBytes;
     static_assert(!FP8 || D >= 64, "fp8 KV needs head_dim >= 64");
 
     __shared__ __attribute__((aligned(16))) unsigned char smem[kDecodeWaves * kWaveBytes];
@@ -85,7 +96,11 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
     const int r = lane & 15;          // key row of K / query column of S^T / d row of V^T
     const int kg = lane >> 4;         // 0..3
 
-    unsigned char* wsm = smem + wave * kWaveBytes;
+    unsigned char* wsm = smem + wave * kWaveBytes;      // this wavefront's V tile (then its K tile)
+    unsigned char* ksm = wsm + kVBytes;
+    // K rows are stored unpadded; the 16-byte chunk c of row q lives in slot c ^ kswz(q) so that the
+    // 16 lanes reading one chunk column of 16 consecutive rows hit 16 different bank groups
+    auto kswz = [&](int row) { return (row / kKRowsPer256) % kKChunks; };
 
     // ---- Q^T B-operand fragments (zero for padded query columns) ----------
     // bf16 cache: step s covers d = 32s + 8kg + j.
@@ -127,21 +142,16 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
         const int64_t phys = __builtin_amdgcn_readlane(my_phys, blk);
         return (phys * p.Hkv + hk) * (int64_t)(kBlock * D);
     };
+    // K and V are both fetched as fully contiguous 1 KiB per instruction (streaming, non-temporal):
+    // partial-line patterns measurably lose HBM bandwidth.  Lane l of load j holds bytes
+    // (64j + l)*16 .. +15 of the (block, kv head) slab.
     auto load_k = [&](int it) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int64_t slab = slab_of(2 * it + t);
-            if constexpr (FP8) {
-                const unsigned char* kb = reinterpret_cast<const unsigned char*>(p.k_cache) + slab;
+            const unsigned char* kb = reinterpret_cast<const unsigned char*>(p.k_cache) + slab_of(2 * it + t) * (FP8 ? 1 : 2);
 #pragma unroll
-                for (int j = 0; j < KL; ++j)
-                    kreg[t][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb + r * D + 64 * j + 16 * kg));
-            } else {
-                const __bf16* kb = reinterpret_cast<const __bf16*>(p.k_cache) + slab;
-#pragma unroll
-                for (int s = 0; s < KL; ++s)
-                    kreg[t][s] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb + r * D + 32 * s + 8 * kg));
-            }
+            for (int j = 0; j < KL; ++j)
+                kreg[t][j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kb + (j * 64 + lane) * 16));
         }
     };
     auto load_v = [&](int it) {
@@ -205,17 +215,37 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
                 }
             }
         }
+        // ---- K: registers -> wavefront-private LDS tile (raw cache bytes, swizzled chunks) --
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int j = 0; j < KL; ++j) {
+                const int cidx = j * 64 + lane;                       // 16-byte chunk index inside the slab
+                const int row = 16 * t + cidx / kKChunks, c = cidx % kKChunks;
+                *reinterpret_cast<u32x4*>(ksm + row * kKRow + ((c ^ kswz(row)) << 4)) = kreg[t][j];
+            }
+        }
+        // The staging registers are free again: fetch the next step now, so that its loads
+        // fly during everything below.  The scheduling barriers keep the compiler from sinking
+        // the loads towards their (next-iteration) uses.
+        __builtin_amdgcn_sched_barrier(0);
         load_v(min(it + 1, n_iter - 1));
+        load_k(min(it + 1, n_iter - 1));
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- S^T = K . Q^T ---------------------------------------------------
+        // A fragment of step s, key row 16t + r: bf16 cache: chunk 4s + kg (d = 32s + 8kg ..);
+        // fp8 cache: chunk 4j + kg holds d = 64j + 16kg .. +15, i.e. the two steps 2j and 2j+1.
         f32x4 s_acc[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             s_acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const int row = 16 * t + r;
+            const unsigned char* krow = ksm + row * kKRow;
             if constexpr (FP8) {
 #pragma unroll
-                for (int j = 0; j < KL; ++j) {
-                    u32x4 raw = kreg[t][j];
+                for (int j = 0; j < D / 64; ++j) {
+                    const u32x4 raw = *reinterpret_cast<const u32x4*>(krow + (((4 * j + kg) ^ kswz(row)) << 4));
                     u32x2 a = fp8x4_to_bf16x4(raw[0]), bq = fp8x4_to_bf16x4(raw[1]);
                     u32x2 c = fp8x4_to_bf16x4(raw[2]), dq = fp8x4_to_bf16x4(raw[3]);
                     s_acc[t] = mfma16(as_bf16x8(u32x4{a[0], a[1], bq[0], bq[1]}), qf[2 * j], s_acc[t]);
@@ -223,10 +253,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
                 }
             } else {
 #pragma unroll
-                for (int s = 0; s < NS; ++s) s_acc[t] = mfma16(as_bf16x8(kreg[t][s]), qf[s], s_acc[t]);
+                for (int s = 0; s < NS; ++s) {
+                    const u32x4 kf = *reinterpret_cast<const u32x4*>(krow + (((4 * s + kg) ^ kswz(row)) << 4));
+                    s_acc[t] = mfma16(as_bf16x8(kf), qf[s], s_acc[t]);
+                }
             }
         }
-        load_k(min(it + 1, n_iter - 1));
 
         // ---- online softmax (lane: query column r, keys 16t + 4kg + i) -------
         float ks2[2] = {1.0f, 1.0f}, vs2[2] = {1.0f, 1.0f};
