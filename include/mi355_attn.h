@@ -103,8 +103,8 @@ int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cac
 
 size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx);
 
-/* Tokens of one sequence handled by one workgroup of the split-K pass. */
-int mi355_paged_decode_chunk_tokens(void);
+/* Tokens of one sequence handled by one workgroup of the split-K pass (grows with max_ctx). */
+int mi355_paged_decode_chunk_tokens(int max_ctx);
 
 /*
  * Plain device-to-device copy of `bytes` bytes (16-byte aligned).  Measurement aid

@@ -1,6 +1,6 @@
 // Paged-KV decode attention for gfx950: split-K pass + combine.
 //
-// Work item of the split-K pass = (sequence, kv head, chunk of kChunk tokens).
+// Work item of the split-K pass = (sequence, kv head, chunk of 4 * tokens_per_wave tokens).
 // One workgroup of 4 wavefronts per work item; each wavefront streams its own
 // quarter of the chunk, 32 keys (two 16-token cache blocks) per step:
 //
@@ -30,8 +30,7 @@
 namespace mi355 {
 
 constexpr int kDecodeWaves = 4;
-constexpr int kTokensPerWave = 256;
-constexpr int kChunk = kDecodeWaves * kTokensPerWave;   // tokens per workgroup
+constexpr int kMaxTokensPerWave = 1024;                 // 64 cache blocks: one block id per lane
 constexpr int kBlock = 16;                              // tokens per cache block
 constexpr int kStage = 32;                              // keys per step (2 blocks)
 
@@ -49,6 +48,7 @@ struct DecodeParams {
     float* ws_m;
     float* ws_l;
     int B, Hq, Hkv, max_chunks, max_ctx;
+    int tokens_per_wave;      // 256, 512 or 1024: a long stream per wavefront amortises its start-up latency
     float scale_log2;
 };
 
@@ -87,7 +87,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
     const int b = (wg / p.Hkv) % p.B;
     const int chunk = wg / (p.Hkv * p.B);
     const int ctx = min(p.context_lens[b], p.max_ctx);     // a length beyond the promised bound is truncated, never chased
-    const int chunk_start = chunk * kChunk;
+    const int chunk_tokens = kDecodeWaves * p.tokens_per_wave;
+    const int chunk_start = chunk * chunk_tokens;
     if (chunk_start >= ctx) return;
 
     const int G = p.Hq / p.Hkv;
@@ -118,8 +119,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
         }
     }
 
-    const int t0 = chunk_start + wave * kTokensPerWave;
-    const int t1 = min(ctx, t0 + kTokensPerWave);
+    const int t0 = chunk_start + wave * p.tokens_per_wave;
+    const int t1 = min(ctx, t0 + p.tokens_per_wave);
     const int n_iter = t1 > t0 ? (t1 - t0 + kStage - 1) / kStage : 0;
     const int last_blk = (ctx - 1) / kBlock;
     const int32_t* bt = p.block_tables + (int64_t)b * p.bt_row_stride;
@@ -332,7 +333,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
     }
     __syncthreads();
 
-    const int n_chunks = (ctx + kChunk - 1) / kChunk;
+    const int n_chunks = (ctx + chunk_tokens - 1) / chunk_tokens;
     for (int idx = threadIdx.x; idx < G * D; idx += kDecodeWaves * 64) {
         const int qi = idx / D, d = idx % D;
         float mw[kDecodeWaves];
@@ -369,7 +370,8 @@ __global__ __launch_bounds__(D) void paged_decode_combine_kernel(DecodeParams p)
     const int row = blockIdx.x;                  // b * Hq + h
     const int b = row / p.Hq;
     const int ctx = min(p.context_lens[b], p.max_ctx);
-    const int n_chunks = (ctx + kChunk - 1) / kChunk;
+    const int chunk_tokens = kDecodeWaves * p.tokens_per_wave;
+    const int n_chunks = (ctx + chunk_tokens - 1) / chunk_tokens;
     if (n_chunks <= 1) return;                   // written by the split pass (or empty)
     const int d = threadIdx.x;
     const int64_t base = (int64_t)row * p.max_chunks;
@@ -399,11 +401,18 @@ using namespace mi355;
 
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-extern "C" int mi355_paged_decode_chunk_tokens(void) { return kChunk; }
+// Tokens per wavefront grow with the longest context: short batches keep all four wavefronts of
+// a workgroup busy, long ones get long uninterrupted streams.
+static int tokens_per_wave_for(int max_ctx) {
+    return max_ctx >= 4096 ? kMaxTokensPerWave : (max_ctx >= 2048 ? 512 : 256);
+}
+
+extern "C" int mi355_paged_decode_chunk_tokens(int max_ctx) { return kDecodeWaves * tokens_per_wave_for(max_ctx); }
 
 extern "C" size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx) {
     if (B <= 0 || Hq <= 0 || D <= 0 || max_ctx <= 0) return 0;
-    const size_t chunks = ((size_t)max_ctx + kChunk - 1) / kChunk;
+    const size_t chunk = (size_t)mi355_paged_decode_chunk_tokens(max_ctx);
+    const size_t chunks = ((size_t)max_ctx + chunk - 1) / chunk;
     const size_t rows = (size_t)B * Hq * chunks;
     return align_up(rows * D * 4, 256) + 2 * align_up(rows * 4, 256);
 }
@@ -421,7 +430,8 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
     if (Hq % Hkv != 0 || Hq / Hkv > 16)
         return set_error(MI355_EINVAL, "paged_decode: Hq must be a multiple of Hkv with Hq/Hkv <= 16");
     if (block_size != kBlock) return set_error(MI355_EINVAL, "paged_decode: block_size must be 16");
-    if ((int64_t)((max_ctx + kChunk - 1) / kChunk) * Hkv * B > 0x7fffffffLL)
+    const int chunk = mi355_paged_decode_chunk_tokens(max_ctx);
+    if ((int64_t)((max_ctx + chunk - 1) / chunk) * Hkv * B > 0x7fffffffLL)
         return set_error(MI355_EINVAL, "paged_decode: chunks * Hkv * B exceeds the grid limit");
     if (kv_dtype != MI355_BF16 && kv_dtype != MI355_FP8_E4M3)
         return set_error(MI355_EDTYPE, "paged_decode: kv_dtype must be MI355_BF16 or MI355_FP8_E4M3");
@@ -431,7 +441,7 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
     if (!(D == 128 || D == 64 || (D == 32 && !fp8)))
         return set_error(MI355_EINVAL, "paged_decode: head_dim must be 64 or 128 (or 32 with a bf16 cache)");
     const size_t need = mi355_paged_decode_workspace_bytes(B, Hq, D, max_ctx);
-    const int max_chunks = (max_ctx + kChunk - 1) / kChunk;
+    const int max_chunks = (max_ctx + chunk - 1) / chunk;
     if (max_chunks > 1 && (!workspace || workspace_bytes < need))
         return set_error(MI355_EWORKSPACE, "paged_decode: workspace smaller than mi355_paged_decode_workspace_bytes()");
 
@@ -455,6 +465,7 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
     p.Hkv = Hkv;
     p.max_chunks = max_chunks;
     p.max_ctx = max_ctx;
+    p.tokens_per_wave = tokens_per_wave_for(max_ctx);
     p.scale_log2 = softmax_scale * kLog2e;
 
     hipStream_t s = (hipStream_t)stream;

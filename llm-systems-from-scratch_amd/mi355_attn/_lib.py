@@ -49,7 +49,7 @@ def load():
     lib.mi355_paged_decode_workspace_bytes.restype = sz
     lib.mi355_paged_decode_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.mi355_paged_decode_chunk_tokens.restype = i32
-    lib.mi355_paged_decode_chunk_tokens.argtypes = []
+    lib.mi355_paged_decode_chunk_tokens.argtypes = [i32]
     lib.mi355_calib_copy.restype = i32
     lib.mi355_calib_copy.argtypes = [vp, vp, sz, vp]
     lib.mi355_last_error.restype = C.c_char_p

@@ -78,6 +78,24 @@ def test_decode_ragged_edges(ops, D, Hq, Hkv):
     check(run_decode(ops, q, kc, vc, bt, cl), ref, what=f"ragged D{D} {Hq}/{Hkv}")
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_decode_long_contexts_multi_chunk(ops, fp8):
+    """Contexts around the 4096-token workgroup chunk used for long batches, several chunks per sequence."""
+    ctx = [4095, 4096, 4097, 8191, 8193, 12000, 33, 1]
+    print(f"case: decode long contexts fp8={fp8}", flush=True)
+    q, kc, vc, bt, cl = orc.make_paged_case(batch=len(ctx), n_q_heads=8, n_kv_heads=2, head_dim=128, block_size=16,
+                                            context_lens=ctx, pool_factor=1.1, seed=77, dtype=torch.bfloat16)
+    if fp8:
+        k8, ks = orc.quantize_kv_fp8(kc)
+        v8, vs = orc.quantize_kv_fp8(vc)
+        got = run_decode(ops, q, k8, v8, bt, cl, k_scale=ks, v_scale=vs)
+        ref = orc.paged_decode_reference(q, k8, v8, bt, cl, k_scale=ks, v_scale=vs)
+    else:
+        got = run_decode(ops, q, kc, vc, bt, cl)
+        ref = orc.paged_decode_reference(q, kc, vc, bt, cl)
+    check(got, ref, what=f"long contexts fp8={fp8}")
+
+
 def test_decode_ignores_pool_garbage_and_table_tail(ops):
     """NaN/Inf bit patterns in unused blocks, in the tail of the last block and junk table entries are never used."""
     ctx = [5, 40, 100, 1030]
