@@ -1,0 +1,130 @@
+"""CPU-side checks: the C-ABI library loads, exports what include/mi355_attn.h declares, and rejects
+bad arguments before touching a GPU; host-side operator validation; workload generators."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+import mi355_attn
+from mi355_attn import _lib, workloads
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return mi355_attn.load()
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "mi355_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = declared_functions()
+    assert "mi355_prefill_fwd" in names and "mi355_paged_decode_fwd" in names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/mi355_attn.h but not exported"
+    assert sorted(_lib.EXPORTS) == names
+
+
+def test_version_and_workspace_queries(lib):
+    assert b"gfx950" in lib.mi355_version()
+    assert lib.mi355_paged_decode_chunk_tokens(256) == 1024
+    assert lib.mi355_paged_decode_chunk_tokens(3000) == 2048
+    assert lib.mi355_paged_decode_chunk_tokens(16384) == 4096
+    # one chunk -> still a (small) partial area; grows with chunks * B * Hq * D
+    small = lib.mi355_paged_decode_workspace_bytes(4, 8, 64, 256)
+    big = lib.mi355_paged_decode_workspace_bytes(128, 32, 128, 16384)
+    assert 0 < small < big
+    chunks = (16384 + 4095) // 4096
+    assert big >= 128 * 32 * chunks * (128 + 2) * 4
+    assert lib.mi355_paged_decode_workspace_bytes(0, 8, 64, 256) == 0
+
+
+def test_prefill_rejects_bad_arguments_without_a_gpu(lib):
+    s3 = _lib.strides3((8, 8, 8))
+    buf = C.create_string_buffer(64)
+    ptr = (C.addressof(buf) + 15) & ~15
+
+    def call(D=64, Hq=2, Hkv=2, q=ptr, mode=_lib.MASK_CAUSAL, dtype=_lib.MI355_BF16, mask=None, cu_q=None, cu_k=None,
+             strides=s3):
+        return lib.mi355_prefill_fwd(q, ptr, ptr, ptr, strides, s3, s3, s3, cu_q, cu_k, mask, s3,
+                                     1, Hq, Hkv, 8, 8, D, 0.125, mode, dtype, None)
+
+    assert call(D=96) == -1 and b"head_dim" in lib.mi355_last_error()
+    assert call(Hq=3, Hkv=2) == -1
+    assert call(q=None) == -1 and b"null" in lib.mi355_last_error()
+    assert call(dtype=7) == -3
+    assert call(mode=9) == -1
+    assert call(mode=_lib.MASK_BOOL, mask=None) == -1
+    assert call(cu_q=ptr, cu_k=None) == -1
+    assert call(strides=_lib.strides3((8, 8, 4))) == -1 and b"strides" in lib.mi355_last_error()
+    assert call(q=ptr + 2) == -1 and b"aligned" in lib.mi355_last_error()
+
+
+def test_decode_rejects_bad_arguments_without_a_gpu(lib):
+    buf = C.create_string_buffer(64)
+    ptr = C.addressof(buf)
+
+    def call(Hq=8, Hkv=2, D=128, bs=16, kv=_lib.MI355_BF16, ks=None, ws=ptr, ws_bytes=1 << 30, max_ctx=64, q=ptr):
+        return lib.mi355_paged_decode_fwd(q, ptr, ptr, ptr, ptr, 4, ptr, ks, ks, ws, ws_bytes,
+                                          2, Hq, Hkv, D, bs, max_ctx, 0.1, kv, None)
+
+    assert call(bs=32) == -1 and b"block_size" in lib.mi355_last_error()
+    assert call(Hq=7) == -1
+    assert call(Hq=64, Hkv=2) == -1            # more than 16 query heads per kv head
+    assert call(D=96) == -1
+    assert call(kv=5) == -3
+    assert call(kv=_lib.MI355_FP8_E4M3, ks=None) == -1 and b"scale" in lib.mi355_last_error()
+    assert call(kv=_lib.MI355_FP8_E4M3, ks=ptr, D=32) == -1
+    assert call(q=None) == -1
+    assert call(max_ctx=100000, ws_bytes=16) == -2 and b"workspace" in lib.mi355_last_error()
+
+
+def test_host_ops_validate_before_launch():
+    q = torch.zeros(2, 4, 64, dtype=torch.bfloat16)
+    kc = torch.zeros(8, 2, 16, 64, dtype=torch.bfloat16)
+    bt = torch.zeros(2, 4, dtype=torch.int32)
+    cl = torch.ones(2, dtype=torch.int32)
+    with pytest.raises(ValueError, match="GPU"):
+        mi355_attn.paged_attention_decode(q, kc, kc, bt, cl)
+    with pytest.raises(ValueError, match="GPU"):
+        mi355_attn.flash_attn_prefill(torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16),
+                                      torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16),
+                                      torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16))
+    with pytest.raises(TypeError):
+        mi355_attn.scaled_dot_product_attention(torch.zeros(2, 8, 64), torch.zeros(2, 8, 64), torch.zeros(2, 8, 64),
+                                                mask=torch.zeros(8, 8))          # mask must be boolean
+
+
+def test_missing_library_is_an_error_not_a_fallback(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmi355attn.so")
+    with pytest.raises(_lib.LibraryMissing):
+        _lib.load()
+
+
+def test_product_package_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "llm-systems-from-scratch_amd")
+    for d, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(d, f)).read()
+                assert "attention_oracle" not in text and "from oracle" not in text and "import oracle" not in text, f
+
+
+def test_workload_draws_match_the_configurations():
+    c3 = workloads.draw_context_lens("uniform", 128, 512, 16384, 0)
+    assert c3.shape == (128,) and c3.min() >= 512 and c3.max() <= 16384
+    assert torch.equal(c3, workloads.draw_context_lens("uniform", 128, 512, 16384, 0))
+    c4 = workloads.draw_context_lens("loguniform", 256, 128, 32768, 0)
+    assert c4.min() >= 128 and c4.max() <= 32768
+    # the oracle's generator (used by the tests) and the product's draw the same lengths
+    from oracle import attention_oracle as orc
+    assert torch.equal(c3, orc.draw_context_lens("uniform", 128, 512, 16384, 0))
+    assert torch.equal(c4, orc.draw_context_lens("loguniform", 256, 128, 32768, 0))
