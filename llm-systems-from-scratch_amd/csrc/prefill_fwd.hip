@@ -46,6 +46,7 @@ struct PrefillParams {
     float scale_log2;
     int mask_mode;
     int n_qtiles;
+    int n_pairs;
 };
 
 // XOR pattern applied to the 16-byte chunk index of LDS row `row` (rows hold D bf16).
@@ -71,9 +72,16 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kTile];
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kTile];
 
-    const int pair = blockIdx.x;
-    const int h = blockIdx.y;
-    const int b = blockIdx.z;
+    // Workgroup ids are dealt round-robin to the 8 XCDs, each with a private L2.  The id is
+    // remapped so that every XCD works through a contiguous range of the logical order
+    // (pair fastest, then the query heads of one kv head, then kv head, then batch): the
+    // workgroups that stream the same K/V are then resident on the same XCD at the same time.
+    const int n_wg = gridDim.x;
+    int lid = blockIdx.x;
+    if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
+    const int pair = lid % p.n_pairs;
+    const int h = (lid / p.n_pairs) % p.Hq;
+    const int b = lid / (p.n_pairs * p.Hq);
     const int hk = h / (p.Hq / p.Hkv);
 
     int sq, sk;
@@ -353,7 +361,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
 
 template <int D>
 static int launch_prefill(const PrefillParams& p, hipStream_t stream) {
-    dim3 grid((p.n_qtiles + 1) / 2, p.Hq, p.B);     // one workgroup per PAIR of query tiles
+    dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B));    // one workgroup per PAIR of query tiles, 1-D (see the id remap)
     dim3 block(kPfWaves * 64);
     if (p.mask_mode == MI355_MASK_CAUSAL)
         hipLaunchKernelGGL((prefill_fwd_kernel<D, MI355_MASK_CAUSAL>), grid, block, 0, stream, p);
@@ -382,7 +390,6 @@ extern "C" int mi355_prefill_fwd(const void* q, const void* k, const void* v, vo
         return set_error(MI355_EINVAL, "prefill: B, Hq, Hkv, Sq_max and Sk_max must be positive");
     if (Hq % Hkv != 0) return set_error(MI355_EINVAL, "prefill: Hq must be a multiple of Hkv");
     if (!(D == 128 || D == 64 || D == 32)) return set_error(MI355_EINVAL, "prefill: head_dim must be 32, 64 or 128");
-    if (Hq > 65535 || B > 65535) return set_error(MI355_EINVAL, "prefill: Hq and B must be <= 65535");
     if ((cu_seqlens_q == nullptr) != (cu_seqlens_k == nullptr))
         return set_error(MI355_EINVAL, "prefill: cu_seqlens_q and cu_seqlens_k must be given together");
     if (mask_mode < MI355_MASK_NONE || mask_mode > MI355_MASK_BOOL)
@@ -421,6 +428,8 @@ extern "C" int mi355_prefill_fwd(const void* q, const void* k, const void* v, vo
     p.scale_log2 = softmax_scale * kLog2e;
     p.mask_mode = mask_mode;
     p.n_qtiles = (Sq_max + kBM - 1) / kBM;
+    p.n_pairs = (p.n_qtiles + 1) / 2;
+    if ((int64_t)p.n_pairs * Hq * B > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill: too many workgroups");
 
     hipStream_t s = (hipStream_t)stream;
     int rc = D == 128 ? launch_prefill<128>(p, s) : (D == 64 ? launch_prefill<64>(p, s) : launch_prefill<32>(p, s));
