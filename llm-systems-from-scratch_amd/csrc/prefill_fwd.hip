@@ -233,10 +233,12 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
             constexpr bool MASKED = decltype(masked_c)::value;
             wait_vmcnt<0>();                 // this wavefront's share of tile `tile` has landed
             __syncthreads();                 // ... and everybody's; also: all are done reading the other buffer
-            if (tile + 1 < n_tiles) issue_tile(tile + 1, (tile + 1) & 1);
 
             const int k0 = tile * kBN;
-            if (causal && MASKED && k0 > qw0 + 31 + coff) return false;
+            if (causal && MASKED && k0 > qw0 + 31 + coff) {
+                if (tile + 1 < n_tiles) issue_tile(tile + 1, (tile + 1) & 1);
+                return false;
+            }
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -247,6 +249,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
                     s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s_acc[t]);
                 }
             }
+            // The next tile's direct-to-LDS loads go out only now, after the last K fragment read:
+            // LDS reads issued after them wait until they have landed, so placing them here lets
+            // the rest of the K.Q^T MFMAs and the row-max pass run under the memory latency.
+            if (tile + 1 < n_tiles) issue_tile(tile + 1, (tile + 1) & 1);
+
             // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
             if constexpr (MASKED) {
 #pragma unroll
