@@ -107,6 +107,35 @@ size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx);
 int mi355_paged_decode_chunk_tokens(int max_ctx);
 
 /*
+ * RoPE + KV-cache write: the producer of the paged cache (the step right before the
+ * attention path).  Rotates adjacent pairs (x[2i], x[2i+1]) of q and k by the angle of
+ * (position, i) exactly as RotaryEmbedding.forward does -- llm-core/llm_core/model.py:93-104
+ * -- reading cos/sin from the reference's own table layout `_freq_cache`
+ * (2, context_length, D/2) fp32, model.py:86-91; fp32 math, one rounding to bf16.
+ * The rotated queries go to q_out (may alias q_in); rotated keys and the unrotated values
+ * of token t are scattered to cache slot slot_mapping[t] = block*16 + offset (negative:
+ * token not cached; NULL slot_mapping: rotate q only... k/v are then ignored).
+ * The scatter has no counterpart in the reference (it has no KV cache).
+ *   q_in/q_out (T,Hq,D), k_in/v_in (T,Hkv,D) bf16, heads contiguous, token strides in elements;
+ *   positions int32 (T), each < context_length; k_cache/v_cache (num_blocks,Hkv,16,D) bf16.
+ */
+int mi355_rope_and_cache(const void* q_in, const void* k_in, const void* v_in, void* q_out,
+                         void* k_cache, void* v_cache, const float* freq_cache,
+                         const int32_t* positions, const int64_t* slot_mapping,
+                         int T, int Hq, int Hkv, int D, int context_length,
+                         int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
+                         int64_t q_out_token_stride, void* stream);
+
+/*
+ * Per-(block, kv head) absmax quantisation of a bf16 cache (num_blocks,Hkv,16,D) to OCP
+ * fp8-e4m3 bytes + fp32 scales (num_blocks,Hkv): scale = absmax/448 (1 for an all-zero
+ * slab), value = round_to_nearest_even(clamp(x/scale, +-448)).  No reference counterpart;
+ * it produces the cache format MI355_FP8_E4M3 of mi355_paged_decode_fwd.
+ */
+int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, float* scale,
+                          int64_t num_blocks, int Hkv, int D, int block_size, void* stream);
+
+/*
  * Plain device-to-device copy of `bytes` bytes (16-byte aligned).  Measurement aid
  * with no counterpart in the reference: a copy of known size whose FETCH_SIZE /
  * WRITE_SIZE counter readings calibrate the HBM-traffic figures of the kernels above.

@@ -7,10 +7,15 @@ llm-core/llm_core/model.py:308-325 and the SDPA slot at model.py:382):
     flash_attn_prefill(q, k, v, causal=True)            # f(Q, K, V, is_causal=True) slot
     flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, ...)
     paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, ...)
+    rope_and_cache(q, k, v, positions, freq_cache, k_cache, v_cache, slot_mapping)   # cache producer
+    quantize_kv_cache_fp8(cache)
 
 Every function runs on the HIP library; there is no CPU or PyTorch fallback.
 """
 from .ops import (  # noqa: F401
+    build_rope_cache,
+    quantize_kv_cache_fp8,
+    rope_and_cache,
     flash_attn_prefill,
     flash_attn_varlen_prefill,
     paged_attention_decode,

@@ -19,6 +19,8 @@ EXPORTS = (
     "mi355_paged_decode_fwd",
     "mi355_paged_decode_workspace_bytes",
     "mi355_paged_decode_chunk_tokens",
+    "mi355_rope_and_cache",
+    "mi355_quantize_kv_fp8",
     "mi355_calib_copy",
     "mi355_last_error",
     "mi355_version",
@@ -50,6 +52,11 @@ def load():
     lib.mi355_paged_decode_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.mi355_paged_decode_chunk_tokens.restype = i32
     lib.mi355_paged_decode_chunk_tokens.argtypes = [i32]
+    lib.mi355_rope_and_cache.restype = i32
+    lib.mi355_rope_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32,
+                                         i64, i64, i64, i64, vp]
+    lib.mi355_quantize_kv_fp8.restype = i32
+    lib.mi355_quantize_kv_fp8.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
     lib.mi355_calib_copy.restype = i32
     lib.mi355_calib_copy.argtypes = [vp, vp, sz, vp]
     lib.mi355_last_error.restype = C.c_char_p

@@ -226,3 +226,65 @@ def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, s
         _lib.MI355_FP8_E4M3 if fp8 else _lib.MI355_BF16, _stream())
     _lib.check(rc, "mi355_paged_decode_fwd")
     return out
+
+
+def build_rope_cache(context_length, d, theta=10000.0, device="cuda"):
+    """cos/sin table in the reference's layout (2, context_length, d/2) fp32, as
+    RotaryEmbedding._build_cache builds it (llm-core/llm_core/model.py:86-91)."""
+    inv_freq = theta ** -(torch.arange(0, d, 2, dtype=torch.float32) / d)
+    angles = torch.arange(context_length, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    return torch.stack((torch.cos(angles), torch.sin(angles))).to(device)
+
+
+def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, slot_mapping=None):
+    """RoPE on q and k (interleaved pairs, llm-core/llm_core/model.py:93-104) and scatter of the
+    rotated k and of v into the paged cache.
+
+    q (T,Hq,D), k, v (T,Hkv,D) bf16 with contiguous heads; positions (T,) int32; freq_cache
+    (2, context_length, D/2) fp32; slot_mapping (T,) int64 = block*16 + offset (negative: skip).
+    Returns the rotated q (T,Hq,D); the caches are updated in place.
+    """
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        _require_gpu_bf16(n, t)
+        if t.dim() != 3 or t.stride(2) != 1 or t.stride(1) != t.shape[2]:
+            raise ValueError(f"{n} must be (tokens, heads, d_head) with contiguous heads")
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    if k.shape != v.shape or k.shape[0] != T or k.shape[2] != D:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if freq_cache.dtype != torch.float32 or freq_cache.dim() != 3 or freq_cache.shape[0] != 2 \
+            or freq_cache.shape[2] * 2 != D or not freq_cache.is_contiguous() or not freq_cache.is_cuda:
+        raise ValueError("freq_cache must be a contiguous float32 GPU tensor (2, context_length, d_head/2)")
+    if positions.dtype != torch.int32 or positions.shape != (T,) or not positions.is_contiguous():
+        raise TypeError("positions must be a contiguous int32 (tokens,) tensor")
+    if slot_mapping is not None:
+        if slot_mapping.dtype != torch.int64 or slot_mapping.shape != (T,) or not slot_mapping.is_contiguous():
+            raise TypeError("slot_mapping must be a contiguous int64 (tokens,) tensor")
+        for n, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+            if c is None or c.dtype != torch.bfloat16 or c.dim() != 4 or c.shape[1:] != (Hkv, _BLOCK, D) \
+                    or not c.is_contiguous():
+                raise ValueError(f"{n} must be a contiguous bf16 (num_blocks, {Hkv}, {_BLOCK}, {D}) tensor")
+    q_out = torch.empty(T, Hq, D, dtype=q.dtype, device=q.device)
+    if T == 0:
+        return q_out
+    rc = _lib.load().mi355_rope_and_cache(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
+        None if slot_mapping is None else k_cache.data_ptr(), None if slot_mapping is None else v_cache.data_ptr(),
+        freq_cache.data_ptr(), positions.data_ptr(), None if slot_mapping is None else slot_mapping.data_ptr(),
+        T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0), _stream())
+    _lib.check(rc, "mi355_rope_and_cache")
+    return q_out
+
+
+def quantize_kv_cache_fp8(cache):
+    """bf16 cache (num_blocks,Hkv,16,D) -> (uint8 e4m3 cache, fp32 scale (num_blocks,Hkv)), scale = absmax/448."""
+    _require_gpu_bf16("cache", cache)
+    if cache.dim() != 4 or cache.shape[2] != _BLOCK or not cache.is_contiguous():
+        raise ValueError(f"cache must be a contiguous (num_blocks, kv_heads, {_BLOCK}, d_head) tensor")
+    nb, Hkv, _, D = cache.shape
+    out = torch.empty(cache.shape, dtype=torch.uint8, device=cache.device)
+    scale = torch.empty(nb, Hkv, dtype=torch.float32, device=cache.device)
+    rc = _lib.load().mi355_quantize_kv_fp8(cache.data_ptr(), out.data_ptr(), scale.data_ptr(), nb, Hkv, D, _BLOCK,
+                                           _stream())
+    _lib.check(rc, "mi355_quantize_kv_fp8")
+    return out, scale

@@ -234,6 +234,42 @@ def combine_splits_reference(parts):
 
 
 # --------------------------------------------------------------------------
+# RoPE + cache write (the step before the path)
+# --------------------------------------------------------------------------
+def build_rope_cache(context_length, d, theta=10000.0):
+    """(2, context_length, d/2) cos/sin table; follows llm-core/llm_core/model.py:86-91."""
+    inv_freq = theta ** -(torch.arange(0, d, 2) / d)
+    angles = torch.arange(context_length)[:, None] * inv_freq[None, :]
+    return torch.stack((torch.cos(angles), torch.sin(angles)))
+
+
+def rope_reference(x, pos_ids, freq_cache):
+    """Interleaved-pair rotation; follows llm-core/llm_core/model.py:93-104.  x (..., seq, d), pos_ids (..., seq)."""
+    x1 = x[..., 0::2]
+    x2 = x[..., 1::2]
+    cos, sin = freq_cache[:, pos_ids, :]
+    x1_rot = cos * x1 - sin * x2
+    x2_rot = sin * x1 + cos * x2
+    return torch.stack((x1_rot, x2_rot), dim=-1).flatten(-2)
+
+
+def rope_and_cache_reference(q, k, v, positions, freq_cache, k_cache, v_cache, slot_mapping):
+    """q (T,Hq,D), k/v (T,Hkv,D): returns rotated q (fp32) and updates fp32 copies of the caches."""
+    pos = positions.long()
+    q_rot = rope_reference(q.float().transpose(0, 1), pos, freq_cache).transpose(0, 1)
+    k_rot = rope_reference(k.float().transpose(0, 1), pos, freq_cache).transpose(0, 1)
+    kc, vc = k_cache.float().clone(), v_cache.float().clone()
+    bs = kc.shape[2]
+    for t in range(q.shape[0]):
+        s = int(slot_mapping[t])
+        if s < 0:
+            continue
+        kc[s // bs, :, s % bs] = k_rot[t]
+        vc[s // bs, :, s % bs] = v[t].float()
+    return q_rot, kc, vc
+
+
+# --------------------------------------------------------------------------
 # Independent brute force (float64 loops) used only to pin the functions above
 # --------------------------------------------------------------------------
 def bruteforce_attention_f64(Q, K, V, keep=None):

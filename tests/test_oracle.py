@@ -298,3 +298,42 @@ def test_workload_generators_are_seeded_and_well_formed():
                                             context_lens=[256] * 4, seed=0)
     assert kc.shape == (64, 8, 16, 64) and bt.shape == (4, 16)
     assert sorted(bt.flatten().tolist()) == list(range(64))     # a permutation of the 64 physical blocks
+
+
+# ---- RoPE ------------------------------------------------------------------
+def test_rope_equals_complex_rotation_and_cache_layout():
+    d, ctx = 16, 50
+    fc = orc.build_rope_cache(ctx, d)
+    assert fc.shape == (2, ctx, d // 2)
+    x = rnd(3, 7, d, seed=80)
+    pos = torch.tensor([0, 1, 5, 17, 49, 3, 3])
+    got = orc.rope_reference(x, pos, fc)
+    # independent formulation: (x1 + i x2) * exp(i * pos * theta^(-2j/d)), in float64
+    inv = 10000.0 ** (-np.arange(0, d, 2) / d)
+    ang = pos.numpy()[:, None] * inv[None, :]
+    z = (x[..., 0::2].numpy().astype(np.float64) + 1j * x[..., 1::2].numpy().astype(np.float64)) * np.exp(1j * ang)
+    want = np.stack([z.real, z.imag], axis=-1).reshape(3, 7, d)
+    np.testing.assert_allclose(got.numpy(), want, atol=2e-5, rtol=1e-5)
+    torch.testing.assert_close(got[:, 0], x[:, 0])                       # position 0 is the identity
+    # pair norms are preserved and scores depend on the position difference only
+    torch.testing.assert_close(got.pow(2).unflatten(-1, (d // 2, 2)).sum(-1), x.pow(2).unflatten(-1, (d // 2, 2)).sum(-1),
+                               atol=1e-5, rtol=1e-5)
+    a, b = rnd(1, d, seed=81), rnd(1, d, seed=82)
+    s1 = (orc.rope_reference(a, torch.tensor([9]), fc) * orc.rope_reference(b, torch.tensor([4]), fc)).sum()
+    s2 = (orc.rope_reference(a, torch.tensor([25]), fc) * orc.rope_reference(b, torch.tensor([20]), fc)).sum()
+    torch.testing.assert_close(s1, s2, atol=1e-4, rtol=1e-4)
+
+
+def test_rope_and_cache_reference_scatters_to_slots():
+    T, Hq, Hkv, D = 5, 4, 2, 8
+    fc = orc.build_rope_cache(32, D)
+    q, k, v = rnd(T, Hq, D, seed=83), rnd(T, Hkv, D, seed=84), rnd(T, Hkv, D, seed=85)
+    pos = torch.tensor([3, 4, 5, 0, 9], dtype=torch.int32)
+    slots = torch.tensor([16 * 2 + 3, 16 * 2 + 4, 16 * 0 + 15, -1, 16 * 1 + 0])
+    kc, vc = torch.zeros(3, Hkv, 16, D), torch.zeros(3, Hkv, 16, D)
+    q_rot, kc2, vc2 = orc.rope_and_cache_reference(q, k, v, pos, fc, kc, vc, slots)
+    torch.testing.assert_close(q_rot[3], q[3])                                  # position 0
+    torch.testing.assert_close(vc2[2, :, 3], v[0])
+    torch.testing.assert_close(vc2[0, :, 15], v[2])
+    torch.testing.assert_close(kc2[1, :, 0], orc.rope_reference(k[4][:, None], torch.tensor([9]), fc)[:, 0])
+    assert kc2.abs().sum(dim=(1, 3)).count_nonzero() == 4                       # token 3 (slot -1) was not written
