@@ -23,4 +23,5 @@ from .ops import (  # noqa: F401
     scaled_dot_product_attention,
     sdpa_slot,
 )
+from .engine import BlockAllocator, OutOfBlocks, PagedAttentionEngine  # noqa: F401
 from ._lib import LIB_PATH, LibraryMissing, load  # noqa: F401
