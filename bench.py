@@ -13,7 +13,7 @@ The CPU baseline is the oracle (a restatement of the reference's PyTorch attenti
 timed on the host cores over a bounded sample of the same inputs; its outputs also
 check the GPU results of that sample.
 
-usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--seed S] [--only decode|prefill|fp8]
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--seed S] [--only decode|prefill|fp8|producers]
                        [--no-cpu]
 """
 from __future__ import annotations
@@ -96,7 +96,71 @@ def bench_decode(cfg, args, with_cpu):
     return res
 
 
-def cpu_decode(case, gpu_out, cfg, n_seq=48):
+def bench_producers(args):
+    """The two cache producers at the shapes the attention configs imply: RoPE + cache write for the
+    32768 packed tokens of configs[2], and fp8 quantisation of a K pool of configs[4]'s size."""
+    import torch
+    import mi355_attn
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(args.seed)
+    res = {}
+    # --- rope_and_cache: T = 8 x 4096 tokens, 32 q / 8 kv heads, head_dim 128, blocks dealt as a random permutation
+    B, S, Hq, Hkv, D = 8, 4096, 32, 8, 128
+    T = B * S
+    q = torch.randn(T, Hq, D, device=dev, generator=g).mul_(0.5).to(torch.bfloat16)
+    k = torch.randn(T, Hkv, D, device=dev, generator=g).mul_(0.5).to(torch.bfloat16)
+    v = torch.randn(T, Hkv, D, device=dev, generator=g).mul_(0.5).to(torch.bfloat16)
+    n_blocks = T // 16
+    perm = torch.randperm(n_blocks, device=dev, generator=g)
+    slots = (perm.repeat_interleave(16) * 16 + torch.arange(16, device=dev).repeat(n_blocks)).to(torch.int64)
+    pos = torch.arange(S, device=dev, dtype=torch.int32).repeat(B)
+    freq = mi355_attn.build_rope_cache(S, D, 10000.0, dev)
+    k_cache = torch.zeros(n_blocks, Hkv, 16, D, dtype=torch.bfloat16, device=dev)
+    v_cache = torch.zeros_like(k_cache)
+    q_out = torch.empty_like(q)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.rope_and_cache(q, k, v, pos, freq, k_cache, v_cache, slots, out=q_out),
+                            args.steps, args.warmup)
+    nbytes = 2 * (q.numel() + k.numel() + v.numel()) * 2 + T * 12 + freq.numel() * 4
+    res["rope_and_cache"] = {
+        "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 (fp32 rotation)",
+        "config": {"workload": "RoPE + paged cache write of configs[2]'s 32768 packed tokens (32 q / 8 kv heads, "
+                               "head_dim 128), blocks a random permutation", "algorithmic_bytes": nbytes},
+        "roofline": {"bound": "hbm", "kernel": "rope_and_cache_kernel", "achieved": nbytes / dev_ms / 1e6,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS,
+                     "device_ms": dev_ms, "traffic": _traffic("rope_and_cache")},
+    }
+    del q, k, v, q_out, k_cache, v_cache
+    # --- quantize_kv_fp8: a pool of configs[4]'s size (about 103k blocks x 8 kv heads x 16 x 128)
+    nb = 103_000
+    pool = torch.randn(nb, Hkv, 16, D, device=dev, generator=g).to(torch.bfloat16)
+    out8 = torch.empty(nb, Hkv, 16, D, dtype=torch.uint8, device=dev)
+    scale = torch.empty(nb, Hkv, dtype=torch.float32, device=dev)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.quantize_kv_cache_fp8(pool, out=(out8, scale)), args.steps, args.warmup)
+    nbytes = pool.numel() * 3 + scale.numel() * 4
+    res["quantize_kv_fp8"] = {
+        "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 -> fp8-e4m3",
+        "config": {"workload": f"per-(block, kv head) fp8 quantisation of a {nb}-block bf16 pool (8 kv heads, block 16, "
+                               "head_dim 128)", "algorithmic_bytes": nbytes},
+        "roofline": {"bound": "hbm", "kernel": "quantize_kv_fp8_kernel", "achieved": nbytes / dev_ms / 1e6,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS,
+                     "device_ms": dev_ms, "traffic": _traffic("quantize_kv_fp8")},
+    }
+    return res
+
+
+def _timed_repeats(fn, min_seconds=10.0, max_reps=20):
+    """Run fn until min_seconds of wall time have been spent; returns (last result, seconds per call, calls)."""
+    total, reps, out = 0.0, 0, None
+    while total < min_seconds and reps < max_reps:
+        t0 = time.perf_counter()
+        out = fn()
+        total += time.perf_counter() - t0
+        reps += 1
+    return out, total / reps, reps
+
+
+def cpu_decode(case, gpu_out, cfg, n_seq=128):
     """Oracle on the host cores over the first n_seq sequences; also checks the GPU result of those."""
     import torch
     from oracle import attention_oracle as orc
@@ -116,17 +180,15 @@ def cpu_decode(case, gpu_out, cfg, n_seq=48):
         off += int(nblk[b])
     q = case.q[:n_seq].cpu()
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
-    t0 = time.perf_counter()
-    ref = orc.paged_decode_reference(q, kc, vc, bt, ctx, k_scale=ks, v_scale=vs)
-    dt = time.perf_counter() - t0
+    ref, dt, reps = _timed_repeats(lambda: orc.paged_decode_reference(q, kc, vc, bt, ctx, k_scale=ks, v_scale=vs))
     per_token = 2 * kc.shape[1] * kc.shape[3] * kc.element_size() + (8 * kc.shape[1] / 16 if ks is not None else 0)
     sample_bytes = int(ctx.sum()) * per_token
     err = (gpu_out[:n_seq].float().cpu() - ref).abs()
     bound = 2e-2 + 1e-2 * ref.abs()
     base = {"value": sample_bytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-            "seconds": dt,
+            "seconds_per_pass": dt, "passes": reps,
             "sample": f"configs[{cfg}] first {n_seq} of {case.q.shape[0]} sequences ({int(ctx.sum())} tokens), "
-                      "oracle paged_decode_reference, torch CPU fp32"}
+                      f"{reps} passes of oracle paged_decode_reference, torch CPU fp32"}
     parity = {"checked_sequences": n_seq, "max_abs_err": float(err.max()),
               "within_2e-2_abs_1e-2_rel": bool((err <= bound).all())}
     return base, parity
@@ -185,16 +247,14 @@ def cpu_prefill(case, gpu_out, cfg, n_heads=8):
         q, k, v = (t[:1, :n_heads].cpu() for t in (case.q, case.k, case.v))
         got = gpu_out[:1, :n_heads].float().cpu()
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
-    t0 = time.perf_counter()
-    ref = orc.prefill_reference(q, k, v, causal=True, head_chunk=4)
-    dt = time.perf_counter() - t0
+    ref, dt, reps = _timed_repeats(lambda: orc.prefill_reference(q, k, v, causal=True, head_chunk=4))
     flops = 4 * n_heads * q.shape[-1] * S * S // 2
     err = (got - ref).abs()
     bound = 2e-2 + 1e-2 * ref.abs()
     base = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-            "seconds": dt,
-            "sample": f"configs[{cfg}] sequence 0, query heads 0..{n_heads - 1} (S={S}), oracle prefill_reference, "
-                      "torch CPU fp32, causal-convention FLOPs"}
+            "seconds_per_pass": dt, "passes": reps,
+            "sample": f"configs[{cfg}] sequence 0, query heads 0..{n_heads - 1} (S={S}), {reps} passes of oracle "
+                      "prefill_reference, torch CPU fp32, causal-convention FLOPs"}
     parity = {"checked_heads": n_heads, "max_abs_err": float(err.max()),
               "within_2e-2_abs_1e-2_rel": bool((err <= bound).all())}
     return base, parity
@@ -206,7 +266,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", choices=["decode", "prefill", "fp8"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "fp8", "producers"], default=None)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the 1 GiB plain copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
@@ -276,6 +336,8 @@ def main():
                          "dtype": f8["dtype"], "config": f8["config"], "roofline": f8["roofline"]})
             if with_cpu:
                 line["cpu_baseline"] = f8["cpu_baseline"]
+    if args.only in (None, "producers"):
+        line["cache_producers"] = bench_producers(args)
     print(json.dumps(line))
 
 

@@ -62,21 +62,60 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeCacheParams p) 
     }
 }
 
+// The same work with 16-byte accesses: one thread per (token, head slot, group of 4 pairs).
+// Requires D % 8 == 0, token strides that are multiples of 8 elements and 16-byte aligned bases.
+__global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParams p) {
+    const int groups = p.D / 8;
+    const int half = p.D / 2;
+    const int slots_per_tok = p.Hq + 2 * p.Hkv;
+    const int64_t total = (int64_t)p.T * slots_per_tok * groups;
+    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(idx % groups);
+        const int hs = (int)((idx / groups) % slots_per_tok);
+        const int t = (int)(idx / ((int64_t)groups * slots_per_tok));
+        const int64_t slot = p.slots ? p.slots[t] : -1;
+        const bool is_q = hs < p.Hq;
+        if (!is_q && slot < 0) continue;
+        const bool is_v = hs >= p.Hq + p.Hkv;
+        const int hk = is_v ? hs - p.Hq - p.Hkv : hs - p.Hq;
+        const __bf16* src = is_q ? p.q_in + t * p.q_tok + (int64_t)hs * p.D
+                                 : (is_v ? p.v_in + t * p.v_tok : p.k_in + t * p.k_tok) + (int64_t)hk * p.D;
+        u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 8 * c));
+        if (!is_v) {
+            const int pos = p.positions[t];
+            const f32x4 cs = *reinterpret_cast<const f32x4*>(p.freq + (int64_t)pos * half + 4 * c);
+            const f32x4 sn = *reinterpret_cast<const f32x4*>(p.freq + ((int64_t)p.ctx_len + pos) * half + 4 * c);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t w = raw[j];           // scalar copy first: a bit_cast of a vector element misreads it
+                const bf16x2 x = __builtin_bit_cast(bf16x2, w);
+                const float x1 = (float)x[0], x2 = (float)x[1];
+                raw[j] = pack_bf16(cs[j] * x1 - sn[j] * x2, sn[j] * x1 + cs[j] * x2);
+            }
+        }
+        __bf16* dst = is_q ? p.q_out + t * p.qo_tok + (int64_t)hs * p.D
+                           : (is_v ? p.v_cache : p.k_cache) + (((slot >> 4) * p.Hkv + hk) * 16 + (slot & 15)) * p.D;
+        *reinterpret_cast<u32x4*>(dst + 8 * c) = raw;
+    }
+}
+
 // One wavefront per (block, kv head) slab of 16*D bf16: absmax -> scale = absmax/448 (1 for an
 // all-zero slab) -> x/scale clamped to +-448 -> e4m3 (round to nearest even).
 template <int D>
-__global__ __launch_bounds__(64) void quantize_kv_fp8_kernel(const __bf16* __restrict__ src, unsigned char* __restrict__ dst,
-                                                            float* __restrict__ scale, int64_t n_slabs) {
-    constexpr int PER_LANE = 16 * D / 64;           // elements per lane (multiple of 8)
-    constexpr int NV = PER_LANE / 8;                // 16-byte loads per lane
-    const int lane = threadIdx.x;
-    for (int64_t slab = blockIdx.x; slab < n_slabs; slab += gridDim.x) {
-        const __bf16* s = src + slab * (16 * D) + lane * PER_LANE;
+__global__ __launch_bounds__(256) void quantize_kv_fp8_kernel(const __bf16* __restrict__ src, unsigned char* __restrict__ dst,
+                                                             float* __restrict__ scale, int64_t n_slabs) {
+    constexpr int NV = 16 * D / 8 / 64;             // 16-byte loads per lane: load j covers elements [512 j, 512 j + 512)
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    for (int64_t slab = wave; slab < n_slabs; slab += (int64_t)gridDim.x * 4) {
+        const __bf16* s = src + slab * (16 * D) + lane * 8;
         u32x4 raw[NV];
         float amax = 0.f;
 #pragma unroll
+        for (int j = 0; j < NV; ++j) raw[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + 512 * j));
+#pragma unroll
         for (int j = 0; j < NV; ++j) {
-            raw[j] = *reinterpret_cast<const u32x4*>(s + 8 * j);
             const bf16x8 x = as_bf16x8(raw[j]);
 #pragma unroll
             for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf((float)x[e]));
@@ -85,7 +124,7 @@ __global__ __launch_bounds__(64) void quantize_kv_fp8_kernel(const __bf16* __res
         for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
         const float sc = amax > 0.f ? amax / 448.0f : 1.0f;
         if (lane == 0) scale[slab] = sc;
-        unsigned char* d = dst + slab * (16 * D) + lane * PER_LANE;
+        unsigned char* d = dst + slab * (16 * D) + lane * 8;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const bf16x8 x = as_bf16x8(raw[j]);
@@ -100,7 +139,7 @@ __global__ __launch_bounds__(64) void quantize_kv_fp8_kernel(const __bf16* __res
             u32x2 out;
             out[0] = (uint32_t)w0;
             out[1] = (uint32_t)w1;
-            *reinterpret_cast<u32x2*>(d + 8 * j) = out;
+            *reinterpret_cast<u32x2*>(d + 512 * j) = out;
         }
     }
 }
@@ -143,10 +182,17 @@ extern "C" int mi355_rope_and_cache(const void* q_in, const void* k_in, const vo
     p.Hkv = Hkv;
     p.D = D;
     p.ctx_len = context_length;
-    const int64_t total = (int64_t)T * (Hq + 2 * Hkv) * (D / 2);
+    const auto aligned16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+    const bool vec8 = D % 8 == 0 && ((q_token_stride | k_token_stride | v_token_stride | q_out_token_stride) & 7) == 0 &&
+                      aligned16(q_in) && aligned16(k_in) && aligned16(v_in) && aligned16(q_out) && aligned16(k_cache) &&
+                      aligned16(v_cache) && aligned16(freq_cache);
+    const int64_t total = (int64_t)T * (Hq + 2 * Hkv) * (vec8 ? D / 8 : D / 2);
     const int64_t blocks = (total + 255) / 256;
     const unsigned grid = (unsigned)(blocks < 256 * 64 ? blocks : 256 * 64);
-    hipLaunchKernelGGL(rope_and_cache_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, p);
+    if (vec8)
+        hipLaunchKernelGGL(rope_and_cache_vec8_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, p);
+    else
+        hipLaunchKernelGGL(rope_and_cache_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, p);
     const int rc = (int)hipGetLastError();
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;
@@ -160,16 +206,17 @@ extern "C" int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, fl
     if (!(D == 32 || D == 64 || D == 128)) return set_error(MI355_EINVAL, "quantize_kv_fp8: head_dim must be 32, 64 or 128");
     const int64_t n_slabs = num_blocks * Hkv;
     if (n_slabs == 0) return MI355_OK;
-    const unsigned grid = (unsigned)(n_slabs < 256 * 256 ? n_slabs : 256 * 256);
+    const int64_t wgs = (n_slabs + 3) / 4;                  // four wavefronts (slabs) per workgroup
+    const unsigned grid = (unsigned)(wgs < 256 * 64 ? wgs : 256 * 64);
     hipStream_t s = (hipStream_t)stream;
     if (D == 128)
-        hipLaunchKernelGGL(quantize_kv_fp8_kernel<128>, dim3(grid), dim3(64), 0, s, (const __bf16*)cache_bf16,
+        hipLaunchKernelGGL(quantize_kv_fp8_kernel<128>, dim3(grid), dim3(256), 0, s, (const __bf16*)cache_bf16,
                            (unsigned char*)cache_fp8, scale, n_slabs);
     else if (D == 64)
-        hipLaunchKernelGGL(quantize_kv_fp8_kernel<64>, dim3(grid), dim3(64), 0, s, (const __bf16*)cache_bf16,
+        hipLaunchKernelGGL(quantize_kv_fp8_kernel<64>, dim3(grid), dim3(256), 0, s, (const __bf16*)cache_bf16,
                            (unsigned char*)cache_fp8, scale, n_slabs);
     else
-        hipLaunchKernelGGL(quantize_kv_fp8_kernel<32>, dim3(grid), dim3(64), 0, s, (const __bf16*)cache_bf16,
+        hipLaunchKernelGGL(quantize_kv_fp8_kernel<32>, dim3(grid), dim3(256), 0, s, (const __bf16*)cache_bf16,
                            (unsigned char*)cache_fp8, scale, n_slabs);
     const int rc = (int)hipGetLastError();
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));

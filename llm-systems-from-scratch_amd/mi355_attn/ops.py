@@ -236,13 +236,14 @@ def build_rope_cache(context_length, d, theta=10000.0, device="cuda"):
     return torch.stack((torch.cos(angles), torch.sin(angles))).to(device)
 
 
-def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, slot_mapping=None):
+def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, slot_mapping=None, *, out=None):
     """RoPE on q and k (interleaved pairs, llm-core/llm_core/model.py:93-104) and scatter of the
     rotated k and of v into the paged cache.
 
     q (T,Hq,D), k, v (T,Hkv,D) bf16 with contiguous heads; positions (T,) int32; freq_cache
     (2, context_length, D/2) fp32; slot_mapping (T,) int64 = block*16 + offset (negative: skip).
-    Returns the rotated q (T,Hq,D); the caches are updated in place.
+    Returns the rotated q (T,Hq,D) (written into `out` when given; `out` may be q itself); the
+    caches are updated in place.
     """
     for n, t in (("q", q), ("k", k), ("v", v)):
         _require_gpu_bf16(n, t)
@@ -264,7 +265,13 @@ def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, s
             if c is None or c.dtype != torch.bfloat16 or c.dim() != 4 or c.shape[1:] != (Hkv, _BLOCK, D) \
                     or not c.is_contiguous():
                 raise ValueError(f"{n} must be a contiguous bf16 (num_blocks, {Hkv}, {_BLOCK}, {D}) tensor")
-    q_out = torch.empty(T, Hq, D, dtype=q.dtype, device=q.device)
+    if out is None:
+        q_out = torch.empty(T, Hq, D, dtype=q.dtype, device=q.device)
+    else:
+        q_out = out
+        _require_gpu_bf16("out", q_out)
+        if q_out.shape != q.shape or q_out.stride(2) != 1 or q_out.stride(1) != D:
+            raise ValueError("out must have q's shape with contiguous heads")
     if T == 0:
         return q_out
     rc = _lib.load().mi355_rope_and_cache(
@@ -276,14 +283,23 @@ def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, s
     return q_out
 
 
-def quantize_kv_cache_fp8(cache):
-    """bf16 cache (num_blocks,Hkv,16,D) -> (uint8 e4m3 cache, fp32 scale (num_blocks,Hkv)), scale = absmax/448."""
+def quantize_kv_cache_fp8(cache, *, out=None):
+    """bf16 cache (num_blocks,Hkv,16,D) -> (uint8 e4m3 cache, fp32 scale (num_blocks,Hkv)), scale = absmax/448.
+    `out` = (uint8 cache, fp32 scale) tensors to write into instead of new ones."""
     _require_gpu_bf16("cache", cache)
     if cache.dim() != 4 or cache.shape[2] != _BLOCK or not cache.is_contiguous():
         raise ValueError(f"cache must be a contiguous (num_blocks, kv_heads, {_BLOCK}, d_head) tensor")
     nb, Hkv, _, D = cache.shape
-    out = torch.empty(cache.shape, dtype=torch.uint8, device=cache.device)
-    scale = torch.empty(nb, Hkv, dtype=torch.float32, device=cache.device)
+    if out is None:
+        out = torch.empty(cache.shape, dtype=torch.uint8, device=cache.device)
+        scale = torch.empty(nb, Hkv, dtype=torch.float32, device=cache.device)
+    else:
+        out, scale = out
+        if out.dtype != torch.uint8 or out.shape != cache.shape or not out.is_contiguous() or out.device != cache.device:
+            raise ValueError("out[0] must be a contiguous uint8 tensor of the cache's shape on its device")
+        if scale.dtype != torch.float32 or scale.shape != (nb, Hkv) or not scale.is_contiguous() \
+                or scale.device != cache.device:
+            raise ValueError("out[1] must be a contiguous float32 (num_blocks, kv_heads) tensor on the cache's device")
     rc = _lib.load().mi355_quantize_kv_fp8(cache.data_ptr(), out.data_ptr(), scale.data_ptr(), nb, Hkv, D, _BLOCK,
                                            _stream())
     _lib.check(rc, "mi355_quantize_kv_fp8")

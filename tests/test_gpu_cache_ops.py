@@ -46,6 +46,35 @@ def test_rope_and_cache_matches_oracle(ops, D):
     assert torch.equal(q_rot[0].cpu(), q[0])                          # position 0: identity, exact
 
 
+def test_rope_and_cache_pair_path_and_out_argument(ops):
+    """Token strides that are not multiples of 8 elements take the 4-byte kernel; it and the
+    16-byte kernel must give identical bits.  Also covers out= (in place on q)."""
+    print("case: rope_and_cache pair path / out=", flush=True)
+    T, Hq, Hkv, D, ctx = 53, 4, 2, 64, 128
+    g = torch.Generator().manual_seed(11)
+    pos = torch.randint(0, ctx, (T,), generator=g).to(torch.int32).cuda()
+    slots = torch.randperm(4 * 16, generator=g)[:T].to(torch.int64).cuda()
+    fcg = ops.build_rope_cache(ctx, D)
+    q, k, v = rnd(T, Hq, D, seed=12).cuda(), rnd(T, Hkv, D, seed=13).cuda(), rnd(T, Hkv, D, seed=14).cuda()
+    kc_a, vc_a = torch.zeros(4, Hkv, 16, D, dtype=torch.bfloat16, device="cuda"), torch.zeros(4, Hkv, 16, D, dtype=torch.bfloat16, device="cuda")
+    kc_b, vc_b = torch.zeros_like(kc_a), torch.zeros_like(vc_a)
+    q_a = ops.rope_and_cache(q, k, v, pos, fcg, kc_a, vc_a, slots)
+    # the same rows inside a wider buffer: token stride Hq*D + 2 elements (even, not a multiple of 8)
+    wide = torch.zeros(T, Hq * D + 2, dtype=torch.bfloat16, device="cuda")
+    q_view = wide[:, :Hq * D].view(T, Hq, D)
+    q_view.copy_(q)
+    assert q_view.stride(0) % 8 != 0
+    q_b = ops.rope_and_cache(q_view, k, v, pos, fcg, kc_b, vc_b, slots)
+    torch.cuda.synchronize()
+    assert torch.equal(q_a, q_b) and torch.equal(kc_a, kc_b) and torch.equal(vc_a, vc_b)
+    q_inplace = q.clone()
+    ret = ops.rope_and_cache(q_inplace, k, v, pos, fcg, kc_b, vc_b, slots, out=q_inplace)
+    torch.cuda.synchronize()
+    assert ret is q_inplace and torch.equal(q_inplace, q_a)
+    with pytest.raises(ValueError):
+        ops.rope_and_cache(q, k, v, pos, fcg, kc_b, vc_b, slots, out=torch.empty(T, Hq, D + 8, dtype=torch.bfloat16, device="cuda"))
+
+
 @pytest.mark.parametrize("D", [32, 64, 128])
 def test_quantize_kv_fp8_is_bit_exact(ops, D):
     print(f"case: quantize D={D}", flush=True)
@@ -56,6 +85,10 @@ def test_quantize_kv_fp8_is_bit_exact(ops, D):
     torch.cuda.synchronize()
     assert torch.equal(sc.cpu(), sc_ref)
     assert torch.equal(q8.cpu(), q8_ref)
+    out8, outs = torch.zeros_like(q8), torch.zeros_like(sc)
+    ops.quantize_kv_cache_fp8(cache.cuda(), out=(out8, outs))
+    torch.cuda.synchronize()
+    assert torch.equal(out8, q8) and torch.equal(outs, sc)
 
 
 def test_decode_loop_over_growing_cache_equals_causal_prefill(ops):
