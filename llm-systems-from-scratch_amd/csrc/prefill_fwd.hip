@@ -134,13 +134,13 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
     auto issue_tile = [&](int tile, int buf) {
         const unsigned char* kbase = reinterpret_cast<const unsigned char*>(kb + (int64_t)tile * kBN * p.ks[2]);
         const unsigned char* vbase = reinterpret_cast<const unsigned char*>(vb + (int64_t)tile * kBN * p.vs[2]);
-        unsigned char* kdst = k_lds + buf * kTile + wave * NI * 1024;
-        unsigned char* vdst = v_lds + buf * kTile + wave * NI * 1024;
+        const uint32_t kdst = __builtin_amdgcn_readfirstlane(lds_address(k_lds + buf * kTile + wave * NI * 1024));
+        const uint32_t vdst = __builtin_amdgcn_readfirstlane(lds_address(v_lds + buf * kTile + wave * NI * 1024));
         if (tile * kBN + kBN <= sk) {
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
-                load_to_lds_16(kbase + k_voff[j], kdst + j * 1024);
-                load_to_lds_16(vbase + v_voff[j], vdst + j * 1024);
+                dma_to_lds_16(kbase, k_voff[j], kdst + j * 1024);
+                dma_to_lds_16(vbase, v_voff[j], vdst + j * 1024);
             }
         } else {
             // last, partial tile: rows past the end re-read the last row (finite; their scores are masked)
@@ -148,8 +148,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
                 const int row = min(ld_row[j], last);
-                load_to_lds_16(kbase + (uint32_t)(row * (int)p.ks[2] * 2 + ld_col[j]), kdst + j * 1024);
-                load_to_lds_16(vbase + (uint32_t)(row * (int)p.vs[2] * 2 + ld_col[j]), vdst + j * 1024);
+                dma_to_lds_16(kbase, (uint32_t)(row * (int)p.ks[2] * 2 + ld_col[j]), kdst + j * 1024);
+                dma_to_lds_16(vbase, (uint32_t)(row * (int)p.vs[2] * 2 + ld_col[j]), vdst + j * 1024);
             }
         }
     };
@@ -234,11 +234,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
             wait_vmcnt<0>();                 // this wavefront's share of tile `tile` has landed
             __syncthreads();                 // ... and everybody's; also: all are done reading the other buffer
 
+            // The next tile's direct-to-LDS loads go out first: a whole tile of work hides their latency.
+            if (tile + 1 < n_tiles) issue_tile(tile + 1, (tile + 1) & 1);
+
             const int k0 = tile * kBN;
-            if (causal && MASKED && k0 > qw0 + 31 + coff) {
-                if (tile + 1 < n_tiles) issue_tile(tile + 1, (tile + 1) & 1);
-                return false;
-            }
+            if (causal && MASKED && k0 > qw0 + 31 + coff) return false;
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -249,11 +249,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
                     s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s_acc[t]);
                 }
             }
-            // The next tile's direct-to-LDS loads go out only now, after the last K fragment read:
-            // LDS reads issued after them wait until they have landed, so placing them here lets
-            // the rest of the K.Q^T MFMAs and the row-max pass run under the memory latency.
-            if (tile + 1 < n_tiles) issue_tile(tile + 1, (tile + 1) & 1);
-
             // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
             if constexpr (MASKED) {
 #pragma unroll
