@@ -13,7 +13,7 @@ The CPU baseline is the oracle (a restatement of the reference's PyTorch attenti
 timed on the host cores over a bounded sample of the same inputs; its outputs also
 check the GPU results of that sample.
 
-usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--seed S] [--only decode|prefill|fp8|producers]
+usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|fp8|producers]
                        [--no-cpu]
 """
 from __future__ import annotations
@@ -263,8 +263,8 @@ def cpu_prefill(case, gpu_out, cfg, n_heads=8):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", choices=["decode", "prefill", "fp8", "producers"], default=None)
     ap.add_argument("--no-cpu", action="store_true")
