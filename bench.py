@@ -13,7 +13,7 @@ The CPU baseline is the oracle (a restatement of the reference's PyTorch attenti
 timed on the host cores over a bounded sample of the same inputs; its outputs also
 check the GPU results of that sample.
 
-usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|fp8|producers]
+usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|fp8|producers|layer]
                        [--no-cpu]
 """
 from __future__ import annotations
@@ -149,6 +149,43 @@ def bench_producers(args):
     return res
 
 
+def bench_layer_ops(args):
+    """RMSNorm (with the fused residual add) and silu(gate)*up on the activations of configs[2]'s
+    32768 tokens at d_model 4096 (32 heads x 128) and d_ff 11008."""
+    import torch
+    import mi355_attn
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(args.seed)
+    T, d, ff = 32768, 4096, 11008
+    res = {}
+    x = torch.randn(T, d, device=dev, generator=g).to(torch.bfloat16)
+    r = torch.randn(T, d, device=dev, generator=g).to(torch.bfloat16)
+    w = torch.ones(d, device=dev)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.rms_norm(x, w, 1e-5, residual=r, return_sum=True), args.steps, args.warmup)
+    nbytes = 4 * T * d * 2 + d * 4                   # read x, residual; write y, sum
+    res["rms_norm_residual"] = {
+        "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 (fp32 math)",
+        "config": {"workload": f"y, h = rms_norm(x + residual): {T} rows x {d} bf16, fp32 weight", "algorithmic_bytes": nbytes},
+        "roofline": {"bound": "hbm", "kernel": "rms_norm_rows_kernel<8>", "achieved": nbytes / dev_ms / 1e6,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS,
+                     "device_ms": dev_ms, "traffic": _traffic("rms_norm_residual")},
+    }
+    del x, r
+    gu = torch.randn(T, 2 * ff, device=dev, generator=g).to(torch.bfloat16)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.silu_mul(gu[:, :ff], gu[:, ff:]), args.steps, args.warmup)
+    nbytes = 3 * T * ff * 2
+    res["silu_mul"] = {
+        "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 (fp32 silu)",
+        "config": {"workload": f"silu(gate) * up on the two halves of a ({T}, {2 * ff}) bf16 projection output",
+                   "algorithmic_bytes": nbytes},
+        "roofline": {"bound": "hbm", "kernel": "silu_mul_vec8_kernel", "achieved": nbytes / dev_ms / 1e6,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS,
+                     "device_ms": dev_ms, "traffic": _traffic("silu_mul")},
+    }
+    return res
+
+
 def _timed_repeats(fn, min_seconds=10.0, max_reps=20):
     """Run fn until min_seconds of wall time have been spent; returns (last result, seconds per call, calls)."""
     total, reps, out = 0.0, 0, None
@@ -266,7 +303,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", choices=["decode", "prefill", "fp8", "producers"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "fp8", "producers", "layer"], default=None)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the 1 GiB plain copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
@@ -338,6 +375,8 @@ def main():
                 line["cpu_baseline"] = f8["cpu_baseline"]
     if args.only in (None, "producers"):
         line["cache_producers"] = bench_producers(args)
+    if args.only in (None, "layer"):
+        line["layer_ops"] = bench_layer_ops(args)
     print(json.dumps(line))
 
 

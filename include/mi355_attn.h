@@ -33,7 +33,8 @@ enum {
 /* element type codes */
 enum {
     MI355_BF16 = 0,         /* bfloat16 q/k/v/out and bf16 KV cache              */
-    MI355_FP8_E4M3 = 1      /* OCP fp8-e4m3 KV cache (max 448) + fp32 scales     */
+    MI355_FP8_E4M3 = 1,     /* OCP fp8-e4m3 KV cache (max 448) + fp32 scales     */
+    MI355_FP32 = 2          /* float32 (RMSNorm weight only)                     */
 };
 
 /* mask modes of the prefill entry point */
@@ -134,6 +135,31 @@ int mi355_rope_and_cache(const void* q_in, const void* k_in, const void* v_in, v
  */
 int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, float* scale,
                           int64_t num_blocks, int Hkv, int D, int block_size, void* stream);
+
+/*
+ * RMSNorm forward over the rows of a (n_rows, n_cols) bf16 matrix:
+ *   y = weight * (h * rsqrt(mean(h^2) + eps)),  h = x, or h = bf16(x + residual)
+ * fp32 math, one rounding to bf16 -- RMSNorm.forward, llm-core/llm_core/model.py:60-67, and the
+ * forward of its Triton twin, llm-systems/llm_systems/kernels/triton_rms_norm.py:30-74.
+ * `residual` (optional) fuses the residual add in front of the norm (TransformerBlock.forward,
+ * model.py:293-294, adds and then normalises); `sum_out` (optional, needs residual) receives h;
+ * `rstd_out` (optional, fp32 n_rows) receives 1/rms as the Triton kernel caches it (:68).
+ * Row strides in elements; weight is bf16 (MI355_BF16) or fp32 (MI355_FP32), n_cols long.
+ */
+int mi355_rms_norm_fwd(const void* x, const void* residual, const void* weight, void* y, void* sum_out,
+                       float* rstd_out, int64_t n_rows, int n_cols, int64_t x_row_stride,
+                       int64_t residual_row_stride, int64_t y_row_stride, int64_t sum_row_stride, float eps,
+                       int weight_dtype, void* stream);
+
+/*
+ * out = bf16(silu(gate)) * up over (n_rows, n_cols) bf16 matrices with row strides (elements):
+ * silu in fp32, rounded to bf16, product rounded to bf16 -- _silu_mul_fwd_kernel,
+ * llm-systems/llm_systems/kernels/triton_swiglu.py:27-47 (and SwiGLU.forward, model.py:304-305).
+ * Strided rows let gate and up be the two halves of one merged projection output
+ * (FusedSwiGLU.forward, triton_swiglu.py:190-194) without the copies made there.
+ */
+int mi355_silu_mul_fwd(const void* gate, const void* up, void* out, int64_t n_rows, int n_cols,
+                       int64_t gate_row_stride, int64_t up_row_stride, int64_t out_row_stride, void* stream);
 
 /*
  * Plain device-to-device copy of `bytes` bytes (16-byte aligned).  Measurement aid

@@ -9,13 +9,17 @@ llm-core/llm_core/model.py:308-325 and the SDPA slot at model.py:382):
     paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, ...)
     rope_and_cache(q, k, v, positions, freq_cache, k_cache, v_cache, slot_mapping)   # cache producer
     quantize_kv_cache_fp8(cache)
+    rms_norm(x, weight, eps, residual=None)             # RMSNorm.forward / TritonRMSNorm forward
+    silu_mul(gate, up)                                  # fused kernel of FusedSwiGLU
 
 Every function runs on the HIP library; there is no CPU or PyTorch fallback.
 """
 from .ops import (  # noqa: F401
     build_rope_cache,
     quantize_kv_cache_fp8,
+    rms_norm,
     rope_and_cache,
+    silu_mul,
     flash_attn_prefill,
     flash_attn_varlen_prefill,
     paged_attention_decode,
@@ -24,4 +28,5 @@ from .ops import (  # noqa: F401
     sdpa_slot,
 )
 from .engine import BlockAllocator, OutOfBlocks, PagedAttentionEngine  # noqa: F401
+from .model import CachedTransformerLM  # noqa: F401
 from ._lib import LIB_PATH, LibraryMissing, load  # noqa: F401

@@ -9,6 +9,7 @@ LIB_PATH = os.path.join(_HERE, "libmi355attn.so")
 
 MI355_BF16 = 0
 MI355_FP8_E4M3 = 1
+MI355_FP32 = 2
 MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2
 
 _i64x3 = C.c_int64 * 3
@@ -21,6 +22,8 @@ EXPORTS = (
     "mi355_paged_decode_chunk_tokens",
     "mi355_rope_and_cache",
     "mi355_quantize_kv_fp8",
+    "mi355_rms_norm_fwd",
+    "mi355_silu_mul_fwd",
     "mi355_calib_copy",
     "mi355_last_error",
     "mi355_version",
@@ -57,6 +60,10 @@ def load():
                                          i64, i64, i64, i64, vp]
     lib.mi355_quantize_kv_fp8.restype = i32
     lib.mi355_quantize_kv_fp8.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
+    lib.mi355_rms_norm_fwd.restype = i32
+    lib.mi355_rms_norm_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i64, i32, i64, i64, i64, i64, f32, i32, vp]
+    lib.mi355_silu_mul_fwd.restype = i32
+    lib.mi355_silu_mul_fwd.argtypes = [vp, vp, vp, i64, i32, i64, i64, i64, vp]
     lib.mi355_calib_copy.restype = i32
     lib.mi355_calib_copy.argtypes = [vp, vp, sz, vp]
     lib.mi355_last_error.restype = C.c_char_p

@@ -4,13 +4,18 @@ What a KV-cached replacement of TransformerLM.generate (llm-core/llm_core/model.
 which re-runs the whole forward per token at :218) needs around the attention kernels: a block
 allocator, per-sequence block tables, slot mapping for cache writes, a prefill call for newly
 admitted sequences and a decode call that serves every running sequence with one kernel launch
-per step.  One engine instance serves ONE attention layer (its own K/V pools); a model keeps one
-per layer.  Projections, sampling and the scheduler policy stay with the caller.
+per layer and step.  The bookkeeping (blocks, lengths, tables) is shared by all attention layers
+of a model; every layer has its own K/V pools.  A step is planned once (`plan_prefill`,
+`plan_decode`: host integers -> a few small device tensors) and then applied per layer
+(`attend_prefill`, `attend_decode`).  Projections, sampling and the scheduler policy stay with
+the caller.
 
 All tensor work runs on the HIP kernels (rope_and_cache, flash_attn_varlen_prefill,
 paged_attention_decode); the bookkeeping here is plain Python on host integers.
 """
 from __future__ import annotations
+
+from dataclasses import dataclass
 
 import torch
 
@@ -43,14 +48,34 @@ class BlockAllocator:
         self._free.extend(blocks)
 
 
+@dataclass
+class PrefillPlan:
+    positions: torch.Tensor      # (T,) int32
+    slots: torch.Tensor          # (T,) int64
+    cu_seqlens: torch.Tensor     # (B+1,) int32
+    max_len: int
+    last_rows: torch.Tensor      # (B,) int64: packed row of each sequence's last token
+
+
+@dataclass
+class DecodePlan:
+    positions: torch.Tensor      # (B,) int32
+    slots: torch.Tensor          # (B,) int64
+    tables: torch.Tensor         # (B, max_blocks) int32
+    context_lens: torch.Tensor   # (B,) int32, the new token included
+    max_context: int
+
+
 class PagedAttentionEngine:
     def __init__(self, num_blocks, n_q_heads, n_kv_heads, head_dim, context_length, *, rope_theta=10000.0,
-                 max_batch=256, device="cuda:0"):
+                 max_batch=256, num_layers=1, device="cuda:0"):
         self.device = torch.device(device)
         self.Hq, self.Hkv, self.D = n_q_heads, n_kv_heads, head_dim
         self.context_length = context_length
-        self.k_cache = torch.zeros(num_blocks, n_kv_heads, BLOCK, head_dim, dtype=torch.bfloat16, device=self.device)
-        self.v_cache = torch.zeros_like(self.k_cache)
+        self.num_layers = num_layers
+        self.k_caches = [torch.zeros(num_blocks, n_kv_heads, BLOCK, head_dim, dtype=torch.bfloat16, device=self.device)
+                         for _ in range(num_layers)]
+        self.v_caches = [torch.zeros_like(k) for k in self.k_caches]
         self.freq_cache = ops.build_rope_cache(context_length, head_dim, rope_theta, self.device)
         self.allocator = BlockAllocator(num_blocks)
         self.blocks: dict[int, list[int]] = {}      # sequence id -> physical blocks
@@ -60,6 +85,15 @@ class PagedAttentionEngine:
         self._tables = torch.zeros(max_batch, self.max_blocks_per_seq, dtype=torch.int32, device=self.device)
         self._workspace = ops.paged_decode_workspace(max_batch, n_q_heads, head_dim, context_length, self.device)
         self.max_batch = max_batch
+
+    # the pools of layer 0 under their single-layer names
+    @property
+    def k_cache(self):
+        return self.k_caches[0]
+
+    @property
+    def v_cache(self):
+        return self.v_caches[0]
 
     # ---- bookkeeping ---------------------------------------------------------
     def add_sequence(self, seq_id: int) -> None:
@@ -87,35 +121,45 @@ class PagedAttentionEngine:
         self.lengths[seq_id] = length + n_new
         return slots
 
-    # ---- attention calls --------------------------------------------------------
-    def prefill(self, seq_ids, lens, q, k, v):
-        """Prompts of `seq_ids` (new, empty sequences) with `lens` tokens each, packed along dim 0.
-        Writes rotated K and V into the cache and returns causal attention output (T,Hq,D)."""
-        if sum(lens) != q.shape[0]:
-            raise ValueError("sum(lens) must equal the number of packed tokens")
-        slots, positions, cu = [], [], [0]
+    # ---- planning (once per step) ---------------------------------------------
+    def plan_prefill(self, seq_ids, lens) -> PrefillPlan:
+        """Reserves cache slots for the prompts of `seq_ids` (new, empty sequences) with `lens` tokens each."""
+        if len(seq_ids) != len(lens) or not seq_ids:
+            raise ValueError("seq_ids and lens must be non-empty and of equal length")
         for sid, n in zip(seq_ids, lens):
+            if n < 1 or n > self.context_length:
+                raise ValueError(f"prompt lengths must be in 1..{self.context_length}")
             if self.lengths[sid] != 0:
                 raise ValueError(f"sequence {sid} already has tokens; chunked prefill is not supported")
+        need = sum((n + BLOCK - 1) // BLOCK for n in lens)
+        if need > self.allocator.num_free:
+            raise OutOfBlocks(f"prefill needs {need} blocks, {self.allocator.num_free} free")
+        slots, positions, cu = [], [], [0]
+        for sid, n in zip(seq_ids, lens):
             slots += self._reserve(sid, n)
             positions += list(range(n))
             cu.append(cu[-1] + n)
         dev = self.device
-        pos = torch.tensor(positions, dtype=torch.int32, device=dev)
-        slot_t = torch.tensor(slots, dtype=torch.int64, device=dev)
-        cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
-        q_rot = ops.rope_and_cache(q, k, v, pos, self.freq_cache, self.k_cache, self.v_cache, slot_t)
-        k_rot = ops.rope_and_cache(k, k, v, pos, self.freq_cache)            # rotated keys, packed, for the prefill kernel
-        return ops.flash_attn_varlen_prefill(q_rot, k_rot, v, cu_t, cu_t, max(lens), max(lens), causal=True)
+        return PrefillPlan(torch.tensor(positions, dtype=torch.int32, device=dev),
+                           torch.tensor(slots, dtype=torch.int64, device=dev),
+                           torch.tensor(cu, dtype=torch.int32, device=dev), max(lens),
+                           torch.tensor([c - 1 for c in cu[1:]], dtype=torch.int64, device=dev))
 
-    def decode_step(self, seq_ids, q, k, v):
-        """One new token for each running sequence in `seq_ids`: q (B,Hq,D), k/v (B,Hkv,D) bf16.
-        Appends the token's K/V to the cache and returns its attention output (B,Hq,D)."""
+    def plan_decode(self, seq_ids) -> DecodePlan:
+        """Reserves the slot of one new token for each running sequence in `seq_ids`."""
         B = len(seq_ids)
-        if B > self.max_batch:
-            raise ValueError(f"batch {B} exceeds max_batch {self.max_batch}")
-        if q.shape[0] != B:
-            raise ValueError("one query token per sequence expected")
+        if B == 0 or B > self.max_batch:
+            raise ValueError(f"batch {B} must be in 1..{self.max_batch}")
+        if len(set(seq_ids)) != B:
+            raise ValueError("a sequence may appear only once per decode step")
+        for s in seq_ids:
+            if self.lengths[s] == 0:
+                raise ValueError(f"sequence {s} has no tokens; prefill it first")
+            if self.lengths[s] + 1 > self.context_length:
+                raise ValueError(f"sequence {s} would exceed context_length {self.context_length}")
+        need = sum(1 for s in seq_ids if self.lengths[s] % BLOCK == 0)
+        if need > self.allocator.num_free:
+            raise OutOfBlocks(f"decode step needs {need} blocks, {self.allocator.num_free} free")
         positions = [self.lengths[s] for s in seq_ids]
         slots = [self._reserve(s, 1)[0] for s in seq_ids]
         dev = self.device
@@ -127,9 +171,41 @@ class PagedAttentionEngine:
             rows[i, :len(b)] = torch.tensor(b, dtype=torch.int32)
         tables = self._tables[:B, :max_blk]
         tables.copy_(rows, non_blocking=False)
-        ctx = torch.tensor([self.lengths[s] for s in seq_ids], dtype=torch.int32, device=dev)
-        pos = torch.tensor(positions, dtype=torch.int32, device=dev)
-        slot_t = torch.tensor(slots, dtype=torch.int64, device=dev)
-        q_rot = ops.rope_and_cache(q, k, v, pos, self.freq_cache, self.k_cache, self.v_cache, slot_t)
-        return ops.paged_attention_decode(q_rot, self.k_cache, self.v_cache, tables, ctx,
-                                          max_context=max_blk * BLOCK, workspace=self._workspace)
+        return DecodePlan(torch.tensor(positions, dtype=torch.int32, device=dev),
+                          torch.tensor(slots, dtype=torch.int64, device=dev), tables,
+                          torch.tensor([p + 1 for p in positions], dtype=torch.int32, device=dev), max_blk * BLOCK)
+
+    # ---- attention calls (once per layer) -----------------------------------------
+    def attend_prefill(self, layer: int, plan: PrefillPlan, q, k, v):
+        """q (T,Hq,D), k/v (T,Hkv,D) packed along dim 0 (token strides free, heads contiguous).  Writes
+        rotated K and V of layer `layer` into its cache and returns causal attention output (T,Hq,D)."""
+        if q.shape[0] != plan.positions.shape[0]:
+            raise ValueError("the plan and the packed tensors disagree on the number of tokens")
+        kc, vc = self.k_caches[layer], self.v_caches[layer]
+        q_rot = ops.rope_and_cache(q, k, v, plan.positions, self.freq_cache, kc, vc, plan.slots)
+        k_rot = ops.rope_and_cache(k, k, v, plan.positions, self.freq_cache)   # rotated keys, packed, for the prefill kernel
+        return ops.flash_attn_varlen_prefill(q_rot, k_rot, v, plan.cu_seqlens, plan.cu_seqlens, plan.max_len,
+                                             plan.max_len, causal=True)
+
+    def attend_decode(self, layer: int, plan: DecodePlan, q, k, v):
+        """q (B,Hq,D), k/v (B,Hkv,D): appends the token's K/V to layer `layer`'s cache and returns its
+        attention output (B,Hq,D)."""
+        if q.shape[0] != plan.positions.shape[0]:
+            raise ValueError("one query token per sequence expected")
+        kc, vc = self.k_caches[layer], self.v_caches[layer]
+        q_rot = ops.rope_and_cache(q, k, v, plan.positions, self.freq_cache, kc, vc, plan.slots)
+        return ops.paged_attention_decode(q_rot, kc, vc, plan.tables, plan.context_lens,
+                                          max_context=plan.max_context, workspace=self._workspace)
+
+    # ---- single-layer convenience ----------------------------------------------------
+    def prefill(self, seq_ids, lens, q, k, v):
+        """plan_prefill + attend_prefill on layer 0."""
+        if sum(lens) != q.shape[0]:
+            raise ValueError("sum(lens) must equal the number of packed tokens")
+        return self.attend_prefill(0, self.plan_prefill(seq_ids, lens), q, k, v)
+
+    def decode_step(self, seq_ids, q, k, v):
+        """plan_decode + attend_decode on layer 0."""
+        if q.shape[0] != len(seq_ids):
+            raise ValueError("one query token per sequence expected")
+        return self.attend_decode(0, self.plan_decode(seq_ids), q, k, v)

@@ -304,3 +304,71 @@ def quantize_kv_cache_fp8(cache, *, out=None):
                                            _stream())
     _lib.check(rc, "mi355_quantize_kv_fp8")
     return out, scale
+
+
+def _rows2d(name, t):
+    """(…, n_cols) bf16 GPU tensor -> (n_rows, n_cols) view with a unit column stride (copy only if needed)."""
+    _require_gpu_bf16(name, t)
+    if t.dim() < 1:
+        raise ValueError(f"{name} must have at least one dimension")
+    t2 = t.reshape(-1, t.shape[-1])           # a view whenever the leading dims can be merged
+    if t2.stride(1) != 1 and t2.shape[1] > 1:
+        t2 = t2.contiguous()
+    return t2
+
+
+def rms_norm(x, weight, eps: float = 1e-5, *, residual=None, return_sum: bool = False, return_rstd: bool = False):
+    """RMSNorm forward over the last dimension: weight * (h * rsqrt(mean(h^2) + eps)), fp32 math, bf16 in/out --
+    RMSNorm.forward (llm-core/llm_core/model.py:60-67) and TritonRMSNorm's forward kernel
+    (llm-systems/llm_systems/kernels/triton_rms_norm.py:30-74).
+
+    x (..., d) bf16; weight (d,) bf16 or fp32.  With `residual` (same shape as x) the normalised
+    tensor is h = bf16(x + residual), the add in front of each norm of TransformerBlock.forward
+    (model.py:293-294); return_sum=True also returns h.  return_rstd=True also returns 1/rms
+    (fp32, x.shape[:-1]) as the Triton kernel caches it.  Returns y, or (y, [h], [rstd]).
+    """
+    x2 = _rows2d("x", x)
+    n_rows, d = x2.shape
+    if weight.shape != (d,) or not weight.is_cuda or not weight.is_contiguous():
+        raise ValueError(f"weight must be a contiguous GPU tensor of shape ({d},)")
+    if weight.dtype == torch.bfloat16:
+        wcode = _lib.MI355_BF16
+    elif weight.dtype == torch.float32:
+        wcode = _lib.MI355_FP32
+    else:
+        raise TypeError(f"weight must be bfloat16 or float32 (got {weight.dtype})")
+    r2 = None
+    if residual is not None:
+        if residual.shape != x.shape:
+            raise ValueError("residual must have x's shape")
+        r2 = _rows2d("residual", residual)
+    elif return_sum:
+        raise ValueError("return_sum needs residual")
+    y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    h = torch.empty(x.shape, dtype=x.dtype, device=x.device) if return_sum else None
+    rstd = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device) if return_rstd else None
+    if n_rows:
+        rc = _lib.load().mi355_rms_norm_fwd(
+            x2.data_ptr(), None if r2 is None else r2.data_ptr(), weight.data_ptr(), y.data_ptr(),
+            None if h is None else h.data_ptr(), None if rstd is None else rstd.data_ptr(),
+            n_rows, d, x2.stride(0), 0 if r2 is None else r2.stride(0), d, d, float(eps), wcode, _stream())
+        _lib.check(rc, "mi355_rms_norm_fwd")
+    extra = [t for t in (h, rstd) if t is not None]
+    return (y, *extra) if extra else y
+
+
+def silu_mul(gate, up):
+    """bf16(silu(gate)) * up, silu in fp32 -- the fused kernel of FusedSwiGLU
+    (llm-systems/llm_systems/kernels/triton_swiglu.py:27-47; SwiGLU.forward, model.py:304-305).
+    gate and up (..., d_ff) bf16 may be strided row views, e.g. the two halves of a merged
+    gate/up projection output (triton_swiglu.py:190-191): nothing is copied."""
+    if gate.shape != up.shape:
+        raise ValueError(f"shape mismatch: gate {tuple(gate.shape)} up {tuple(up.shape)}")
+    g2, u2 = _rows2d("gate", gate), _rows2d("up", up)
+    out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    n_rows, d = g2.shape
+    if n_rows and d:
+        rc = _lib.load().mi355_silu_mul_fwd(g2.data_ptr(), u2.data_ptr(), out.data_ptr(), n_rows, d,
+                                            g2.stride(0), u2.stride(0), d, _stream())
+        _lib.check(rc, "mi355_silu_mul_fwd")
+    return out
