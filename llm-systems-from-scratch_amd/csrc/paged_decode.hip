@@ -82,10 +82,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
     // 1-D grid, kv head fastest, then sequence, chunk slowest.  Workgroup ids are dealt
     // round-robin to the 8 XCDs, so the low bits of the id must not select the chunk:
     // with ragged lengths late chunks are mostly empty and the XCDs that own them would idle.
+    // Chunks are dealt in DESCENDING order: the full chunks of the long sequences start first
+    // and the first chunks of the short sequences (the smallest work items) form the tail.
     const int wg = blockIdx.x;
     const int hk = wg % p.Hkv;
     const int b = (wg / p.Hkv) % p.B;
-    const int chunk = wg / (p.Hkv * p.B);
+    const int chunk = p.max_chunks - 1 - wg / (p.Hkv * p.B);
     const int ctx = min(p.context_lens[b], p.max_ctx);     // a length beyond the promised bound is truncated, never chased
     const int chunk_tokens = kDecodeWaves * p.tokens_per_wave;
     const int chunk_start = chunk * chunk_tokens;
