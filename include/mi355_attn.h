@@ -74,6 +74,46 @@ int mi355_prefill_fwd(const void* q, const void* k, const void* v, void* out,
                       float softmax_scale, int mask_mode, int dtype, void* stream);
 
 /*
+ * Prefill forward that also returns the log-sum-exp of every query row, which the backward
+ * needs: lse[b,h,i] = log sum_j exp(softmax_scale * q_i.k_j) over the kept keys (natural log,
+ * fp32; -inf for a row with no kept key).  lse is addressed as
+ *   dense : lse + b*lse_strides[0] + h*lse_strides[1] + i
+ *   packed: lse + h*lse_strides[1] + t            (t = row in the packed query buffer)
+ * Same computation and arguments as mi355_prefill_fwd otherwise (mask modes NONE / CAUSAL).
+ * This is the forward half of what torch.nn.functional.scaled_dot_product_attention does under
+ * autograd at llm-core/llm_core/model.py:382 when train.py runs with --flash-attn (train.py:312).
+ */
+int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out, float* lse,
+                          const int64_t q_strides[3], const int64_t k_strides[3],
+                          const int64_t v_strides[3], const int64_t o_strides[3],
+                          const int64_t lse_strides[2],
+                          const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                          int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
+                          float softmax_scale, int mask_mode, int dtype, void* stream);
+
+/*
+ * Prefill backward: dq, dk, dv of out = softmax(q k^T * softmax_scale [causal]) v given dout,
+ * i.e. the gradient that autograd derives for the attention call at model.py:380-385
+ * (model.py:308-325 is its definition) during loss.backward() (train.py:224).
+ *   q, k, v, out, dout, dq, dk, dv : bf16, layouts and stride conventions of mi355_prefill_fwd
+ *                                    (dq like q, dk/dv like k/v, dout like out), each with its own strides
+ *   lse   : as written by mi355_prefill_fwd_lse for the same inputs
+ *   delta : fp32 scratch with lse's layout and size (receives rowsum(dout * out))
+ *   total_q : rows of the packed query buffer (packed layout only; ignored for dense)
+ * GQA: dk/dv of a kv head sum over its Hq/Hkv query heads.  Mask modes NONE / CAUSAL.
+ * A causal query row that sees no key (Sq > Sk) gets dq = 0.  Three launches on `stream`
+ * (delta, dk/dv, dq); no atomics, so the result is deterministic.
+ */
+int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                      const float* lse, float* delta, void* dq, void* dk, void* dv,
+                      const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                      const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
+                      const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[2],
+                      const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t total_q,
+                      int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
+                      float softmax_scale, int mask_mode, int dtype, void* stream);
+
+/*
  * Paged-KV decode attention, one query token per sequence (split-K + combine).
  *
  * No counterpart exists in the reference: it is what a KV-cached replacement of

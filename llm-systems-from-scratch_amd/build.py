@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "mi355_attn")
 LIB_NAME = "libmi355attn.so"
-SOURCES = ["api.hip", "paged_decode.hip", "prefill_fwd.hip", "kv_cache_ops.hip", "layer_ops.hip"]
+SOURCES = ["api.hip", "paged_decode.hip", "prefill_fwd.hip", "prefill_bwd.hip", "kv_cache_ops.hip", "layer_ops.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -1,0 +1,567 @@
+// FlashAttention-style prefill backward for gfx950 (bf16, MFMA 32x32x16): dQ, dK, dV from
+// q, k, v, out, dout and the forward's log-sum-exp.  No atomics; results are deterministic.
+//
+//   delta_i = sum_d dO[i,d] * O[i,d]                       (bwd_delta_kernel)
+//   P_ij    = exp(scale * q_i.k_j - lse_i)                 (recomputed, never stored)
+//   dV_j    = sum_i P_ij dO_i
+//   dP_ij   = dO_i . v_j
+//   dS_ij   = P_ij (dP_ij - delta_i)
+//   dQ_i    = scale * sum_j dS_ij k_j                      (bwd_dq_kernel: one workgroup per query tile)
+//   dK_j    = scale * sum_i dS_ij q_i                      (bwd_dkv_kernel: one workgroup per key tile,
+//                                                           summing over the query heads of a GQA group)
+//
+// Both main kernels work on transposed problems, like the forward: the wavefront owns 32
+// columns (queries in the dQ kernel, keys in the dK/dV kernel) whose operand fragments stay in
+// registers; the other side streams through LDS tiles of 64 rows.  The accumulator of the first
+// MFMA pair (S and dP, column = lane) is, converted to bf16, directly the B operand of the
+// second (dQ^T += K^T dS^T; dV^T += dO^T P, dK^T += Q^T dS), and the matching A operand is a
+// transposed LDS read (ds_read_b64_tr_b16) of the streamed tile with the same row permutation.
+#include "common.hpp"
+#include "launch.hpp"
+#include "prefill_tile.hpp"
+
+namespace mi355 {
+
+constexpr int kBwWaves = 4;
+constexpr int kBwCols = 32 * kBwWaves;   // columns (queries or keys) per workgroup
+constexpr int kBwRows = 64;              // rows of a streamed LDS tile
+
+struct BwdParams {
+    const __bf16* q;
+    const __bf16* k;
+    const __bf16* v;
+    const __bf16* out;
+    const __bf16* dout;
+    const float* lse;
+    float* delta;
+    __bf16* dq;
+    __bf16* dk;
+    __bf16* dv;
+    int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];   // batch, head, row strides (elements)
+    int64_t ls[2];                                                          // lse / delta: batch, head strides
+    const int32_t* cu_q;
+    const int32_t* cu_k;
+    int B, Hq, Hkv, Sq, Sk;
+    float scale, scale_log2;
+    int n_qtiles, n_ktiles;
+};
+
+// Loader of a 64-row tile (rows of D bf16, row stride `stride` elements) into swizzled LDS:
+// wavefront w, instruction j covers LDS chunks (w*NI + j)*64 .. +63; rows past `last` re-read row `last`.
+template <int D>
+struct TileLoader {
+    static constexpr int CPR = D / 8;
+    static constexpr int NI = kBwRows * CPR / 64 / kBwWaves;
+    int row[NI], col[NI];
+    __device__ __forceinline__ void init(int wave, int lane) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int idx = (wave * NI + j) * 64 + lane;
+            row[j] = idx / CPR;
+            col[j] = ((idx % CPR) ^ swz<D>(idx / CPR)) * 16;
+        }
+    }
+    __device__ __forceinline__ void issue(const __bf16* first_row, int stride, int last, uint32_t lds_wave_base) const {
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+            dma_to_lds_16(first_row, (uint32_t)(min(row[j], last) * stride * 2 + col[j]), lds_wave_base + j * 1024);
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// delta = rowsum(dO * O): 16 lanes per (row, head), 8 elements per lane and step.
+template <int D>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(BwdParams p, int64_t total_rows) {
+    const int sub = threadIdx.x & 15;
+    const int64_t item = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;      // (b, h, i) flattened, i fastest
+    if (item >= total_rows * p.Hq) return;
+    const int h = (int)((item / total_rows) % p.Hq);
+    const int64_t r = item % total_rows;                                     // row inside the batch element / packed buffer
+    int64_t o_off, do_off, l_off;
+    if (p.cu_q) {
+        o_off = r * p.os[2] + (int64_t)h * p.os[1];
+        do_off = r * p.dos[2] + (int64_t)h * p.dos[1];
+        l_off = r + (int64_t)h * p.ls[1];
+    } else {
+        const int64_t b = r / p.Sq, i = r % p.Sq;
+        o_off = b * p.os[0] + (int64_t)h * p.os[1] + i * p.os[2];
+        do_off = b * p.dos[0] + (int64_t)h * p.dos[1] + i * p.dos[2];
+        l_off = b * p.ls[0] + (int64_t)h * p.ls[1] + i;
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int c = sub; c < D / 8; c += 16) {
+        const bf16x8 a = as_bf16x8(*reinterpret_cast<const u32x4*>(p.out + o_off + 8 * c));
+        const bf16x8 g = as_bf16x8(*reinterpret_cast<const u32x4*>(p.dout + do_off + 8 * c));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)g[e];
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (sub == 0) p.delta[l_off] = acc;
+}
+
+// Per-lane LDS offsets of the two read patterns of a swizzled 64 x D tile.
+template <int D>
+struct TileReads {
+    static constexpr int NS = D / 16, NDT = D / 32, kRow = D * 2;
+    int row_off[NS];        // A fragment "row n of the tile, k = 16s + 8kg ..": add 32*t*kRow
+    int tr_off[2][NDT];     // transposed fragment of d-tile dt for a 16-row slice: add 16*u*kRow
+    __device__ __forceinline__ void init(int lane) {
+        const int n = lane & 31, kg = lane >> 5;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) row_off[s] = n * kRow + (((2 * s + kg) ^ swz<D>(n)) << 4);
+        const int g16 = lane >> 4, s16 = lane & 15;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int row = 4 * (g16 >> 1) + (s16 >> 2) + 8 * e;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const int d = 32 * dt + 16 * (g16 & 1) + 4 * (s16 & 3);
+                tr_off[e][dt] = row * kRow + (((d >> 3) ^ swz<D>(row)) << 4) + (d & 7) * 2;
+            }
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// dQ: one workgroup per tile of 128 queries of one (batch, query head); K/V stream through LDS.
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
+    using R = TileReads<D>;
+    constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[kTile];
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[kTile];
+
+    const int lid = blockIdx.x;
+    const int qtile = p.n_qtiles - 1 - lid % p.n_qtiles;          // heavy (late) causal tiles first
+    const int h = (lid / p.n_qtiles) % p.Hq;
+    const int b = lid / (p.n_qtiles * p.Hq);
+    const int hk = h / (p.Hq / p.Hkv);
+    int sq, sk;
+    int64_t q_base, k_base, v_base, do_base, dq_base, l_base;
+    if (p.cu_q) {
+        const int q_start = p.cu_q[b], k_start = p.cu_k[b];
+        sq = p.cu_q[b + 1] - q_start;
+        sk = p.cu_k[b + 1] - k_start;
+        q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
+        do_base = (int64_t)q_start * p.dos[2] + (int64_t)h * p.dos[1];
+        dq_base = (int64_t)q_start * p.dqs[2] + (int64_t)h * p.dqs[1];
+        k_base = (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
+        v_base = (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
+        l_base = q_start + (int64_t)h * p.ls[1];
+    } else {
+        sq = p.Sq;
+        sk = p.Sk;
+        q_base = (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
+        do_base = (int64_t)b * p.dos[0] + (int64_t)h * p.dos[1];
+        dq_base = (int64_t)b * p.dqs[0] + (int64_t)h * p.dqs[1];
+        k_base = (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
+        v_base = (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
+        l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
+    }
+    const int q0 = qtile * kBwCols;
+    if (q0 >= sq) return;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, kg = lane >> 5;
+    const int qi = q0 + 32 * wave + n;
+    const bool q_ok = qi < sq;
+    const int coff = sk - sq;
+
+    TileLoader<D> ld;
+    ld.init(wave, lane);
+    R rd;
+    rd.init(lane);
+    const uint32_t k_dst = __builtin_amdgcn_readfirstlane(lds_address(k_lds) + wave * TileLoader<D>::NI * 1024);
+    const uint32_t v_dst = __builtin_amdgcn_readfirstlane(lds_address(v_lds) + wave * TileLoader<D>::NI * 1024);
+
+    // fragments of this lane's query column: step s covers d = 16s + 8kg + j
+    bf16x8 qf[NS], dof[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        u32x4 a = {0u, 0u, 0u, 0u}, g = {0u, 0u, 0u, 0u};
+        if (q_ok) {
+            a = *reinterpret_cast<const u32x4*>(p.q + q_base + (int64_t)qi * p.qs[2] + 16 * s + 8 * kg);
+            g = *reinterpret_cast<const u32x4*>(p.dout + do_base + (int64_t)qi * p.dos[2] + 16 * s + 8 * kg);
+        }
+        qf[s] = as_bf16x8(a);
+        dof[s] = as_bf16x8(g);
+    }
+    // a padded query column gets lse = +inf, i.e. P = 0 everywhere
+    const float lse2 = q_ok ? p.lse[l_base + qi] * kLog2e : INFINITY;
+    const float delta = q_ok ? p.delta[l_base + qi] : 0.f;
+
+    f32x16 dq[NDT];
+#pragma unroll
+    for (int i = 0; i < NDT; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) dq[i][j] = 0.f;
+
+    int kv_end = sk;
+    if (CAUSAL) kv_end = max(0, min(sk, min(sq, q0 + kBwCols) + coff));
+    const int n_tiles = (kv_end + kBwRows - 1) / kBwRows;
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const int k0 = tile * kBwRows;
+        __syncthreads();                                   // everybody is done reading the previous tile
+        ld.issue(p.k + k_base + (int64_t)k0 * p.ks[2], (int)p.ks[2], sk - 1 - k0, k_dst);
+        ld.issue(p.v + v_base + (int64_t)k0 * p.vs[2], (int)p.vs[2], sk - 1 - k0, v_dst);
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (CAUSAL && k0 > q0 + 32 * wave + 31 + coff) continue;   // wholly above this wavefront's diagonal (uniform)
+
+        f32x16 s_acc[2], dp_acc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                s_acc[t][j] = 0.f;
+                dp_acc[t][j] = 0.f;
+            }
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const u32x4 kf = *reinterpret_cast<const u32x4*>(k_lds + t * 32 * kRow + rd.row_off[s]);
+                s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s_acc[t]);
+            }
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const u32x4 vf = *reinterpret_cast<const u32x4*>(v_lds + t * 32 * kRow + rd.row_off[s]);
+                dp_acc[t] = mfma32(as_bf16x8(vf), dof[s], dp_acc[t]);
+            }
+        }
+        // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = k0 + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3);
+                bool keep = key < sk;
+                if (CAUSAL) keep = keep & (key <= qi + coff);
+                const float pr = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -lse2));
+                s_acc[t][i] = keep ? pr * (dp_acc[t][i] - delta) : 0.f;        // dS (without the scale factor)
+            }
+        // dQ^T (D x 32 queries) += K^T . dS^T, 16 keys at a time
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int t = u >> 1, e0 = 8 * (u & 1);
+            u32x4 pw;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
+            const bf16x8 pf = as_bf16x8(pw);
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const i16x4 lo = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[0][dt]);
+                const i16x4 hi = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[1][dt]);
+                dq[dt] = mfma32(join_bf16x8(lo, hi), pf, dq[dt]);
+            }
+        }
+    }
+
+    // store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4
+    if (q_ok) {
+        __bf16* row = p.dq + dq_base + (int64_t)qi * p.dqs[2];
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                u32x2 w;
+                w[0] = pack_bf16(dq[dt][4 * g + 0] * p.scale, dq[dt][4 * g + 1] * p.scale);
+                w[1] = pack_bf16(dq[dt][4 * g + 2] * p.scale, dq[dt][4 * g + 3] * p.scale);
+                *reinterpret_cast<u32x2*>(row + 32 * dt + 8 * g + 4 * kg) = w;
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dK, dV: one workgroup per tile of 128 keys of one (batch, kv head); Q/dO of every query head of
+// the GQA group stream through LDS together with their lse and delta.
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dkv_kernel(BwdParams p) {
+    using R = TileReads<D>;
+    constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
+    __shared__ __attribute__((aligned(1024))) unsigned char q_lds[kTile];
+    __shared__ __attribute__((aligned(1024))) unsigned char do_lds[kTile];
+    __shared__ __attribute__((aligned(16))) float lse_lds[kBwRows];
+    __shared__ __attribute__((aligned(16))) float delta_lds[kBwRows];
+
+    const int lid = blockIdx.x;
+    const int ktile = lid % p.n_ktiles;                            // causal: early key tiles carry the most work
+    const int hk = (lid / p.n_ktiles) % p.Hkv;
+    const int b = lid / (p.n_ktiles * p.Hkv);
+    const int G = p.Hq / p.Hkv;
+    int sq, sk, q_start = 0;
+    int64_t k_base, v_base, dk_base, dv_base;
+    if (p.cu_q) {
+        q_start = p.cu_q[b];
+        const int k_start = p.cu_k[b];
+        sq = p.cu_q[b + 1] - q_start;
+        sk = p.cu_k[b + 1] - k_start;
+        k_base = (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
+        v_base = (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
+        dk_base = (int64_t)k_start * p.dks[2] + (int64_t)hk * p.dks[1];
+        dv_base = (int64_t)k_start * p.dvs[2] + (int64_t)hk * p.dvs[1];
+    } else {
+        sq = p.Sq;
+        sk = p.Sk;
+        k_base = (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
+        v_base = (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
+        dk_base = (int64_t)b * p.dks[0] + (int64_t)hk * p.dks[1];
+        dv_base = (int64_t)b * p.dvs[0] + (int64_t)hk * p.dvs[1];
+    }
+    const int k0 = ktile * kBwCols;
+    if (k0 >= sk) return;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, kg = lane >> 5;
+    const int kj = k0 + 32 * wave + n;
+    const bool k_ok = kj < sk;
+    const int coff = sk - sq;
+
+    TileLoader<D> ld;
+    ld.init(wave, lane);
+    R rd;
+    rd.init(lane);
+    const uint32_t q_dst = __builtin_amdgcn_readfirstlane(lds_address(q_lds) + wave * TileLoader<D>::NI * 1024);
+    const uint32_t do_dst = __builtin_amdgcn_readfirstlane(lds_address(do_lds) + wave * TileLoader<D>::NI * 1024);
+
+    // fragments of this lane's key column: step s covers d = 16s + 8kg + j
+    bf16x8 kf[NS], vf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        u32x4 a = {0u, 0u, 0u, 0u}, g = {0u, 0u, 0u, 0u};
+        if (k_ok) {
+            a = *reinterpret_cast<const u32x4*>(p.k + k_base + (int64_t)kj * p.ks[2] + 16 * s + 8 * kg);
+            g = *reinterpret_cast<const u32x4*>(p.v + v_base + (int64_t)kj * p.vs[2] + 16 * s + 8 * kg);
+        }
+        kf[s] = as_bf16x8(a);
+        vf[s] = as_bf16x8(g);
+    }
+    f32x16 dk[NDT], dv[NDT];
+#pragma unroll
+    for (int i = 0; i < NDT; ++i)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            dk[i][j] = 0.f;
+            dv[i][j] = 0.f;
+        }
+
+    // causal: key kj is seen by queries i >= kj - coff; the first row tile that can see key k0
+    int first_tile = 0;
+    if (CAUSAL) first_tile = max(0, k0 - coff) / kBwRows;
+    const int n_tiles = (sq + kBwRows - 1) / kBwRows;
+
+    for (int g = 0; g < G; ++g) {
+        const int h = hk * G + g;
+        int64_t q_base, do_base, l_base;
+        if (p.cu_q) {
+            q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
+            do_base = (int64_t)q_start * p.dos[2] + (int64_t)h * p.dos[1];
+            l_base = q_start + (int64_t)h * p.ls[1];
+        } else {
+            q_base = (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
+            do_base = (int64_t)b * p.dos[0] + (int64_t)h * p.dos[1];
+            l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
+        }
+        for (int tile = first_tile; tile < n_tiles; ++tile) {
+            const int r0 = tile * kBwRows;
+            __syncthreads();                               // everybody is done reading the previous tile
+            ld.issue(p.q + q_base + (int64_t)r0 * p.qs[2], (int)p.qs[2], sq - 1 - r0, q_dst);
+            ld.issue(p.dout + do_base + (int64_t)r0 * p.dos[2], (int)p.dos[2], sq - 1 - r0, do_dst);
+            if (tid < kBwRows) {                           // a padded query row gets lse = +inf, i.e. P = 0
+                const bool ok = r0 + tid < sq;
+                lse_lds[tid] = ok ? p.lse[l_base + r0 + tid] * kLog2e : INFINITY;
+                delta_lds[tid] = ok ? p.delta[l_base + r0 + tid] : 0.f;
+            }
+            wait_vmcnt<0>();
+            __syncthreads();
+            // wholly above this wavefront's diagonal: its last key column is not seen by the tile's last row
+            if (CAUSAL && k0 + 32 * wave > r0 + kBwRows - 1 + coff) continue;
+
+            f32x16 s_acc[2], dp_acc[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    s_acc[t][j] = 0.f;
+                    dp_acc[t][j] = 0.f;
+                }
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    const u32x4 a = *reinterpret_cast<const u32x4*>(q_lds + t * 32 * kRow + rd.row_off[s]);
+                    s_acc[t] = mfma32(as_bf16x8(a), kf[s], s_acc[t]);
+                }
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    const u32x4 a = *reinterpret_cast<const u32x4*>(do_lds + t * 32 * kRow + rd.row_off[s]);
+                    dp_acc[t] = mfma32(as_bf16x8(a), vf[s], dp_acc[t]);
+                }
+            }
+            // element (t,i) of this lane: query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int rl = 32 * t + 8 * j + 4 * kg;                    // local row of element i = 4j
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_lds + rl);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_lds + rl);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int i = 4 * j + r;
+                        bool keep = true;
+                        if (CAUSAL) keep = kj <= r0 + rl + r + coff;
+                        const float pr = keep ? fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -l4[r])) : 0.f;
+                        s_acc[t][i] = pr;                                      // P
+                        dp_acc[t][i] = pr * (dp_acc[t][i] - d4[r]);            // dS (without the scale factor)
+                    }
+                }
+            // dV^T (D x 32 keys) += dO^T . P ;  dK^T += Q^T . dS, 16 query rows at a time
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int t = u >> 1, e0 = 8 * (u & 1);
+                u32x4 pw, sw;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
+                    sw[w] = pack_bf16(dp_acc[t][e0 + 2 * w], dp_acc[t][e0 + 2 * w + 1]);
+                }
+                const bf16x8 pf = as_bf16x8(pw), sf = as_bf16x8(sw);
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    const i16x4 lo = lds_read_tr16(do_lds + 16 * u * kRow + rd.tr_off[0][dt]);
+                    const i16x4 hi = lds_read_tr16(do_lds + 16 * u * kRow + rd.tr_off[1][dt]);
+                    dv[dt] = mfma32(join_bf16x8(lo, hi), pf, dv[dt]);
+                }
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    const i16x4 lo = lds_read_tr16(q_lds + 16 * u * kRow + rd.tr_off[0][dt]);
+                    const i16x4 hi = lds_read_tr16(q_lds + 16 * u * kRow + rd.tr_off[1][dt]);
+                    dk[dt] = mfma32(join_bf16x8(lo, hi), sf, dk[dt]);
+                }
+            }
+        }
+    }
+
+    // store: lane owns key kj, d = 32dt + 8(i/4) + 4kg + i%4
+    if (k_ok) {
+        __bf16* krow = p.dk + dk_base + (int64_t)kj * p.dks[2];
+        __bf16* vrow = p.dv + dv_base + (int64_t)kj * p.dvs[2];
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                u32x2 w;
+                w[0] = pack_bf16(dk[dt][4 * g + 0] * p.scale, dk[dt][4 * g + 1] * p.scale);
+                w[1] = pack_bf16(dk[dt][4 * g + 2] * p.scale, dk[dt][4 * g + 3] * p.scale);
+                *reinterpret_cast<u32x2*>(krow + 32 * dt + 8 * g + 4 * kg) = w;
+                w[0] = pack_bf16(dv[dt][4 * g + 0], dv[dt][4 * g + 1]);
+                w[1] = pack_bf16(dv[dt][4 * g + 2], dv[dt][4 * g + 3]);
+                *reinterpret_cast<u32x2*>(vrow + 32 * dt + 8 * g + 4 * kg) = w;
+            }
+    }
+}
+
+template <int D>
+static int launch_bwd(const BwdParams& p, bool causal, int64_t total_rows, hipStream_t stream) {
+    const int64_t delta_threads = total_rows * p.Hq * 16;
+    hipLaunchKernelGGL((bwd_delta_kernel<D>), dim3((unsigned)((delta_threads + 255) / 256)), dim3(256), 0, stream, p,
+                       total_rows);
+    const dim3 block(kBwWaves * 64);
+    const dim3 grid_q((unsigned)(p.n_qtiles * p.Hq * p.B)), grid_k((unsigned)(p.n_ktiles * p.Hkv * p.B));
+    if (causal) {
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, true>), grid_k, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dq_kernel<D, true>), grid_q, block, 0, stream, p);
+    } else {
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, false>), grid_k, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dq_kernel<D, false>), grid_q, block, 0, stream, p);
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                                 const float* lse, float* delta, void* dq, void* dk, void* dv,
+                                 const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                                 const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
+                                 const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[2],
+                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t total_q, int B, int Hq,
+                                 int Hkv, int Sq_max, int Sk_max, int D, float softmax_scale, int mask_mode, int dtype,
+                                 void* stream) {
+    if (!q || !k || !v || !out || !dout || !lse || !delta || !dq || !dk || !dv)
+        return set_error(MI355_EINVAL, "prefill_bwd: null pointer argument");
+    if (!q_strides || !k_strides || !v_strides || !o_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides ||
+        !lse_strides)
+        return set_error(MI355_EINVAL, "prefill_bwd: null stride argument");
+    if (dtype != MI355_BF16) return set_error(MI355_EDTYPE, "prefill_bwd: dtype must be MI355_BF16");
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Sq_max <= 0 || Sk_max <= 0)
+        return set_error(MI355_EINVAL, "prefill_bwd: B, Hq, Hkv, Sq_max and Sk_max must be positive");
+    if (Hq % Hkv != 0) return set_error(MI355_EINVAL, "prefill_bwd: Hq must be a multiple of Hkv");
+    if (!(D == 128 || D == 64 || D == 32)) return set_error(MI355_EINVAL, "prefill_bwd: head_dim must be 32, 64 or 128");
+    if ((cu_seqlens_q == nullptr) != (cu_seqlens_k == nullptr))
+        return set_error(MI355_EINVAL, "prefill_bwd: cu_seqlens_q and cu_seqlens_k must be given together");
+    if (mask_mode != MI355_MASK_NONE && mask_mode != MI355_MASK_CAUSAL)
+        return set_error(MI355_EINVAL, "prefill_bwd: mask_mode must be MI355_MASK_NONE or MI355_MASK_CAUSAL");
+    if (cu_seqlens_q && total_q <= 0) return set_error(MI355_EINVAL, "prefill_bwd: total_q must be positive (packed layout)");
+    const int64_t* all[8] = {q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides};
+    for (const int64_t* st : all)
+        for (int i = 0; i < 3; ++i)
+            if (st[i] & 7) return set_error(MI355_EINVAL, "prefill_bwd: strides must be multiples of 8 elements (16-byte rows)");
+    const int64_t* rows[4] = {q_strides, k_strides, v_strides, do_strides};
+    for (const int64_t* st : rows)
+        if (st[2] <= 0 || st[2] >= (1 << 24))
+            return set_error(MI355_EINVAL, "prefill_bwd: row strides must be positive and below 2^24 elements");
+    if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dq | (uintptr_t)dk |
+         (uintptr_t)dv) & 15)
+        return set_error(MI355_EINVAL, "prefill_bwd: tensors must be 16-byte aligned");
+
+    BwdParams p;
+    p.q = (const __bf16*)q;
+    p.k = (const __bf16*)k;
+    p.v = (const __bf16*)v;
+    p.out = (const __bf16*)out;
+    p.dout = (const __bf16*)dout;
+    p.lse = lse;
+    p.delta = delta;
+    p.dq = (__bf16*)dq;
+    p.dk = (__bf16*)dk;
+    p.dv = (__bf16*)dv;
+    for (int i = 0; i < 3; ++i) {
+        p.qs[i] = q_strides[i];
+        p.ks[i] = k_strides[i];
+        p.vs[i] = v_strides[i];
+        p.os[i] = o_strides[i];
+        p.dos[i] = do_strides[i];
+        p.dqs[i] = dq_strides[i];
+        p.dks[i] = dk_strides[i];
+        p.dvs[i] = dv_strides[i];
+    }
+    p.ls[0] = lse_strides[0];
+    p.ls[1] = lse_strides[1];
+    p.cu_q = cu_seqlens_q;
+    p.cu_k = cu_seqlens_k;
+    p.B = B;
+    p.Hq = Hq;
+    p.Hkv = Hkv;
+    p.Sq = Sq_max;
+    p.Sk = Sk_max;
+    p.scale = softmax_scale;
+    p.scale_log2 = softmax_scale * kLog2e;
+    p.n_qtiles = (Sq_max + kBwCols - 1) / kBwCols;
+    p.n_ktiles = (Sk_max + kBwCols - 1) / kBwCols;
+    if ((int64_t)p.n_qtiles * Hq * B > 0x7fffffffLL || (int64_t)p.n_ktiles * Hkv * B > 0x7fffffffLL)
+        return set_error(MI355_EINVAL, "prefill_bwd: too many workgroups");
+    const int64_t total_rows = cu_seqlens_q ? total_q : (int64_t)B * Sq_max;
+    if (total_rows * Hq * 16 / 256 > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill_bwd: too many rows");
+
+    hipStream_t s = (hipStream_t)stream;
+    const bool causal = mask_mode == MI355_MASK_CAUSAL;
+    int rc = D == 128 ? launch_bwd<128>(p, causal, total_rows, s)
+                      : (D == 64 ? launch_bwd<64>(p, causal, total_rows, s) : launch_bwd<32>(p, causal, total_rows, s));
+    if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}

@@ -25,6 +25,7 @@
 
 #include "common.hpp"
 #include "launch.hpp"
+#include "prefill_tile.hpp"
 
 namespace mi355 {
 
@@ -42,23 +43,14 @@ struct PrefillParams {
     const int32_t* cu_k;
     const uint8_t* mask;
     int64_t ms[3];
+    float* lse;                           // optional: natural-log sum of exp of the scaled scores, per query row
+    int64_t ls[2];                        // its batch and head strides (elements); rows are contiguous
     int B, Hq, Hkv, Sq, Sk;
     float scale_log2;
     int mask_mode;
     int n_qtiles;
     int n_pairs;
 };
-
-// XOR pattern applied to the 16-byte chunk index of LDS row `row` (rows hold D bf16).
-// Chosen so that (a) 16 lanes reading one logical chunk of 16 consecutive rows and
-// (b) a transposed read touching 4 consecutive rows x 32 bytes both spread over
-// distinct banks (LDS banks repeat every 256 bytes).
-template <int D>
-__device__ __forceinline__ int swz(int row) {
-    if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
-    else if constexpr (D == 64) return (((row >> 1) & 3) << 1) | ((row >> 3) & 1);
-    else return (row >> 2) & 3;
-}
 
 template <int D, int MODE>
 __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillParams p) {
@@ -87,6 +79,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
     int sq, sk;
     const __bf16 *qb, *kb, *vb;
     __bf16* ob;
+    float* lb;
     if (p.cu_q) {
         const int q_start = p.cu_q[b], k_start = p.cu_k[b];
         sq = p.cu_q[b + 1] - q_start;
@@ -95,6 +88,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
         kb = p.k + (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
         vb = p.v + (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
         ob = p.out + (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
+        lb = p.lse ? p.lse + q_start + (int64_t)h * p.ls[1] : nullptr;
     } else {
         sq = p.Sq;
         sk = p.Sk;
@@ -102,6 +96,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
         kb = p.k + (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
         vb = p.v + (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
         ob = p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[1];
+        lb = p.lse ? p.lse + (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1] : nullptr;
     }
     // Causal work grows with the query-tile index, so a workgroup takes the tiles
     // (nq-1-pair) and (pair): every workgroup of a sequence then carries the same load.
@@ -346,6 +341,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_fwd_kernel(PrefillPa
         // ---- normalise and store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4 ---
         l_run = xor32_sum(l_run);
         const float inv = 1.0f / l_run;          // l == 0 (no key kept) -> NaN row, like the reference softmax
+        // sum_j exp(scale * s_j) = 2^(m_ref * scale_log2) * l  ->  lse = ln2 * (m_ref * scale_log2 + log2 l)
+        if (lb && q_ok && kg == 0)
+            lb[qi] = l_run > 0.f ? 0.69314718056f * (m_ref * p.scale_log2 + __log2f(l_run)) : -INFINITY;
         if (q_ok) {
             __bf16* orow = ob + (int64_t)qi * p.os[2];
 #pragma unroll
@@ -378,13 +376,12 @@ static int launch_prefill(const PrefillParams& p, hipStream_t stream) {
 
 using namespace mi355;
 
-extern "C" int mi355_prefill_fwd(const void* q, const void* k, const void* v, void* out,
-                                 const int64_t q_strides[3], const int64_t k_strides[3],
-                                 const int64_t v_strides[3], const int64_t o_strides[3],
-                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
-                                 const uint8_t* mask, const int64_t mask_strides[3], int B, int Hq, int Hkv,
-                                 int Sq_max, int Sk_max, int D, float softmax_scale, int mask_mode, int dtype,
-                                 void* stream) {
+static int prefill_common(const void* q, const void* k, const void* v, void* out, const int64_t q_strides[3],
+                          const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                          const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const uint8_t* mask,
+                          const int64_t mask_strides[3], int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
+                          float softmax_scale, int mask_mode, int dtype, float* lse, const int64_t* lse_strides,
+                          void* stream) {
     if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !o_strides)
         return set_error(MI355_EINVAL, "prefill: null pointer argument");
     if (dtype != MI355_BF16) return set_error(MI355_EDTYPE, "prefill: dtype must be MI355_BF16");
@@ -422,6 +419,9 @@ extern "C" int mi355_prefill_fwd(const void* q, const void* k, const void* v, vo
     p.cu_q = cu_seqlens_q;
     p.cu_k = cu_seqlens_k;
     p.mask = mask;
+    p.lse = lse;
+    p.ls[0] = lse ? lse_strides[0] : 0;
+    p.ls[1] = lse ? lse_strides[1] : 0;
     p.B = B;
     p.Hq = Hq;
     p.Hkv = Hkv;
@@ -437,4 +437,30 @@ extern "C" int mi355_prefill_fwd(const void* q, const void* k, const void* v, vo
     int rc = D == 128 ? launch_prefill<128>(p, s) : (D == 64 ? launch_prefill<64>(p, s) : launch_prefill<32>(p, s));
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;
+}
+
+extern "C" int mi355_prefill_fwd(const void* q, const void* k, const void* v, void* out,
+                                 const int64_t q_strides[3], const int64_t k_strides[3],
+                                 const int64_t v_strides[3], const int64_t o_strides[3],
+                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                 const uint8_t* mask, const int64_t mask_strides[3], int B, int Hq, int Hkv,
+                                 int Sq_max, int Sk_max, int D, float softmax_scale, int mask_mode, int dtype,
+                                 void* stream) {
+    return prefill_common(q, k, v, out, q_strides, k_strides, v_strides, o_strides, cu_seqlens_q, cu_seqlens_k, mask,
+                          mask_strides, B, Hq, Hkv, Sq_max, Sk_max, D, softmax_scale, mask_mode, dtype, nullptr, nullptr,
+                          stream);
+}
+
+extern "C" int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out, float* lse,
+                                     const int64_t q_strides[3], const int64_t k_strides[3],
+                                     const int64_t v_strides[3], const int64_t o_strides[3],
+                                     const int64_t lse_strides[2], const int32_t* cu_seqlens_q,
+                                     const int32_t* cu_seqlens_k, int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
+                                     float softmax_scale, int mask_mode, int dtype, void* stream) {
+    if (!lse || !lse_strides) return set_error(MI355_EINVAL, "prefill_fwd_lse: null lse argument");
+    if (mask_mode == MI355_MASK_BOOL)
+        return set_error(MI355_EINVAL, "prefill_fwd_lse: mask_mode must be MI355_MASK_NONE or MI355_MASK_CAUSAL");
+    return prefill_common(q, k, v, out, q_strides, k_strides, v_strides, o_strides, cu_seqlens_q, cu_seqlens_k, nullptr,
+                          nullptr, B, Hq, Hkv, Sq_max, Sk_max, D, softmax_scale, mask_mode, dtype, lse, lse_strides,
+                          stream);
 }

@@ -13,10 +13,13 @@ MI355_FP32 = 2
 MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2
 
 _i64x3 = C.c_int64 * 3
+_i64x2 = C.c_int64 * 2
 _lib = None
 
 EXPORTS = (
     "mi355_prefill_fwd",
+    "mi355_prefill_fwd_lse",
+    "mi355_prefill_bwd",
     "mi355_paged_decode_fwd",
     "mi355_paged_decode_workspace_bytes",
     "mi355_paged_decode_chunk_tokens",
@@ -48,6 +51,12 @@ def load():
     lib.mi355_prefill_fwd.restype = i32
     lib.mi355_prefill_fwd.argtypes = [vp, vp, vp, vp, _i64x3, _i64x3, _i64x3, _i64x3, vp, vp, vp, _i64x3,
                                       i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
+    lib.mi355_prefill_fwd_lse.restype = i32
+    lib.mi355_prefill_fwd_lse.argtypes = [vp, vp, vp, vp, vp, _i64x3, _i64x3, _i64x3, _i64x3, _i64x2, vp, vp,
+                                          i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
+    lib.mi355_prefill_bwd.restype = i32
+    lib.mi355_prefill_bwd.argtypes = [vp] * 10 + [_i64x3] * 8 + [_i64x2, vp, vp, i64,
+                                                                 i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
     lib.mi355_paged_decode_fwd.restype = i32
     lib.mi355_paged_decode_fwd.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, sz,
                                            i32, i32, i32, i32, i32, i32, f32, i32, vp]
@@ -74,6 +83,10 @@ def load():
 
 def strides3(values):
     return _i64x3(*[int(v) for v in values])
+
+
+def strides2(values):
+    return _i64x2(*[int(v) for v in values])
 
 
 def check(rc: int, what: str):

@@ -33,8 +33,24 @@ def _rows16(name, t):
     return t if ok else t.contiguous()
 
 
-def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode):
+def _packed_or_dense_strides(t, packed):
+    """[batch, head, row] element strides of a (B,H,S,D) tensor, or of a packed (T,H,D) one (batch unused)."""
+    return (0, t.stride(1), t.stride(0)) if packed else t.stride()[:3]
+
+
+def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode, lse=None):
     lib = _lib.load()
+    if lse is not None:
+        packed = cu_q is not None
+        qs, ks, vs, os_ = (_packed_or_dense_strides(x, packed) for x in (q, k, v, out))
+        ls = (0, lse.stride(0)) if packed else lse.stride()[:2]
+        rc = lib.mi355_prefill_fwd_lse(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_), _lib.strides2(ls),
+            None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(),
+            B, Hq, Hkv, Sq, Sk, D, float(scale), mode, _lib.MI355_BF16, _stream())
+        _lib.check(rc, "mi355_prefill_fwd_lse")
+        return
     if cu_q is None:
         qs, ks, vs, os_ = (x.stride()[:3] for x in (q, k, v, out))
     else:   # packed (T, H, D): [batch (unused), head, row]
@@ -49,7 +65,7 @@ def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode)
     _lib.check(rc, "mi355_prefill_fwd")
 
 
-def _dense(q, k, v, mask, mode, softmax_scale):
+def _dense(q, k, v, mask, mode, softmax_scale, want_lse=False):
     for n, t in (("q", q), ("k", k), ("v", v)):
         _require_gpu_bf16(n, t)
         if t.dim() != 4:
@@ -65,12 +81,85 @@ def _dense(q, k, v, mask, mode, softmax_scale):
     # (B, S, H, D) memory returned as its (B, H, S, D) view: merging heads afterwards
     # (model.py:388) is then a free reshape instead of a copy.
     out = torch.empty(B, Sq, Hq, D, dtype=q.dtype, device=q.device).permute(0, 2, 1, 3)
+    lse = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device) if want_lse else None
     if B == 0 or Sq == 0:
-        return out
+        return (out, lse) if want_lse else out
     if Sk == 0:
         raise ValueError("attention over zero keys is undefined")
-    _prefill(q, k, v, out, None, None, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode)
-    return out
+    _prefill(q, k, v, out, None, None, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode, lse)
+    return (out, lse) if want_lse else out
+
+
+def _grad_like(t):
+    """Gradient buffer with t's shape and, where t is dense, t's memory layout (so the gradient of the
+    reference's strided V view lands in the layout of the projection it is a view of)."""
+    g = torch.empty_like(t)
+    ok = g.stride(-1) == 1 and all(s % 8 == 0 for s in g.stride()[:-1])
+    return g if ok else torch.empty(t.shape, dtype=t.dtype, device=t.device)
+
+
+def _prefill_backward(q, k, v, out, dout, lse, cu_q, cu_k, Sq, Sk, scale, mode):
+    """dq, dk, dv through mi355_prefill_bwd; tensors dense (B,H,S,D) or packed (T,H,D)."""
+    packed = cu_q is not None
+    q, k, v, out, dout = (_rows16(n, t) for n, t in (("q", q), ("k", k), ("v", v), ("out", out), ("dout", dout)))
+    dq, dk, dv = _grad_like(q), _grad_like(k), _grad_like(v)
+    if q.numel() == 0 or k.numel() == 0:
+        return dq.zero_(), dk.zero_(), dv.zero_()
+    delta = torch.empty_like(lse)
+    if packed:
+        B, (T, Hq, D), Hkv = cu_q.numel() - 1, q.shape, k.shape[1]
+        ls = (0, lse.stride(0))
+    else:
+        (B, Hq, _, D), Hkv, T = q.shape, k.shape[1], 0
+        ls = lse.stride()[:2]
+    st = [_lib.strides3(_packed_or_dense_strides(t, packed)) for t in (q, k, v, out, dout, dq, dk, dv)]
+    rc = _lib.load().mi355_prefill_bwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), *st, _lib.strides2(ls),
+        None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(), T,
+        B, Hq, Hkv, int(Sq), int(Sk), D, float(scale), mode, _lib.MI355_BF16, _stream())
+    _lib.check(rc, "mi355_prefill_bwd")
+    return dq, dk, dv
+
+
+class _DensePrefillFn(torch.autograd.Function):
+    """out = attention(q, k, v) on the HIP forward; backward on the HIP backward kernels."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, causal, softmax_scale):
+        mode = _lib.MASK_CAUSAL if causal else _lib.MASK_NONE
+        out, lse = _dense(q, k, v, None, mode, softmax_scale, want_lse=True)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.mode = mode
+        ctx.scale = 1.0 / math.sqrt(q.shape[-1]) if softmax_scale is None else softmax_scale
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        dq, dk, dv = _prefill_backward(q, k, v, out, dout, lse, None, None, q.shape[2], k.shape[2], ctx.scale, ctx.mode)
+        return dq, dk, dv, None, None
+
+
+class _VarlenPrefillFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, cu_q, cu_k, max_q, max_k, causal, softmax_scale):
+        out, lse = _varlen(q, k, v, cu_q, cu_k, max_q, max_k, causal, softmax_scale, want_lse=True)
+        ctx.save_for_backward(q, k, v, out, lse, cu_q, cu_k)
+        ctx.args = (int(max_q), int(max_k), _lib.MASK_CAUSAL if causal else _lib.MASK_NONE,
+                    1.0 / math.sqrt(q.shape[-1]) if softmax_scale is None else softmax_scale)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, cu_q, cu_k = ctx.saved_tensors
+        max_q, max_k, mode, scale = ctx.args
+        dq, dk, dv = _prefill_backward(q, k, v, out, dout, lse, cu_q, cu_k, max_q, max_k, scale, mode)
+        return dq, dk, dv, None, None, None, None, None, None
+
+
+def _needs_grad(*tensors):
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
 
 
 def flash_attn_prefill(q, k, v, *, causal=True, softmax_scale=None):
@@ -79,7 +168,11 @@ def flash_attn_prefill(q, k, v, *, causal=True, softmax_scale=None):
     Fills the slot of torch.nn.functional.scaled_dot_product_attention(Q, K, V,
     is_causal=True) at llm-core/llm_core/model.py:382.  With Sk > Sq the causal
     diagonal is bottom-right aligned (the queries are the last Sq positions).
+    Differentiable: when an input requires grad, dq/dk/dv come from the HIP backward kernels
+    (what autograd computes behind model.py:382 during train.py's loss.backward()).
     """
+    if _needs_grad(q, k, v):
+        return _DensePrefillFn.apply(q, k, v, bool(causal), softmax_scale)
     return _dense(q, k, v, None, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, softmax_scale)
 
 
@@ -126,12 +219,7 @@ def scaled_dot_product_attention(Q, K, V, mask=None):
     return out.reshape(*lead, nq, d)
 
 
-def flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, *,
-                              causal=True, softmax_scale=None):
-    """Packed ("varlen") prefill.  q (Tq,Hq,D); k, v (Tk,Hkv,D) bf16; cu_seqlens int32 (B+1,), cu[0]=0.
-
-    Sequence b owns rows [cu[b], cu[b+1]).  Returns (Tq,Hq,D) bf16.
-    """
+def _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale, want_lse=False):
     for n, t in (("q", q), ("k", k), ("v", v)):
         _require_gpu_bf16(n, t)
         if t.dim() != 3:
@@ -149,11 +237,23 @@ def flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
     B = cu_seqlens_q.numel() - 1
     scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
     out = torch.empty(Tq, Hq, D, dtype=q.dtype, device=q.device)
-    if Tq == 0 or max_seqlen_q == 0:
-        return out
-    _prefill(q, k, v, out, cu_seqlens_q, cu_seqlens_k, None, B, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k),
-             D, scale, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE)
-    return out
+    lse = torch.empty(Hq, Tq, dtype=torch.float32, device=q.device) if want_lse else None
+    if Tq and max_seqlen_q:
+        _prefill(q, k, v, out, cu_seqlens_q, cu_seqlens_k, None, B, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k),
+                 D, scale, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, lse)
+    return (out, lse) if want_lse else out
+
+
+def flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, *,
+                              causal=True, softmax_scale=None):
+    """Packed ("varlen") prefill.  q (Tq,Hq,D); k, v (Tk,Hkv,D) bf16; cu_seqlens int32 (B+1,), cu[0]=0.
+
+    Sequence b owns rows [cu[b], cu[b+1]).  Returns (Tq,Hq,D) bf16.  Differentiable like flash_attn_prefill.
+    """
+    if _needs_grad(q, k, v):
+        return _VarlenPrefillFn.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, bool(causal),
+                                      softmax_scale)
+    return _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale)
 
 
 def paged_decode_workspace(batch, n_q_heads, head_dim, max_context, device):

@@ -153,6 +153,39 @@ def varlen_prefill_reference(q, k, v, cu_seqlens_q, cu_seqlens_k, *, causal=True
     return out
 
 
+def prefill_backward_reference(q, k, v, dout, *, causal=True, softmax_scale=None):
+    """Gradients of prefill_reference w.r.t. q, k, v for an upstream gradient dout, written out by hand
+    (fp32): with P = softmax(scale * q k^T [masked]) and out = P v,
+
+        dV = P^T dO,   dP = dO V^T,   dS = P * (dP - rowsum(dP * P)),   dQ = scale * dS K,   dK = scale * dS^T Q
+
+    (rowsum(dP * P) = rowsum(dO * out)).  This is what autograd derives for the reference's
+    scaled_dot_product_attention (llm-core/llm_core/model.py:308-325) -- tests/test_oracle.py checks it
+    against torch.autograd on that function and against float64 finite differences.  GQA: the gradient of a
+    kv head is the sum over its query heads.  q, dout (B,Hq,Sq,D); k, v (B,Hkv,Sk,D).  Also returns lse
+    (B,Hq,Sq), the natural-log sum of exp of the scaled, masked scores."""
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    n_rep = Hq // Hkv
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    q32, do32 = q.float(), dout.float()
+    k32 = expand_kv_heads(k.float(), n_rep, 1)
+    v32 = expand_kv_heads(v.float(), n_rep, 1)
+    s = torch.einsum("bhqd,bhkd->bhqk", q32, k32) * scale
+    if causal:
+        s = torch.where(causal_keep_mask(Sq, Sk), s, float("-inf"))
+    lse = torch.logsumexp(s, dim=-1)
+    p = torch.exp(s - lse[..., None])
+    dv = torch.einsum("bhqk,bhqd->bhkd", p, do32)
+    dp = torch.einsum("bhqd,bhkd->bhqk", do32, v32)
+    ds = p * (dp - (dp * p).sum(-1, keepdim=True))
+    dq = torch.einsum("bhqk,bhkd->bhqd", ds, k32) * scale
+    dk = torch.einsum("bhqk,bhqd->bhkd", ds, q32) * scale
+    dk = dk.view(B, Hkv, n_rep, Sk, D).sum(2)
+    dv = dv.view(B, Hkv, n_rep, Sk, D).sum(2)
+    return dq, dk, dv, lse
+
+
 def gather_paged_kv(cache, block_table_row, context_len, scale=None):
     """(num_blocks,Hkv,bs,D) cache + one block-table row -> (Hkv, context_len, D) fp32.
 

@@ -337,3 +337,72 @@ def test_rope_and_cache_reference_scatters_to_slots():
     torch.testing.assert_close(vc2[0, :, 15], v[2])
     torch.testing.assert_close(kc2[1, :, 0], orc.rope_reference(k[4][:, None], torch.tensor([9]), fc)[:, 0])
     assert kc2.abs().sum(dim=(1, 3)).count_nonzero() == 4                       # token 3 (slot -1) was not written
+
+
+# ---------------------------------------------------------------------------------------------
+# backward oracle
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("hq,hkv,sq,sk", [(4, 4, 9, 9), (6, 2, 7, 12), (2, 1, 5, 5)])
+def test_backward_oracle_matches_autograd_of_the_dense_function(causal, hq, hkv, sq, sk):
+    g = torch.Generator().manual_seed(hq * 100 + sq)
+    q = torch.randn(2, hq, sq, 16, generator=g, requires_grad=True)
+    k = torch.randn(2, hkv, sk, 16, generator=g, requires_grad=True)
+    v = torch.randn(2, hkv, sk, 16, generator=g, requires_grad=True)
+    dout = torch.randn(2, hq, sq, 16, generator=g)
+    n_rep = hq // hkv
+    mask = orc.causal_keep_mask(sq, sk) if causal else None
+    out = orc.scaled_dot_product_attention(q, orc.expand_kv_heads(k, n_rep, 1), orc.expand_kv_heads(v, n_rep, 1), mask)
+    want = torch.autograd.grad(out, (q, k, v), dout)
+    dq, dk, dv, lse = orc.prefill_backward_reference(q.detach(), k.detach(), v.detach(), dout, causal=causal)
+    for a, b in zip((dq, dk, dv), want):
+        torch.testing.assert_close(a, b, atol=2e-5, rtol=2e-5)
+    # lse is the log of the softmax denominator of the scaled scores
+    s = torch.einsum("bhqd,bhkd->bhqk", q.detach(), orc.expand_kv_heads(k.detach(), n_rep, 1)) / 4.0
+    if causal:
+        s = torch.where(mask, s, float("-inf"))
+    torch.testing.assert_close(lse, torch.log(torch.exp(s).sum(-1)), atol=1e-5, rtol=1e-5)
+
+
+def test_backward_oracle_matches_float64_finite_differences_and_scale():
+    g = torch.Generator().manual_seed(77)
+    q, k, v = (torch.randn(1, 2, 4, 8, generator=g, dtype=torch.float64) for _ in range(3))
+    dout = torch.randn(1, 2, 4, 8, generator=g, dtype=torch.float64)
+    scale = 0.37
+
+    def loss(q_, k_, v_):
+        keep = orc.causal_keep_mask(4).tolist()
+        tot = 0.0
+        for h in range(2):                    # the 2-D float64 loop function, head by head
+            o = orc.bruteforce_attention_f64((q_[0, h] * (scale * math.sqrt(8))).numpy(), k_[0, h].numpy(),
+                                             v_[0, h].numpy(), keep)
+            tot += float((o * dout[0, h].numpy()).sum())
+        return tot
+
+    dq, dk, dv, _ = orc.prefill_backward_reference(q.float(), k.float(), v.float(), dout.float(), causal=True,
+                                                   softmax_scale=scale)
+    eps = 1e-5
+    for name, t, grad in (("q", q, dq), ("k", k, dk), ("v", v, dv)):
+        for idx in [(0, 0, 0, 0), (0, 1, 2, 5), (0, 0, 3, 7), (0, 1, 1, 3)]:
+            tp, tm = t.clone(), t.clone()
+            tp[idx] += eps
+            tm[idx] -= eps
+            args_p = {"q": (tp, k, v), "k": (q, tp, v), "v": (q, k, tp)}[name]
+            args_m = {"q": (tm, k, v), "k": (q, tm, v), "v": (q, k, tm)}[name]
+            fd = (loss(*args_p) - loss(*args_m)) / (2 * eps)
+            assert abs(fd - float(grad[idx])) < 2e-4, (name, idx, fd, float(grad[idx]))
+
+
+def test_backward_oracle_closed_forms():
+    # one key: out = v for every query, so dv = sum of dout rows, dq = dk = 0
+    g = torch.Generator().manual_seed(5)
+    q, dout = torch.randn(1, 1, 6, 8, generator=g), torch.randn(1, 1, 6, 8, generator=g)
+    k, v = torch.randn(1, 1, 1, 8, generator=g), torch.randn(1, 1, 1, 8, generator=g)
+    dq, dk, dv, _ = orc.prefill_backward_reference(q, k, v, dout, causal=False)
+    torch.testing.assert_close(dv[0, 0, 0], dout[0, 0].sum(0))
+    assert dq.abs().max() < 1e-6 and dk.abs().max() < 1e-6
+    # gradients w.r.t. q and k vanish when dout is a multiple of ... a constant-V problem: out is constant
+    v2 = torch.ones(1, 1, 5, 8)
+    k2 = torch.randn(1, 1, 5, 8, generator=g)
+    dq, dk, _, _ = orc.prefill_backward_reference(q, k2, v2, dout, causal=False)
+    assert dq.abs().max() < 1e-5 and dk.abs().max() < 1e-5
