@@ -13,7 +13,7 @@ The CPU baseline is the oracle (a restatement of the reference's PyTorch attenti
 timed on the host cores over a bounded sample of the same inputs; its outputs also
 check the GPU results of that sample.
 
-usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|fp8|producers|layer]
+usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|fp8|backward|producers|layer]
                        [--no-cpu]
 """
 from __future__ import annotations
@@ -94,6 +94,37 @@ def bench_decode(cfg, args, with_cpu):
     if with_cpu:
         res["cpu_baseline"], res["parity"] = cpu_decode(case, out, cfg)
     return res
+
+
+def bench_prefill_backward(cfg, args):
+    """dq, dk, dv at configs[cfg] (the three backward launches: delta, dk/dv, dq).  FLOPs by the usual
+    convention: 2.5 x the forward's (five GEMMs against two), causal = half."""
+    import torch
+    from mi355_attn import ops, workloads
+
+    case = workloads.prefill_config(cfg, seed=args.seed)
+    S = case.seqlen
+    if case.cu_seqlens is not None:
+        out, lse = ops._varlen(case.q, case.k, case.v, case.cu_seqlens, case.cu_seqlens, S, S, True, None, want_lse=True)
+        cu = case.cu_seqlens
+    else:
+        out, lse = ops._dense(case.q, case.k, case.v, None, 1, None, want_lse=True)
+        cu = None
+    g = torch.Generator(device=case.q.device).manual_seed(args.seed + 1)
+    dout = torch.randn(out.shape, device=out.device, generator=g).to(torch.bfloat16)
+    scale = 1.0 / (case.q.shape[-1] ** 0.5)
+    wall_ms, dev_ms = timed(lambda: ops._prefill_backward(case.q, case.k, case.v, out, dout, lse, cu, cu, S, S, scale, 1),
+                            args.steps, args.warmup)
+    flops = case.flops() * 5 // 2
+    return {
+        "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
+        "algorithmic_flops": flops,
+        "config": {"workload": f"configs[{cfg}] backward: dq, dk, dv of the causal prefill (seed {args.seed})"},
+        "roofline": {"bound": "mfma", "kernel": "bwd_dkv_kernel + bwd_dq_kernel (+ bwd_delta_kernel)",
+                     "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms,
+                     "traffic": _traffic(f"prefill_bwd_cfg{cfg}")},
+    }
 
 
 def bench_producers(args):
@@ -303,7 +334,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", choices=["decode", "prefill", "fp8", "producers", "layer"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "fp8", "backward", "producers", "layer"], default=None)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the 1 GiB plain copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
@@ -373,6 +404,8 @@ def main():
                          "dtype": f8["dtype"], "config": f8["config"], "roofline": f8["roofline"]})
             if with_cpu:
                 line["cpu_baseline"] = f8["cpu_baseline"]
+    if args.only in (None, "backward"):
+        line["prefill_backward"] = bench_prefill_backward(2, args)
     if args.only in (None, "producers"):
         line["cache_producers"] = bench_producers(args)
     if args.only in (None, "layer"):

@@ -16,6 +16,8 @@
 // MFMA pair (S and dP, column = lane) is, converted to bf16, directly the B operand of the
 // second (dQ^T += K^T dS^T; dV^T += dO^T P, dK^T += Q^T dS), and the matching A operand is a
 // transposed LDS read (ds_read_b64_tr_b16) of the streamed tile with the same row permutation.
+#include <type_traits>
+
 #include "common.hpp"
 #include "launch.hpp"
 #include "prefill_tile.hpp"
@@ -126,17 +128,26 @@ struct TileReads {
 
 // ---------------------------------------------------------------------------------------------
 // dQ: one workgroup per tile of 128 queries of one (batch, query head); K/V stream through LDS.
+// Per wavefront: Q and dO fragments of its 32 query columns in registers (64), dQ^T accumulators (64).
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
     using R = TileReads<D>;
     constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
-    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[kTile];
-    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[kTile];
+    // [K buffer 0][K buffer 1][V buffer 0][V buffer 1]
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kTile];
 
-    const int lid = blockIdx.x;
-    const int qtile = p.n_qtiles - 1 - lid % p.n_qtiles;          // heavy (late) causal tiles first
-    const int h = (lid / p.n_qtiles) % p.Hq;
-    const int b = lid / (p.n_qtiles * p.Hq);
+    // Workgroup ids are dealt round-robin to the 8 XCDs (private L2s) and, in order, to their shader
+    // engines: workgroups must carry EQUAL work (a periodic heavy/light pattern starves the engines that
+    // always draw the light ones), and the workgroups that stream the same K/V should share an XCD.  So a
+    // workgroup takes the query-tile PAIR (nq-1-i, i), and the id is remapped so that every XCD works
+    // through a contiguous range of (pair, query head, batch).
+    const int n_wg = gridDim.x;
+    int lid = blockIdx.x;
+    if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
+    const int n_pairs = (p.n_qtiles + 1) / 2;
+    const int pair = lid % n_pairs;
+    const int h = (lid / n_pairs) % p.Hq;
+    const int b = lid / (n_pairs * p.Hq);
     const int hk = h / (p.Hq / p.Hkv);
     int sq, sk;
     int64_t q_base, k_base, v_base, do_base, dq_base, l_base;
@@ -160,22 +171,28 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
         v_base = (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
         l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
     }
-    const int q0 = qtile * kBwCols;
-    if (q0 >= sq) return;
+    const int nq = (sq + kBwCols - 1) / kBwCols;
+    if (sk <= 0 || 2 * pair >= nq) return;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, kg = lane >> 5;
-    const int qi = q0 + 32 * wave + n;
-    const bool q_ok = qi < sq;
     const int coff = sk - sq;
 
     TileLoader<D> ld;
     ld.init(wave, lane);
     R rd;
     rd.init(lane);
-    const uint32_t k_dst = __builtin_amdgcn_readfirstlane(lds_address(k_lds) + wave * TileLoader<D>::NI * 1024);
-    const uint32_t v_dst = __builtin_amdgcn_readfirstlane(lds_address(v_lds) + wave * TileLoader<D>::NI * 1024);
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D>::NI * 1024);
+
+  for (int half = 0; half < 2; ++half) {
+    const int qtile = half == 0 ? nq - 1 - pair : pair;
+    if (half == 1 && qtile == nq - 1 - pair) break;                 // odd tile count: the middle tile has no partner
+    const int q0 = qtile * kBwCols;
+    const int qw0 = q0 + 32 * wave;
+    const int qi = qw0 + n;
+    const bool q_ok = qi < sq;
+    __syncthreads();                                                // the previous half's readers are done with the LDS buffers
 
     // fragments of this lane's query column: step s covers d = 16s + 8kg + j
     bf16x8 qf[NS], dof[NS];
@@ -198,37 +215,35 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
     for (int i = 0; i < NDT; ++i)
 #pragma unroll
         for (int j = 0; j < 16; ++j) dq[i][j] = 0.f;
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     int kv_end = sk;
     if (CAUSAL) kv_end = max(0, min(sk, min(sq, q0 + kBwCols) + coff));
     const int n_tiles = (kv_end + kBwRows - 1) / kBwRows;
-
-    for (int tile = 0; tile < n_tiles; ++tile) {
+    const int last_key = CAUSAL ? min(sk - 1, qi + coff) : sk - 1;      // last key this lane's query sees
+    const auto issue = [&](int tile) {
+        const int r0 = tile * kBwRows, buf = (tile & 1) * kTile;
+        ld.issue(p.k + k_base + (int64_t)r0 * p.ks[2], (int)p.ks[2], sk - 1 - r0, dst + buf);
+        ld.issue(p.v + v_base + (int64_t)r0 * p.vs[2], (int)p.vs[2], sk - 1 - r0, dst + 2 * kTile + buf);
+    };
+    const auto step = [&](auto masked_c, int tile) {
+        constexpr bool MASKED = decltype(masked_c)::value;
         const int k0 = tile * kBwRows;
-        __syncthreads();                                   // everybody is done reading the previous tile
-        ld.issue(p.k + k_base + (int64_t)k0 * p.ks[2], (int)p.ks[2], sk - 1 - k0, k_dst);
-        ld.issue(p.v + v_base + (int64_t)k0 * p.vs[2], (int)p.vs[2], sk - 1 - k0, v_dst);
-        wait_vmcnt<0>();
-        __syncthreads();
-        if (CAUSAL && k0 > q0 + 32 * wave + 31 + coff) continue;   // wholly above this wavefront's diagonal (uniform)
-
+        const unsigned char* k_lds = lds + (tile & 1) * kTile;
+        const unsigned char* v_lds = k_lds + 2 * kTile;
+        const int key_lim = last_key - k0 - 4 * kg;      // element (t,i) is kept iff its tile-relative key index <= key_lim
         f32x16 s_acc[2], dp_acc[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                s_acc[t][j] = 0.f;
-                dp_acc[t][j] = 0.f;
-            }
-#pragma unroll
             for (int s = 0; s < NS; ++s) {
                 const u32x4 kf = *reinterpret_cast<const u32x4*>(k_lds + t * 32 * kRow + rd.row_off[s]);
-                s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s_acc[t]);
+                s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s == 0 ? zero16 : s_acc[t]);
             }
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 const u32x4 vf = *reinterpret_cast<const u32x4*>(v_lds + t * 32 * kRow + rd.row_off[s]);
-                dp_acc[t] = mfma32(as_bf16x8(vf), dof[s], dp_acc[t]);
+                dp_acc[t] = mfma32(as_bf16x8(vf), dof[s], s == 0 ? zero16 : dp_acc[t]);
             }
         }
         // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
@@ -236,11 +251,13 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int key = k0 + 32 * t + 8 * (i >> 2) + 4 * kg + (i & 3);
-                bool keep = key < sk;
-                if (CAUSAL) keep = keep & (key <= qi + coff);
                 const float pr = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -lse2));
-                s_acc[t][i] = keep ? pr * (dp_acc[t][i] - delta) : 0.f;        // dS (without the scale factor)
+                float ds = pr * (dp_acc[t][i] - delta);                        // dS (without the scale factor)
+                if constexpr (MASKED) {
+                    // key index relative to the tile (compile-time part) against this lane's last visible key
+                    ds = (32 * t + 8 * (i >> 2) + (i & 3) <= key_lim) ? ds : 0.f;
+                }
+                s_acc[t][i] = ds;
             }
         // dQ^T (D x 32 queries) += K^T . dS^T, 16 keys at a time
 #pragma unroll
@@ -257,6 +274,15 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
                 dq[dt] = mfma32(join_bf16x8(lo, hi), pf, dq[dt]);
             }
         }
+    };
+
+    if (n_tiles > 0) issue(0);
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        wait_vmcnt<0>();                                   // this wavefront's share of tile `tile` has landed
+        __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
+        if (tile + 1 < n_tiles) issue(tile + 1);
+        if (CAUSAL && tile * kBwRows > qw0 + 31 + coff) continue;      // wholly above this wavefront's diagonal (uniform)
+        step(std::true_type{}, tile);
     }
 
     // store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4
@@ -272,27 +298,35 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
                 *reinterpret_cast<u32x2*>(row + 32 * dt + 8 * g + 4 * kg) = w;
             }
     }
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
-// dK, dV: one workgroup per tile of 128 keys of one (batch, kv head); Q/dO of every query head of
-// the GQA group stream through LDS together with their lse and delta.
-template <int D, bool CAUSAL>
-__global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dkv_kernel(BwdParams p) {
+// dK (WANT_DK) or dV: one workgroup per tile of 128 keys of one (batch, kv head); Q/dO of every query
+// head of the GQA group stream through LDS together with their lse (and delta).  Two launches instead of
+// one kernel that holds both accumulators keep each under 256 registers, i.e. two wavefronts per SIMD.
+// Per wavefront: K (and, for dK, V) fragments of its 32 key columns in registers, one accumulator set (64).
+template <int D, bool CAUSAL, bool WANT_DK>
+__global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dkv_kernel(BwdParams p) {
     using R = TileReads<D>;
     constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
-    __shared__ __attribute__((aligned(1024))) unsigned char q_lds[kTile];
-    __shared__ __attribute__((aligned(1024))) unsigned char do_lds[kTile];
-    __shared__ __attribute__((aligned(16))) float lse_lds[kBwRows];
-    __shared__ __attribute__((aligned(16))) float delta_lds[kBwRows];
+    // [Q buffer 0][Q buffer 1][dO buffer 0][dO buffer 1]
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kTile];
+    __shared__ __attribute__((aligned(16))) float lse_lds2[2 * kBwRows];
+    __shared__ __attribute__((aligned(16))) float delta_lds2[2 * kBwRows];
 
-    const int lid = blockIdx.x;
-    const int ktile = lid % p.n_ktiles;                            // causal: early key tiles carry the most work
-    const int hk = (lid / p.n_ktiles) % p.Hkv;
-    const int b = lid / (p.n_ktiles * p.Hkv);
+    // equal work per workgroup and one XCD per contiguous id range, as in the dQ kernel: a workgroup takes
+    // the key-tile PAIR (i, nk-1-i)
+    const int n_wg = gridDim.x;
+    int lid = blockIdx.x;
+    if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
+    const int n_pairs = (p.n_ktiles + 1) / 2;
+    const int pair = lid % n_pairs;
+    const int hk = (lid / n_pairs) % p.Hkv;
+    const int b = lid / (n_pairs * p.Hkv);
     const int G = p.Hq / p.Hkv;
     int sq, sk, q_start = 0;
-    int64_t k_base, v_base, dk_base, dv_base;
+    int64_t k_base, v_base, o_base;
     if (p.cu_q) {
         q_start = p.cu_q[b];
         const int k_start = p.cu_k[b];
@@ -300,61 +334,72 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dkv_kernel(BwdParams p) 
         sk = p.cu_k[b + 1] - k_start;
         k_base = (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
         v_base = (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
-        dk_base = (int64_t)k_start * p.dks[2] + (int64_t)hk * p.dks[1];
-        dv_base = (int64_t)k_start * p.dvs[2] + (int64_t)hk * p.dvs[1];
+        o_base = WANT_DK ? (int64_t)k_start * p.dks[2] + (int64_t)hk * p.dks[1]
+                         : (int64_t)k_start * p.dvs[2] + (int64_t)hk * p.dvs[1];
     } else {
         sq = p.Sq;
         sk = p.Sk;
         k_base = (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
         v_base = (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
-        dk_base = (int64_t)b * p.dks[0] + (int64_t)hk * p.dks[1];
-        dv_base = (int64_t)b * p.dvs[0] + (int64_t)hk * p.dvs[1];
+        o_base = WANT_DK ? (int64_t)b * p.dks[0] + (int64_t)hk * p.dks[1] : (int64_t)b * p.dvs[0] + (int64_t)hk * p.dvs[1];
     }
-    const int k0 = ktile * kBwCols;
-    if (k0 >= sk) return;
+    const int nk = (sk + kBwCols - 1) / kBwCols;
+    if (sq <= 0 || 2 * pair >= nk) return;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, kg = lane >> 5;
-    const int kj = k0 + 32 * wave + n;
-    const bool k_ok = kj < sk;
     const int coff = sk - sq;
 
     TileLoader<D> ld;
     ld.init(wave, lane);
     R rd;
     rd.init(lane);
-    const uint32_t q_dst = __builtin_amdgcn_readfirstlane(lds_address(q_lds) + wave * TileLoader<D>::NI * 1024);
-    const uint32_t do_dst = __builtin_amdgcn_readfirstlane(lds_address(do_lds) + wave * TileLoader<D>::NI * 1024);
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D>::NI * 1024);
+
+  for (int half = 0; half < 2; ++half) {
+    const int ktile = half == 0 ? pair : nk - 1 - pair;
+    if (half == 1 && ktile == pair) break;                          // odd tile count: the middle tile has no partner
+    const int k0 = ktile * kBwCols;
+    const int kw0 = k0 + 32 * wave;
+    const int kj = kw0 + n;
+    const bool k_ok = kj < sk;
+    __syncthreads();                                                // the previous half's readers are done with the LDS buffers
 
     // fragments of this lane's key column: step s covers d = 16s + 8kg + j
-    bf16x8 kf[NS], vf[NS];
+    bf16x8 kf[NS], vf[WANT_DK ? NS : 1];
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
         u32x4 a = {0u, 0u, 0u, 0u}, g = {0u, 0u, 0u, 0u};
         if (k_ok) {
             a = *reinterpret_cast<const u32x4*>(p.k + k_base + (int64_t)kj * p.ks[2] + 16 * s + 8 * kg);
-            g = *reinterpret_cast<const u32x4*>(p.v + v_base + (int64_t)kj * p.vs[2] + 16 * s + 8 * kg);
+            if (WANT_DK) g = *reinterpret_cast<const u32x4*>(p.v + v_base + (int64_t)kj * p.vs[2] + 16 * s + 8 * kg);
         }
         kf[s] = as_bf16x8(a);
-        vf[s] = as_bf16x8(g);
+        if (WANT_DK) vf[s] = as_bf16x8(g);
     }
-    f32x16 dk[NDT], dv[NDT];
+    f32x16 acc[NDT];
 #pragma unroll
     for (int i = 0; i < NDT; ++i)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            dk[i][j] = 0.f;
-            dv[i][j] = 0.f;
-        }
+        for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // causal: key kj is seen by queries i >= kj - coff; the first row tile that can see key k0
     int first_tile = 0;
     if (CAUSAL) first_tile = max(0, k0 - coff) / kBwRows;
     const int n_tiles = (sq + kBwRows - 1) / kBwRows;
+    // The (query head, row tile) pairs of the GQA group form one stream of steps through the two LDS buffers.
+    const int tiles_per_head = max(0, n_tiles - first_tile);
+    const int n_steps = G * tiles_per_head;
 
-    for (int g = 0; g < G; ++g) {
-        const int h = hk * G + g;
+    // lse (pre-multiplied by log2 e) and delta of the step's 64 rows: loaded into registers by the first
+    // wavefront when the step's tiles are issued, stored to LDS only after the current step's arithmetic,
+    // so that waiting for them never sits in front of it.
+    float pend_lse = 0.f, pend_delta = 0.f;
+    const auto issue = [&](int st) {
+        const int h = hk * G + st / tiles_per_head;
+        const int r0 = (first_tile + st % tiles_per_head) * kBwRows, buf = (st & 1) * kTile;
         int64_t q_base, do_base, l_base;
         if (p.cu_q) {
             q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
@@ -365,102 +410,113 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dkv_kernel(BwdParams p) 
             do_base = (int64_t)b * p.dos[0] + (int64_t)h * p.dos[1];
             l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
         }
-        for (int tile = first_tile; tile < n_tiles; ++tile) {
-            const int r0 = tile * kBwRows;
-            __syncthreads();                               // everybody is done reading the previous tile
-            ld.issue(p.q + q_base + (int64_t)r0 * p.qs[2], (int)p.qs[2], sq - 1 - r0, q_dst);
-            ld.issue(p.dout + do_base + (int64_t)r0 * p.dos[2], (int)p.dos[2], sq - 1 - r0, do_dst);
-            if (tid < kBwRows) {                           // a padded query row gets lse = +inf, i.e. P = 0
-                const bool ok = r0 + tid < sq;
-                lse_lds[tid] = ok ? p.lse[l_base + r0 + tid] * kLog2e : INFINITY;
-                delta_lds[tid] = ok ? p.delta[l_base + r0 + tid] : 0.f;
+        ld.issue(p.q + q_base + (int64_t)r0 * p.qs[2], (int)p.qs[2], sq - 1 - r0, dst + buf);
+        ld.issue(p.dout + do_base + (int64_t)r0 * p.dos[2], (int)p.dos[2], sq - 1 - r0, dst + 2 * kTile + buf);
+        if (tid < kBwRows) {                               // a padded query row gets lse = +inf, i.e. P = 0
+            const bool ok = r0 + tid < sq;
+            pend_lse = ok ? p.lse[l_base + r0 + tid] * kLog2e : INFINITY;
+            if (WANT_DK) pend_delta = ok ? p.delta[l_base + r0 + tid] : 0.f;
+        }
+    };
+    const auto publish = [&](int st) {
+        if (tid < kBwRows) {
+            lse_lds2[(st & 1) * kBwRows + tid] = pend_lse;
+            if (WANT_DK) delta_lds2[(st & 1) * kBwRows + tid] = pend_delta;
+        }
+    };
+    const auto step = [&](auto masked_c, int st, int r0) {
+        constexpr bool MASKED = decltype(masked_c)::value;
+        const unsigned char* q_lds = lds + (st & 1) * kTile;
+        const unsigned char* do_lds = q_lds + 2 * kTile;
+        const float* lse_lds = lse_lds2 + (st & 1) * kBwRows;
+        const float* delta_lds = delta_lds2 + (st & 1) * kBwRows;
+        const int row_lim = CAUSAL ? kj - coff - r0 - 4 * kg : -1;
+        f32x16 s_acc[2], dp_acc[WANT_DK ? 2 : 1];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const u32x4 a = *reinterpret_cast<const u32x4*>(q_lds + t * 32 * kRow + rd.row_off[s]);
+                s_acc[t] = mfma32(as_bf16x8(a), kf[s], s == 0 ? zero16 : s_acc[t]);
             }
-            wait_vmcnt<0>();
-            __syncthreads();
-            // wholly above this wavefront's diagonal: its last key column is not seen by the tile's last row
-            if (CAUSAL && k0 + 32 * wave > r0 + kBwRows - 1 + coff) continue;
-
-            f32x16 s_acc[2], dp_acc[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    s_acc[t][j] = 0.f;
-                    dp_acc[t][j] = 0.f;
-                }
-#pragma unroll
-                for (int s = 0; s < NS; ++s) {
-                    const u32x4 a = *reinterpret_cast<const u32x4*>(q_lds + t * 32 * kRow + rd.row_off[s]);
-                    s_acc[t] = mfma32(as_bf16x8(a), kf[s], s_acc[t]);
-                }
+            if constexpr (WANT_DK) {
 #pragma unroll
                 for (int s = 0; s < NS; ++s) {
                     const u32x4 a = *reinterpret_cast<const u32x4*>(do_lds + t * 32 * kRow + rd.row_off[s]);
-                    dp_acc[t] = mfma32(as_bf16x8(a), vf[s], dp_acc[t]);
-                }
-            }
-            // element (t,i) of this lane: query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int rl = 32 * t + 8 * j + 4 * kg;                    // local row of element i = 4j
-                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_lds + rl);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_lds + rl);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int i = 4 * j + r;
-                        bool keep = true;
-                        if (CAUSAL) keep = kj <= r0 + rl + r + coff;
-                        const float pr = keep ? fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -l4[r])) : 0.f;
-                        s_acc[t][i] = pr;                                      // P
-                        dp_acc[t][i] = pr * (dp_acc[t][i] - d4[r]);            // dS (without the scale factor)
-                    }
-                }
-            // dV^T (D x 32 keys) += dO^T . P ;  dK^T += Q^T . dS, 16 query rows at a time
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int t = u >> 1, e0 = 8 * (u & 1);
-                u32x4 pw, sw;
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
-                    sw[w] = pack_bf16(dp_acc[t][e0 + 2 * w], dp_acc[t][e0 + 2 * w + 1]);
-                }
-                const bf16x8 pf = as_bf16x8(pw), sf = as_bf16x8(sw);
-#pragma unroll
-                for (int dt = 0; dt < NDT; ++dt) {
-                    const i16x4 lo = lds_read_tr16(do_lds + 16 * u * kRow + rd.tr_off[0][dt]);
-                    const i16x4 hi = lds_read_tr16(do_lds + 16 * u * kRow + rd.tr_off[1][dt]);
-                    dv[dt] = mfma32(join_bf16x8(lo, hi), pf, dv[dt]);
-                }
-#pragma unroll
-                for (int dt = 0; dt < NDT; ++dt) {
-                    const i16x4 lo = lds_read_tr16(q_lds + 16 * u * kRow + rd.tr_off[0][dt]);
-                    const i16x4 hi = lds_read_tr16(q_lds + 16 * u * kRow + rd.tr_off[1][dt]);
-                    dk[dt] = mfma32(join_bf16x8(lo, hi), sf, dk[dt]);
+                    dp_acc[t] = mfma32(as_bf16x8(a), vf[s], s == 0 ? zero16 : dp_acc[t]);
                 }
             }
         }
+        // element (t,i) of this lane: query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int rl = 32 * t + 8 * j + 4 * kg;                        // local row of element i = 4j
+                const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_lds + rl);
+                f32x4 d4 = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (WANT_DK) d4 = *reinterpret_cast<const f32x4*>(delta_lds + rl);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 4 * j + r;
+                    float x = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -l4[r]));     // P
+                    if constexpr (WANT_DK) x *= dp_acc[t][i] - d4[r];                  // dS (without the scale factor)
+                    // kept iff kj <= r0 + rl + r + coff, i.e. the tile-relative row (compile-time part) >= row_lim
+                    if constexpr (MASKED) x = (32 * t + 8 * j + r >= row_lim) ? x : 0.f;
+                    s_acc[t][i] = x;
+                }
+            }
+        // dV^T (D x 32 keys) += dO^T . P   or   dK^T += Q^T . dS, 16 query rows at a time
+        const unsigned char* a_lds = WANT_DK ? q_lds : do_lds;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int t = u >> 1, e0 = 8 * (u & 1);
+            u32x4 pw;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
+            const bf16x8 pf = as_bf16x8(pw);
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const i16x4 lo = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[0][dt]);
+                const i16x4 hi = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[1][dt]);
+                acc[dt] = mfma32(join_bf16x8(lo, hi), pf, acc[dt]);
+            }
+        }
+    };
+
+    if (n_steps > 0) {
+        issue(0);
+        publish(0);
+    }
+    for (int st = 0; st < n_steps; ++st) {
+        const bool more = st + 1 < n_steps;
+        const int r0 = (first_tile + st % tiles_per_head) * kBwRows;
+        wait_vmcnt<0>();                                   // this wavefront's share of the step's tiles has landed
+        __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
+        if (more) issue(st + 1);
+        // nothing to do when the tile lies wholly above this wavefront's diagonal (its first key column is
+        // not seen by the tile's last row); no mask when the tile's first row sees the last key column
+        if (!(CAUSAL && kw0 > r0 + kBwRows - 1 + coff)) {
+            step(std::true_type{}, st, r0);
+        }
+        if (more) publish(st + 1);
     }
 
     // store: lane owns key kj, d = 32dt + 8(i/4) + 4kg + i%4
     if (k_ok) {
-        __bf16* krow = p.dk + dk_base + (int64_t)kj * p.dks[2];
-        __bf16* vrow = p.dv + dv_base + (int64_t)kj * p.dvs[2];
+        const float f = WANT_DK ? p.scale : 1.0f;
+        __bf16* row = (WANT_DK ? p.dk + (int64_t)kj * p.dks[2] : p.dv + (int64_t)kj * p.dvs[2]) + o_base;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 u32x2 w;
-                w[0] = pack_bf16(dk[dt][4 * g + 0] * p.scale, dk[dt][4 * g + 1] * p.scale);
-                w[1] = pack_bf16(dk[dt][4 * g + 2] * p.scale, dk[dt][4 * g + 3] * p.scale);
-                *reinterpret_cast<u32x2*>(krow + 32 * dt + 8 * g + 4 * kg) = w;
-                w[0] = pack_bf16(dv[dt][4 * g + 0], dv[dt][4 * g + 1]);
-                w[1] = pack_bf16(dv[dt][4 * g + 2], dv[dt][4 * g + 3]);
-                *reinterpret_cast<u32x2*>(vrow + 32 * dt + 8 * g + 4 * kg) = w;
+                w[0] = pack_bf16(acc[dt][4 * g + 0] * f, acc[dt][4 * g + 1] * f);
+                w[1] = pack_bf16(acc[dt][4 * g + 2] * f, acc[dt][4 * g + 3] * f);
+                *reinterpret_cast<u32x2*>(row + 32 * dt + 8 * g + 4 * kg) = w;
             }
     }
+  }
 }
 
 template <int D>
@@ -469,12 +525,14 @@ static int launch_bwd(const BwdParams& p, bool causal, int64_t total_rows, hipSt
     hipLaunchKernelGGL((bwd_delta_kernel<D>), dim3((unsigned)((delta_threads + 255) / 256)), dim3(256), 0, stream, p,
                        total_rows);
     const dim3 block(kBwWaves * 64);
-    const dim3 grid_q((unsigned)(p.n_qtiles * p.Hq * p.B)), grid_k((unsigned)(p.n_ktiles * p.Hkv * p.B));
+    const dim3 grid_q((unsigned)((p.n_qtiles + 1) / 2 * p.Hq * p.B)), grid_k((unsigned)((p.n_ktiles + 1) / 2 * p.Hkv * p.B));
     if (causal) {
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, true>), grid_k, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, true, false>), grid_k, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, true, true>), grid_k, block, 0, stream, p);
         hipLaunchKernelGGL((bwd_dq_kernel<D, true>), grid_q, block, 0, stream, p);
     } else {
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, false>), grid_k, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, false, false>), grid_k, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, false, true>), grid_k, block, 0, stream, p);
         hipLaunchKernelGGL((bwd_dq_kernel<D, false>), grid_q, block, 0, stream, p);
     }
     return (int)hipGetLastError();
