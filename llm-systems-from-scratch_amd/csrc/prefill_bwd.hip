@@ -185,120 +185,120 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
     rd.init(lane);
     const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D>::NI * 1024);
 
-  for (int half = 0; half < 2; ++half) {
-    const int qtile = half == 0 ? nq - 1 - pair : pair;
-    if (half == 1 && qtile == nq - 1 - pair) break;                 // odd tile count: the middle tile has no partner
-    const int q0 = qtile * kBwCols;
-    const int qw0 = q0 + 32 * wave;
-    const int qi = qw0 + n;
-    const bool q_ok = qi < sq;
-    __syncthreads();                                                // the previous half's readers are done with the LDS buffers
+    for (int half = 0; half < 2; ++half) {
+        const int qtile = half == 0 ? nq - 1 - pair : pair;
+        if (half == 1 && qtile == nq - 1 - pair) break;                 // odd tile count: the middle tile has no partner
+        const int q0 = qtile * kBwCols;
+        const int qw0 = q0 + 32 * wave;
+        const int qi = qw0 + n;
+        const bool q_ok = qi < sq;
+        __syncthreads();                                                // the previous half's readers are done with the LDS buffers
 
-    // fragments of this lane's query column: step s covers d = 16s + 8kg + j
-    bf16x8 qf[NS], dof[NS];
+        // fragments of this lane's query column: step s covers d = 16s + 8kg + j
+        bf16x8 qf[NS], dof[NS];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        u32x4 a = {0u, 0u, 0u, 0u}, g = {0u, 0u, 0u, 0u};
-        if (q_ok) {
-            a = *reinterpret_cast<const u32x4*>(p.q + q_base + (int64_t)qi * p.qs[2] + 16 * s + 8 * kg);
-            g = *reinterpret_cast<const u32x4*>(p.dout + do_base + (int64_t)qi * p.dos[2] + 16 * s + 8 * kg);
-        }
-        qf[s] = as_bf16x8(a);
-        dof[s] = as_bf16x8(g);
-    }
-    // a padded query column gets lse = +inf, i.e. P = 0 everywhere
-    const float lse2 = q_ok ? p.lse[l_base + qi] * kLog2e : INFINITY;
-    const float delta = q_ok ? p.delta[l_base + qi] : 0.f;
-
-    f32x16 dq[NDT];
-#pragma unroll
-    for (int i = 0; i < NDT; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) dq[i][j] = 0.f;
-    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-    int kv_end = sk;
-    if (CAUSAL) kv_end = max(0, min(sk, min(sq, q0 + kBwCols) + coff));
-    const int n_tiles = (kv_end + kBwRows - 1) / kBwRows;
-    const int last_key = CAUSAL ? min(sk - 1, qi + coff) : sk - 1;      // last key this lane's query sees
-    const auto issue = [&](int tile) {
-        const int r0 = tile * kBwRows, buf = (tile & 1) * kTile;
-        ld.issue(p.k + k_base + (int64_t)r0 * p.ks[2], (int)p.ks[2], sk - 1 - r0, dst + buf);
-        ld.issue(p.v + v_base + (int64_t)r0 * p.vs[2], (int)p.vs[2], sk - 1 - r0, dst + 2 * kTile + buf);
-    };
-    const auto step = [&](auto masked_c, int tile) {
-        constexpr bool MASKED = decltype(masked_c)::value;
-        const int k0 = tile * kBwRows;
-        const unsigned char* k_lds = lds + (tile & 1) * kTile;
-        const unsigned char* v_lds = k_lds + 2 * kTile;
-        const int key_lim = last_key - k0 - 4 * kg;      // element (t,i) is kept iff its tile-relative key index <= key_lim
-        f32x16 s_acc[2], dp_acc[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-#pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                const u32x4 kf = *reinterpret_cast<const u32x4*>(k_lds + t * 32 * kRow + rd.row_off[s]);
-                s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s == 0 ? zero16 : s_acc[t]);
+        for (int s = 0; s < NS; ++s) {
+            u32x4 a = {0u, 0u, 0u, 0u}, g = {0u, 0u, 0u, 0u};
+            if (q_ok) {
+                a = *reinterpret_cast<const u32x4*>(p.q + q_base + (int64_t)qi * p.qs[2] + 16 * s + 8 * kg);
+                g = *reinterpret_cast<const u32x4*>(p.dout + do_base + (int64_t)qi * p.dos[2] + 16 * s + 8 * kg);
             }
-#pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                const u32x4 vf = *reinterpret_cast<const u32x4*>(v_lds + t * 32 * kRow + rd.row_off[s]);
-                dp_acc[t] = mfma32(as_bf16x8(vf), dof[s], s == 0 ? zero16 : dp_acc[t]);
-            }
+            qf[s] = as_bf16x8(a);
+            dof[s] = as_bf16x8(g);
         }
-        // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
+        // a padded query column gets lse = +inf, i.e. P = 0 everywhere
+        const float lse2 = q_ok ? p.lse[l_base + qi] * kLog2e : INFINITY;
+        const float delta = q_ok ? p.delta[l_base + qi] : 0.f;
+
+        f32x16 dq[NDT];
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int i = 0; i < NDT; ++i)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float pr = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -lse2));
-                float ds = pr * (dp_acc[t][i] - delta);                        // dS (without the scale factor)
-                if constexpr (MASKED) {
-                    // key index relative to the tile (compile-time part) against this lane's last visible key
-                    ds = (32 * t + 8 * (i >> 2) + (i & 3) <= key_lim) ? ds : 0.f;
+            for (int j = 0; j < 16; ++j) dq[i][j] = 0.f;
+        const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+        int kv_end = sk;
+        if (CAUSAL) kv_end = max(0, min(sk, min(sq, q0 + kBwCols) + coff));
+        const int n_tiles = (kv_end + kBwRows - 1) / kBwRows;
+        const int last_key = CAUSAL ? min(sk - 1, qi + coff) : sk - 1;      // last key this lane's query sees
+        const auto issue = [&](int tile) {
+            const int r0 = tile * kBwRows, buf = (tile & 1) * kTile;
+            ld.issue(p.k + k_base + (int64_t)r0 * p.ks[2], (int)p.ks[2], sk - 1 - r0, dst + buf);
+            ld.issue(p.v + v_base + (int64_t)r0 * p.vs[2], (int)p.vs[2], sk - 1 - r0, dst + 2 * kTile + buf);
+        };
+        const auto step = [&](auto masked_c, int tile) {
+            constexpr bool MASKED = decltype(masked_c)::value;
+            const int k0 = tile * kBwRows;
+            const unsigned char* k_lds = lds + (tile & 1) * kTile;
+            const unsigned char* v_lds = k_lds + 2 * kTile;
+            const int key_lim = last_key - k0 - 4 * kg;      // element (t,i) is kept iff its tile-relative key index <= key_lim
+            f32x16 s_acc[2], dp_acc[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    const u32x4 kf = *reinterpret_cast<const u32x4*>(k_lds + t * 32 * kRow + rd.row_off[s]);
+                    s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s == 0 ? zero16 : s_acc[t]);
                 }
-                s_acc[t][i] = ds;
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    const u32x4 vf = *reinterpret_cast<const u32x4*>(v_lds + t * 32 * kRow + rd.row_off[s]);
+                    dp_acc[t] = mfma32(as_bf16x8(vf), dof[s], s == 0 ? zero16 : dp_acc[t]);
+                }
             }
-        // dQ^T (D x 32 queries) += K^T . dS^T, 16 keys at a time
+            // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int t = u >> 1, e0 = 8 * (u & 1);
-            u32x4 pw;
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int w = 0; w < 4; ++w) pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
-            const bf16x8 pf = as_bf16x8(pw);
+                for (int i = 0; i < 16; ++i) {
+                    const float pr = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -lse2));
+                    float ds = pr * (dp_acc[t][i] - delta);                        // dS (without the scale factor)
+                    if constexpr (MASKED) {
+                        // key index relative to the tile (compile-time part) against this lane's last visible key
+                        ds = (32 * t + 8 * (i >> 2) + (i & 3) <= key_lim) ? ds : 0.f;
+                    }
+                    s_acc[t][i] = ds;
+                }
+            // dQ^T (D x 32 queries) += K^T . dS^T, 16 keys at a time
 #pragma unroll
-            for (int dt = 0; dt < NDT; ++dt) {
-                const i16x4 lo = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[0][dt]);
-                const i16x4 hi = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[1][dt]);
-                dq[dt] = mfma32(join_bf16x8(lo, hi), pf, dq[dt]);
+            for (int u = 0; u < 4; ++u) {
+                const int t = u >> 1, e0 = 8 * (u & 1);
+                u32x4 pw;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
+                const bf16x8 pf = as_bf16x8(pw);
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    const i16x4 lo = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[0][dt]);
+                    const i16x4 hi = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[1][dt]);
+                    dq[dt] = mfma32(join_bf16x8(lo, hi), pf, dq[dt]);
+                }
             }
+        };
+
+        if (n_tiles > 0) issue(0);
+        for (int tile = 0; tile < n_tiles; ++tile) {
+            wait_vmcnt<0>();                                   // this wavefront's share of tile `tile` has landed
+            __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
+            if (tile + 1 < n_tiles) issue(tile + 1);
+            if (CAUSAL && tile * kBwRows > qw0 + 31 + coff) continue;      // wholly above this wavefront's diagonal (uniform)
+            step(std::true_type{}, tile);
         }
-    };
 
-    if (n_tiles > 0) issue(0);
-    for (int tile = 0; tile < n_tiles; ++tile) {
-        wait_vmcnt<0>();                                   // this wavefront's share of tile `tile` has landed
-        __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
-        if (tile + 1 < n_tiles) issue(tile + 1);
-        if (CAUSAL && tile * kBwRows > qw0 + 31 + coff) continue;      // wholly above this wavefront's diagonal (uniform)
-        step(std::true_type{}, tile);
-    }
-
-    // store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4
-    if (q_ok) {
-        __bf16* row = p.dq + dq_base + (int64_t)qi * p.dqs[2];
+        // store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4
+        if (q_ok) {
+            __bf16* row = p.dq + dq_base + (int64_t)qi * p.dqs[2];
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 w;
-                w[0] = pack_bf16(dq[dt][4 * g + 0] * p.scale, dq[dt][4 * g + 1] * p.scale);
-                w[1] = pack_bf16(dq[dt][4 * g + 2] * p.scale, dq[dt][4 * g + 3] * p.scale);
-                *reinterpret_cast<u32x2*>(row + 32 * dt + 8 * g + 4 * kg) = w;
-            }
+                for (int g = 0; g < 4; ++g) {
+                    u32x2 w;
+                    w[0] = pack_bf16(dq[dt][4 * g + 0] * p.scale, dq[dt][4 * g + 1] * p.scale);
+                    w[1] = pack_bf16(dq[dt][4 * g + 2] * p.scale, dq[dt][4 * g + 3] * p.scale);
+                    *reinterpret_cast<u32x2*>(row + 32 * dt + 8 * g + 4 * kg) = w;
+                }
+        }
     }
-  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -357,168 +357,168 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dkv_kernel(BwdParams p) 
     rd.init(lane);
     const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D>::NI * 1024);
 
-  for (int half = 0; half < 2; ++half) {
-    const int ktile = half == 0 ? pair : nk - 1 - pair;
-    if (half == 1 && ktile == pair) break;                          // odd tile count: the middle tile has no partner
-    const int k0 = ktile * kBwCols;
-    const int kw0 = k0 + 32 * wave;
-    const int kj = kw0 + n;
-    const bool k_ok = kj < sk;
-    __syncthreads();                                                // the previous half's readers are done with the LDS buffers
+    for (int half = 0; half < 2; ++half) {
+        const int ktile = half == 0 ? pair : nk - 1 - pair;
+        if (half == 1 && ktile == pair) break;                          // odd tile count: the middle tile has no partner
+        const int k0 = ktile * kBwCols;
+        const int kw0 = k0 + 32 * wave;
+        const int kj = kw0 + n;
+        const bool k_ok = kj < sk;
+        __syncthreads();                                                // the previous half's readers are done with the LDS buffers
 
-    // fragments of this lane's key column: step s covers d = 16s + 8kg + j
-    bf16x8 kf[NS], vf[WANT_DK ? NS : 1];
+        // fragments of this lane's key column: step s covers d = 16s + 8kg + j
+        bf16x8 kf[NS], vf[WANT_DK ? NS : 1];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        u32x4 a = {0u, 0u, 0u, 0u}, g = {0u, 0u, 0u, 0u};
-        if (k_ok) {
-            a = *reinterpret_cast<const u32x4*>(p.k + k_base + (int64_t)kj * p.ks[2] + 16 * s + 8 * kg);
-            if (WANT_DK) g = *reinterpret_cast<const u32x4*>(p.v + v_base + (int64_t)kj * p.vs[2] + 16 * s + 8 * kg);
-        }
-        kf[s] = as_bf16x8(a);
-        if (WANT_DK) vf[s] = as_bf16x8(g);
-    }
-    f32x16 acc[NDT];
-#pragma unroll
-    for (int i = 0; i < NDT; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
-    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-    // causal: key kj is seen by queries i >= kj - coff; the first row tile that can see key k0
-    int first_tile = 0;
-    if (CAUSAL) first_tile = max(0, k0 - coff) / kBwRows;
-    const int n_tiles = (sq + kBwRows - 1) / kBwRows;
-    // The (query head, row tile) pairs of the GQA group form one stream of steps through the two LDS buffers.
-    // Row tiles are walked from the LAST one down: every key tile needs the last rows, so the workgroups of
-    // one (batch, kv head) start on the same Q/dO tiles and share them through the XCD's L2.
-    const int tiles_per_head = max(0, n_tiles - first_tile);
-    const int n_steps = G * tiles_per_head;
-
-    // lse (pre-multiplied by log2 e) and delta of the step's 64 rows: loaded into registers by the first
-    // wavefront when the step's tiles are issued, stored to LDS only after the current step's arithmetic,
-    // so that waiting for them never sits in front of it.
-    float pend_lse = 0.f, pend_delta = 0.f;
-    const auto issue = [&](int st) {
-        const int h = hk * G + st / tiles_per_head;
-        const int r0 = (n_tiles - 1 - st % tiles_per_head) * kBwRows, buf = (st & 1) * kTile;
-        int64_t q_base, do_base, l_base;
-        if (p.cu_q) {
-            q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
-            do_base = (int64_t)q_start * p.dos[2] + (int64_t)h * p.dos[1];
-            l_base = q_start + (int64_t)h * p.ls[1];
-        } else {
-            q_base = (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
-            do_base = (int64_t)b * p.dos[0] + (int64_t)h * p.dos[1];
-            l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
-        }
-        ld.issue(p.q + q_base + (int64_t)r0 * p.qs[2], (int)p.qs[2], sq - 1 - r0, dst + buf);
-        ld.issue(p.dout + do_base + (int64_t)r0 * p.dos[2], (int)p.dos[2], sq - 1 - r0, dst + 2 * kTile + buf);
-        if (tid < kBwRows) {                               // a padded query row gets lse = +inf, i.e. P = 0
-            const bool ok = r0 + tid < sq;
-            pend_lse = ok ? p.lse[l_base + r0 + tid] * kLog2e : INFINITY;
-            if (WANT_DK) pend_delta = ok ? p.delta[l_base + r0 + tid] : 0.f;
-        }
-    };
-    const auto publish = [&](int st) {
-        if (tid < kBwRows) {
-            lse_lds2[(st & 1) * kBwRows + tid] = pend_lse;
-            if (WANT_DK) delta_lds2[(st & 1) * kBwRows + tid] = pend_delta;
-        }
-    };
-    const auto step = [&](auto masked_c, int st, int r0) {
-        constexpr bool MASKED = decltype(masked_c)::value;
-        const unsigned char* q_lds = lds + (st & 1) * kTile;
-        const unsigned char* do_lds = q_lds + 2 * kTile;
-        const float* lse_lds = lse_lds2 + (st & 1) * kBwRows;
-        const float* delta_lds = delta_lds2 + (st & 1) * kBwRows;
-        const int row_lim = CAUSAL ? kj - coff - r0 - 4 * kg : -1;
-        f32x16 s_acc[2], dp_acc[WANT_DK ? 2 : 1];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-#pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                const u32x4 a = *reinterpret_cast<const u32x4*>(q_lds + t * 32 * kRow + rd.row_off[s]);
-                s_acc[t] = mfma32(as_bf16x8(a), kf[s], s == 0 ? zero16 : s_acc[t]);
+        for (int s = 0; s < NS; ++s) {
+            u32x4 a = {0u, 0u, 0u, 0u}, g = {0u, 0u, 0u, 0u};
+            if (k_ok) {
+                a = *reinterpret_cast<const u32x4*>(p.k + k_base + (int64_t)kj * p.ks[2] + 16 * s + 8 * kg);
+                if (WANT_DK) g = *reinterpret_cast<const u32x4*>(p.v + v_base + (int64_t)kj * p.vs[2] + 16 * s + 8 * kg);
             }
-            if constexpr (WANT_DK) {
+            kf[s] = as_bf16x8(a);
+            if (WANT_DK) vf[s] = as_bf16x8(g);
+        }
+        f32x16 acc[NDT];
+#pragma unroll
+        for (int i = 0; i < NDT; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+        const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+        // causal: key kj is seen by queries i >= kj - coff; the first row tile that can see key k0
+        int first_tile = 0;
+        if (CAUSAL) first_tile = max(0, k0 - coff) / kBwRows;
+        const int n_tiles = (sq + kBwRows - 1) / kBwRows;
+        // The (query head, row tile) pairs of the GQA group form one stream of steps through the two LDS buffers.
+        // Row tiles are walked from the LAST one down: every key tile needs the last rows, so the workgroups of
+        // one (batch, kv head) start on the same Q/dO tiles and share them through the XCD's L2.
+        const int tiles_per_head = max(0, n_tiles - first_tile);
+        const int n_steps = G * tiles_per_head;
+
+        // lse (pre-multiplied by log2 e) and delta of the step's 64 rows: loaded into registers by the first
+        // wavefront when the step's tiles are issued, stored to LDS only after the current step's arithmetic,
+        // so that waiting for them never sits in front of it.
+        float pend_lse = 0.f, pend_delta = 0.f;
+        const auto issue = [&](int st) {
+            const int h = hk * G + st / tiles_per_head;
+            const int r0 = (n_tiles - 1 - st % tiles_per_head) * kBwRows, buf = (st & 1) * kTile;
+            int64_t q_base, do_base, l_base;
+            if (p.cu_q) {
+                q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
+                do_base = (int64_t)q_start * p.dos[2] + (int64_t)h * p.dos[1];
+                l_base = q_start + (int64_t)h * p.ls[1];
+            } else {
+                q_base = (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
+                do_base = (int64_t)b * p.dos[0] + (int64_t)h * p.dos[1];
+                l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
+            }
+            ld.issue(p.q + q_base + (int64_t)r0 * p.qs[2], (int)p.qs[2], sq - 1 - r0, dst + buf);
+            ld.issue(p.dout + do_base + (int64_t)r0 * p.dos[2], (int)p.dos[2], sq - 1 - r0, dst + 2 * kTile + buf);
+            if (tid < kBwRows) {                               // a padded query row gets lse = +inf, i.e. P = 0
+                const bool ok = r0 + tid < sq;
+                pend_lse = ok ? p.lse[l_base + r0 + tid] * kLog2e : INFINITY;
+                if (WANT_DK) pend_delta = ok ? p.delta[l_base + r0 + tid] : 0.f;
+            }
+        };
+        const auto publish = [&](int st) {
+            if (tid < kBwRows) {
+                lse_lds2[(st & 1) * kBwRows + tid] = pend_lse;
+                if (WANT_DK) delta_lds2[(st & 1) * kBwRows + tid] = pend_delta;
+            }
+        };
+        const auto step = [&](auto masked_c, int st, int r0) {
+            constexpr bool MASKED = decltype(masked_c)::value;
+            const unsigned char* q_lds = lds + (st & 1) * kTile;
+            const unsigned char* do_lds = q_lds + 2 * kTile;
+            const float* lse_lds = lse_lds2 + (st & 1) * kBwRows;
+            const float* delta_lds = delta_lds2 + (st & 1) * kBwRows;
+            const int row_lim = CAUSAL ? kj - coff - r0 - 4 * kg : -1;
+            f32x16 s_acc[2], dp_acc[WANT_DK ? 2 : 1];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
 #pragma unroll
                 for (int s = 0; s < NS; ++s) {
-                    const u32x4 a = *reinterpret_cast<const u32x4*>(do_lds + t * 32 * kRow + rd.row_off[s]);
-                    dp_acc[t] = mfma32(as_bf16x8(a), vf[s], s == 0 ? zero16 : dp_acc[t]);
+                    const u32x4 a = *reinterpret_cast<const u32x4*>(q_lds + t * 32 * kRow + rd.row_off[s]);
+                    s_acc[t] = mfma32(as_bf16x8(a), kf[s], s == 0 ? zero16 : s_acc[t]);
+                }
+                if constexpr (WANT_DK) {
+#pragma unroll
+                    for (int s = 0; s < NS; ++s) {
+                        const u32x4 a = *reinterpret_cast<const u32x4*>(do_lds + t * 32 * kRow + rd.row_off[s]);
+                        dp_acc[t] = mfma32(as_bf16x8(a), vf[s], s == 0 ? zero16 : dp_acc[t]);
+                    }
                 }
             }
-        }
-        // element (t,i) of this lane: query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
+            // element (t,i) of this lane: query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int rl = 32 * t + 8 * j + 4 * kg;                        // local row of element i = 4j
-                const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_lds + rl);
-                f32x4 d4 = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (WANT_DK) d4 = *reinterpret_cast<const f32x4*>(delta_lds + rl);
+                for (int j = 0; j < 4; ++j) {
+                    const int rl = 32 * t + 8 * j + 4 * kg;                        // local row of element i = 4j
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_lds + rl);
+                    f32x4 d4 = {0.f, 0.f, 0.f, 0.f};
+                    if constexpr (WANT_DK) d4 = *reinterpret_cast<const f32x4*>(delta_lds + rl);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 4 * j + r;
-                    float x = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -l4[r]));     // P
-                    if constexpr (WANT_DK) x *= dp_acc[t][i] - d4[r];                  // dS (without the scale factor)
-                    // kept iff kj <= r0 + rl + r + coff, i.e. the tile-relative row (compile-time part) >= row_lim
-                    if constexpr (MASKED) x = (32 * t + 8 * j + r >= row_lim) ? x : 0.f;
-                    s_acc[t][i] = x;
+                    for (int r = 0; r < 4; ++r) {
+                        const int i = 4 * j + r;
+                        float x = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -l4[r]));     // P
+                        if constexpr (WANT_DK) x *= dp_acc[t][i] - d4[r];                  // dS (without the scale factor)
+                        // kept iff kj <= r0 + rl + r + coff, i.e. the tile-relative row (compile-time part) >= row_lim
+                        if constexpr (MASKED) x = (32 * t + 8 * j + r >= row_lim) ? x : 0.f;
+                        s_acc[t][i] = x;
+                    }
+                }
+            // dV^T (D x 32 keys) += dO^T . P   or   dK^T += Q^T . dS, 16 query rows at a time
+            const unsigned char* a_lds = WANT_DK ? q_lds : do_lds;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int t = u >> 1, e0 = 8 * (u & 1);
+                u32x4 pw;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
+                const bf16x8 pf = as_bf16x8(pw);
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) {
+                    const i16x4 lo = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[0][dt]);
+                    const i16x4 hi = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[1][dt]);
+                    acc[dt] = mfma32(join_bf16x8(lo, hi), pf, acc[dt]);
                 }
             }
-        // dV^T (D x 32 keys) += dO^T . P   or   dK^T += Q^T . dS, 16 query rows at a time
-        const unsigned char* a_lds = WANT_DK ? q_lds : do_lds;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int t = u >> 1, e0 = 8 * (u & 1);
-            u32x4 pw;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
-            const bf16x8 pf = as_bf16x8(pw);
-#pragma unroll
-            for (int dt = 0; dt < NDT; ++dt) {
-                const i16x4 lo = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[0][dt]);
-                const i16x4 hi = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[1][dt]);
-                acc[dt] = mfma32(join_bf16x8(lo, hi), pf, acc[dt]);
-            }
-        }
-    };
+        };
 
-    if (n_steps > 0) {
-        issue(0);
-        publish(0);
-    }
-    for (int st = 0; st < n_steps; ++st) {
-        const bool more = st + 1 < n_steps;
-        const int r0 = (n_tiles - 1 - st % tiles_per_head) * kBwRows;
-        wait_vmcnt<0>();                                   // this wavefront's share of the step's tiles has landed
-        __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
-        if (more) issue(st + 1);
-        // nothing to do when the tile lies wholly above this wavefront's diagonal (its first key column is
-        // not seen by the tile's last row); no mask when the tile's first row sees the last key column
-        if (!(CAUSAL && kw0 > r0 + kBwRows - 1 + coff)) {
-            step(std::true_type{}, st, r0);
+        if (n_steps > 0) {
+            issue(0);
+            publish(0);
         }
-        if (more) publish(st + 1);
-    }
-
-    // store: lane owns key kj, d = 32dt + 8(i/4) + 4kg + i%4
-    if (k_ok) {
-        const float f = WANT_DK ? p.scale : 1.0f;
-        __bf16* row = (WANT_DK ? p.dk + (int64_t)kj * p.dks[2] : p.dv + (int64_t)kj * p.dvs[2]) + o_base;
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 w;
-                w[0] = pack_bf16(acc[dt][4 * g + 0] * f, acc[dt][4 * g + 1] * f);
-                w[1] = pack_bf16(acc[dt][4 * g + 2] * f, acc[dt][4 * g + 3] * f);
-                *reinterpret_cast<u32x2*>(row + 32 * dt + 8 * g + 4 * kg) = w;
+        for (int st = 0; st < n_steps; ++st) {
+            const bool more = st + 1 < n_steps;
+            const int r0 = (n_tiles - 1 - st % tiles_per_head) * kBwRows;
+            wait_vmcnt<0>();                                   // this wavefront's share of the step's tiles has landed
+            __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
+            if (more) issue(st + 1);
+            // nothing to do when the tile lies wholly above this wavefront's diagonal (its first key column is
+            // not seen by the tile's last row); no mask when the tile's first row sees the last key column
+            if (!(CAUSAL && kw0 > r0 + kBwRows - 1 + coff)) {
+                step(std::true_type{}, st, r0);
             }
+            if (more) publish(st + 1);
+        }
+
+        // store: lane owns key kj, d = 32dt + 8(i/4) + 4kg + i%4
+        if (k_ok) {
+            const float f = WANT_DK ? p.scale : 1.0f;
+            __bf16* row = (WANT_DK ? p.dk + (int64_t)kj * p.dks[2] : p.dv + (int64_t)kj * p.dvs[2]) + o_base;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    u32x2 w;
+                    w[0] = pack_bf16(acc[dt][4 * g + 0] * f, acc[dt][4 * g + 1] * f);
+                    w[1] = pack_bf16(acc[dt][4 * g + 2] * f, acc[dt][4 * g + 3] * f);
+                    *reinterpret_cast<u32x2*>(row + 32 * dt + 8 * g + 4 * kg) = w;
+                }
+        }
     }
-  }
 }
 
 template <int D>
