@@ -132,14 +132,18 @@ int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* o
  *                   real value = fp8 value * scale
  *   workspace     : >= mi355_paged_decode_workspace_bytes(...) bytes, 16-byte
  *                   aligned, contents irrelevant on entry (split-K partials)
- *   max_ctx       : upper bound on every context_lens[b] (sizes the grid)
+ *   num_blocks    : blocks in the pool; a table entry outside [0, num_blocks) is clamped into
+ *                   the pool (the result for that sequence is then meaningless, but no
+ *                   memory outside the caches is touched)
+ *   max_ctx       : upper bound on every context_lens[b] (sizes the grid); a larger
+ *                   context_lens[b] is truncated to it
  */
 int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
                            const int32_t* block_tables, int64_t bt_row_stride,
                            const int32_t* context_lens,
                            const float* k_scale, const float* v_scale,
                            void* workspace, size_t workspace_bytes,
-                           int B, int Hq, int Hkv, int D, int block_size, int max_ctx,
+                           int B, int Hq, int Hkv, int D, int block_size, int64_t num_blocks, int max_ctx,
                            float softmax_scale, int kv_dtype, void* stream);
 
 size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx);

@@ -41,6 +41,7 @@ struct DecodeParams {
     __bf16* out;
     const int32_t* block_tables;
     int64_t bt_row_stride;
+    int num_blocks;
     const int32_t* context_lens;
     const float* k_scale;
     const float* v_scale;
@@ -131,7 +132,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
     // once: lane l holds logical block t0/16 + l, clamped to the sequence's last block so that
     // every id is a real block.  The step loop reads them with v_readlane, so no dependent
     // table load sits between two steps.
-    const int my_phys = bt[min(t0 / kBlock + lane, last_blk)];
+    // a block id outside the pool (a corrupted table) is clamped into it: wrong numbers, never a wild read
+    const int my_phys = min(max(bt[min(t0 / kBlock + lane, last_blk)], 0), p.num_blocks - 1);
     float my_ks = 1.0f, my_vs = 1.0f;
     if constexpr (FP8) {
         my_ks = p.k_scale[(int64_t)my_phys * p.Hkv + hk];
@@ -423,7 +425,7 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
                                       const int32_t* block_tables, int64_t bt_row_stride,
                                       const int32_t* context_lens, const float* k_scale,
                                       const float* v_scale, void* workspace, size_t workspace_bytes, int B,
-                                      int Hq, int Hkv, int D, int block_size, int max_ctx,
+                                      int Hq, int Hkv, int D, int block_size, int64_t num_blocks, int max_ctx,
                                       float softmax_scale, int kv_dtype, void* stream) {
     if (!q || !k_cache || !v_cache || !out || !block_tables || !context_lens)
         return set_error(MI355_EINVAL, "paged_decode: null pointer argument");
@@ -432,6 +434,8 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
     if (Hq % Hkv != 0 || Hq / Hkv > 16)
         return set_error(MI355_EINVAL, "paged_decode: Hq must be a multiple of Hkv with Hq/Hkv <= 16");
     if (block_size != kBlock) return set_error(MI355_EINVAL, "paged_decode: block_size must be 16");
+    if (num_blocks <= 0 || num_blocks > 0x7fffffffLL)
+        return set_error(MI355_EINVAL, "paged_decode: num_blocks must be positive (and below 2^31)");
     const int chunk = mi355_paged_decode_chunk_tokens(max_ctx);
     if ((int64_t)((max_ctx + chunk - 1) / chunk) * Hkv * B > 0x7fffffffLL)
         return set_error(MI355_EINVAL, "paged_decode: chunks * Hkv * B exceeds the grid limit");
@@ -454,6 +458,7 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
     p.out = (__bf16*)out;
     p.block_tables = block_tables;
     p.bt_row_stride = bt_row_stride;
+    p.num_blocks = (int)num_blocks;
     p.context_lens = context_lens;
     p.k_scale = k_scale;
     p.v_scale = v_scale;

@@ -59,7 +59,7 @@ def load():
                                                                  i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
     lib.mi355_paged_decode_fwd.restype = i32
     lib.mi355_paged_decode_fwd.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, sz,
-                                           i32, i32, i32, i32, i32, i32, f32, i32, vp]
+                                           i32, i32, i32, i32, i32, i64, i32, f32, i32, vp]
     lib.mi355_paged_decode_workspace_bytes.restype = sz
     lib.mi355_paged_decode_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.mi355_paged_decode_chunk_tokens.restype = i32

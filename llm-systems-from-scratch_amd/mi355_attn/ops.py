@@ -16,8 +16,26 @@ from . import _lib
 _BLOCK = 16
 
 
-def _stream():
-    return torch.cuda.current_stream().cuda_stream
+class _on:
+    """`with _on(t0, t1, ...) as stream:` -- checks that every given tensor lives on one GPU, makes that GPU
+    the current device for the launch and yields its current stream (as the integer the C ABI takes)."""
+
+    def __init__(self, *tensors):
+        ts = [t for t in tensors if t is not None]
+        self.device = ts[0].device
+        for t in ts:
+            if t.device != self.device:
+                raise ValueError(f"all tensors of one call must be on one device (got {self.device} and {t.device})")
+        if self.device.type != "cuda":
+            raise ValueError(f"tensors must live on the GPU (got {self.device}); this library has no CPU path")
+        self._guard = torch.cuda.device(self.device)
+
+    def __enter__(self):
+        self._guard.__enter__()
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def __exit__(self, *exc):
+        return self._guard.__exit__(*exc)
 
 
 def _require_gpu_bf16(name, t):
@@ -44,11 +62,12 @@ def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode,
         packed = cu_q is not None
         qs, ks, vs, os_ = (_packed_or_dense_strides(x, packed) for x in (q, k, v, out))
         ls = (0, lse.stride(0)) if packed else lse.stride()[:2]
-        rc = lib.mi355_prefill_fwd_lse(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
-            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_), _lib.strides2(ls),
-            None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(),
-            B, Hq, Hkv, Sq, Sk, D, float(scale), mode, _lib.MI355_BF16, _stream())
+        with _on(q, k, v, out, lse, cu_q, cu_k) as stream:
+            rc = lib.mi355_prefill_fwd_lse(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_), _lib.strides2(ls),
+                None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(),
+                B, Hq, Hkv, Sq, Sk, D, float(scale), mode, _lib.MI355_BF16, stream)
         _lib.check(rc, "mi355_prefill_fwd_lse")
         return
     if cu_q is None:
@@ -56,12 +75,13 @@ def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode,
     else:   # packed (T, H, D): [batch (unused), head, row]
         qs, ks, vs, os_ = ((0, x.stride(1), x.stride(0)) for x in (q, k, v, out))
     ms = (0, 0, 0) if mask is None else mask.stride()[:3]
-    rc = lib.mi355_prefill_fwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-        _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
-        None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(),
-        None if mask is None else mask.data_ptr(), _lib.strides3(ms),
-        B, Hq, Hkv, Sq, Sk, D, float(scale), mode, _lib.MI355_BF16, _stream())
+    with _on(q, k, v, out, cu_q, cu_k, mask) as stream:
+        rc = lib.mi355_prefill_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
+            None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(),
+            None if mask is None else mask.data_ptr(), _lib.strides3(ms),
+            B, Hq, Hkv, Sq, Sk, D, float(scale), mode, _lib.MI355_BF16, stream)
     _lib.check(rc, "mi355_prefill_fwd")
 
 
@@ -113,11 +133,12 @@ def _prefill_backward(q, k, v, out, dout, lse, cu_q, cu_k, Sq, Sk, scale, mode):
         (B, Hq, _, D), Hkv, T = q.shape, k.shape[1], 0
         ls = lse.stride()[:2]
     st = [_lib.strides3(_packed_or_dense_strides(t, packed)) for t in (q, k, v, out, dout, dq, dk, dv)]
-    rc = _lib.load().mi355_prefill_bwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), *st, _lib.strides2(ls),
-        None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(), T,
-        B, Hq, Hkv, int(Sq), int(Sk), D, float(scale), mode, _lib.MI355_BF16, _stream())
+    with _on(q, k, v, out, dout, lse, cu_q, cu_k) as stream:
+        rc = _lib.load().mi355_prefill_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), *st, _lib.strides2(ls),
+            None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(), T,
+            B, Hq, Hkv, int(Sq), int(Sk), D, float(scale), mode, _lib.MI355_BF16, stream)
     _lib.check(rc, "mi355_prefill_bwd")
     return dq, dk, dv
 
@@ -317,13 +338,14 @@ def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, s
     lib = _lib.load()
     if workspace is None:
         workspace = paged_decode_workspace(B, Hq, D, max_context, q.device)
-    rc = lib.mi355_paged_decode_fwd(
-        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
-        block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
-        k_scale.data_ptr() if fp8 else None, v_scale.data_ptr() if fp8 else None,
-        workspace.data_ptr(), workspace.numel() * workspace.element_size(),
-        B, Hq, Hkv, D, bs, int(max_context), float(scale),
-        _lib.MI355_FP8_E4M3 if fp8 else _lib.MI355_BF16, _stream())
+    with _on(q, k_cache, v_cache, out, block_tables, context_lens, k_scale, v_scale, workspace) as stream:
+        rc = lib.mi355_paged_decode_fwd(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+            block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
+            k_scale.data_ptr() if fp8 else None, v_scale.data_ptr() if fp8 else None,
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+            B, Hq, Hkv, D, bs, k_cache.shape[0], int(max_context), float(scale),
+            _lib.MI355_FP8_E4M3 if fp8 else _lib.MI355_BF16, stream)
     _lib.check(rc, "mi355_paged_decode_fwd")
     return out
 
@@ -374,11 +396,12 @@ def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, s
             raise ValueError("out must have q's shape with contiguous heads")
     if T == 0:
         return q_out
-    rc = _lib.load().mi355_rope_and_cache(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
-        None if slot_mapping is None else k_cache.data_ptr(), None if slot_mapping is None else v_cache.data_ptr(),
-        freq_cache.data_ptr(), positions.data_ptr(), None if slot_mapping is None else slot_mapping.data_ptr(),
-        T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0), _stream())
+    with _on(q, k, v, q_out, freq_cache, positions, slot_mapping, k_cache, v_cache) as stream:
+        rc = _lib.load().mi355_rope_and_cache(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
+            None if slot_mapping is None else k_cache.data_ptr(), None if slot_mapping is None else v_cache.data_ptr(),
+            freq_cache.data_ptr(), positions.data_ptr(), None if slot_mapping is None else slot_mapping.data_ptr(),
+            T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0), stream)
     _lib.check(rc, "mi355_rope_and_cache")
     return q_out
 
@@ -400,8 +423,9 @@ def quantize_kv_cache_fp8(cache, *, out=None):
         if scale.dtype != torch.float32 or scale.shape != (nb, Hkv) or not scale.is_contiguous() \
                 or scale.device != cache.device:
             raise ValueError("out[1] must be a contiguous float32 (num_blocks, kv_heads) tensor on the cache's device")
-    rc = _lib.load().mi355_quantize_kv_fp8(cache.data_ptr(), out.data_ptr(), scale.data_ptr(), nb, Hkv, D, _BLOCK,
-                                           _stream())
+    with _on(cache, out, scale) as stream:
+        rc = _lib.load().mi355_quantize_kv_fp8(cache.data_ptr(), out.data_ptr(), scale.data_ptr(), nb, Hkv, D, _BLOCK,
+                                               stream)
     _lib.check(rc, "mi355_quantize_kv_fp8")
     return out, scale
 
@@ -448,10 +472,11 @@ def rms_norm(x, weight, eps: float = 1e-5, *, residual=None, return_sum: bool = 
     h = torch.empty(x.shape, dtype=x.dtype, device=x.device) if return_sum else None
     rstd = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device) if return_rstd else None
     if n_rows:
-        rc = _lib.load().mi355_rms_norm_fwd(
-            x2.data_ptr(), None if r2 is None else r2.data_ptr(), weight.data_ptr(), y.data_ptr(),
-            None if h is None else h.data_ptr(), None if rstd is None else rstd.data_ptr(),
-            n_rows, d, x2.stride(0), 0 if r2 is None else r2.stride(0), d, d, float(eps), wcode, _stream())
+        with _on(x2, r2, weight) as stream:
+            rc = _lib.load().mi355_rms_norm_fwd(
+                x2.data_ptr(), None if r2 is None else r2.data_ptr(), weight.data_ptr(), y.data_ptr(),
+                None if h is None else h.data_ptr(), None if rstd is None else rstd.data_ptr(),
+                n_rows, d, x2.stride(0), 0 if r2 is None else r2.stride(0), d, d, float(eps), wcode, stream)
         _lib.check(rc, "mi355_rms_norm_fwd")
     extra = [t for t in (h, rstd) if t is not None]
     return (y, *extra) if extra else y
@@ -468,7 +493,8 @@ def silu_mul(gate, up):
     out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
     n_rows, d = g2.shape
     if n_rows and d:
-        rc = _lib.load().mi355_silu_mul_fwd(g2.data_ptr(), u2.data_ptr(), out.data_ptr(), n_rows, d,
-                                            g2.stride(0), u2.stride(0), d, _stream())
+        with _on(g2, u2) as stream:
+            rc = _lib.load().mi355_silu_mul_fwd(g2.data_ptr(), u2.data_ptr(), out.data_ptr(), n_rows, d,
+                                                g2.stride(0), u2.stride(0), d, stream)
         _lib.check(rc, "mi355_silu_mul_fwd")
     return out

@@ -71,9 +71,9 @@ def test_decode_rejects_bad_arguments_without_a_gpu(lib):
     buf = C.create_string_buffer(64)
     ptr = C.addressof(buf)
 
-    def call(Hq=8, Hkv=2, D=128, bs=16, kv=_lib.MI355_BF16, ks=None, ws=ptr, ws_bytes=1 << 30, max_ctx=64, q=ptr):
+    def call(Hq=8, Hkv=2, D=128, bs=16, kv=_lib.MI355_BF16, ks=None, ws=ptr, ws_bytes=1 << 30, max_ctx=64, q=ptr, nb=8):
         return lib.mi355_paged_decode_fwd(q, ptr, ptr, ptr, ptr, 4, ptr, ks, ks, ws, ws_bytes,
-                                          2, Hq, Hkv, D, bs, max_ctx, 0.1, kv, None)
+                                          2, Hq, Hkv, D, bs, nb, max_ctx, 0.1, kv, None)
 
     assert call(bs=32) == -1 and b"block_size" in lib.mi355_last_error()
     assert call(Hq=7) == -1
@@ -83,6 +83,7 @@ def test_decode_rejects_bad_arguments_without_a_gpu(lib):
     assert call(kv=_lib.MI355_FP8_E4M3, ks=None) == -1 and b"scale" in lib.mi355_last_error()
     assert call(kv=_lib.MI355_FP8_E4M3, ks=ptr, D=32) == -1
     assert call(q=None) == -1
+    assert call(nb=0) == -1 and b"num_blocks" in lib.mi355_last_error()
     assert call(max_ctx=100000, ws_bytes=16) == -2 and b"workspace" in lib.mi355_last_error()
 
 

@@ -286,3 +286,32 @@ def test_errors_are_python_exceptions(ops):
     q96 = torch.zeros(1, 2, 8, 96, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ValueError, match="head_dim"):
         ops.flash_attn_prefill(q96, q96, q96)
+
+
+def test_decode_clamps_block_ids_outside_the_pool(ops):
+    """A corrupted block table must not make the kernel read outside the caches: entries outside
+    [0, num_blocks) are clamped (the affected sequence's result is meaningless, the others' are exact)."""
+    print("case: decode bad block ids", flush=True)
+    ctx = [40, 300, 77]
+    q, kc, vc, bt, cl = orc.make_paged_case(batch=3, n_q_heads=8, n_kv_heads=2, head_dim=128, block_size=16,
+                                            context_lens=ctx, pool_factor=1.0, seed=5, dtype=torch.bfloat16)
+    good = ops.paged_attention_decode(q.cuda(), kc.cuda(), vc.cuda(), bt.cuda(), cl.cuda())
+    bad = bt.clone()
+    bad[1, 3] = 2 ** 30
+    bad[1, 5] = -7
+    out = ops.paged_attention_decode(q.cuda(), kc.cuda(), vc.cuda(), bad.cuda(), cl.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(out[0], good[0]) and torch.equal(out[2], good[2])
+    assert torch.isfinite(out[1].float()).all()
+    # what the clamp means: ids above the pool read the last block, negative ids block 0
+    fixed = bt.clone()
+    fixed[1, 3] = kc.shape[0] - 1
+    fixed[1, 5] = 0
+    assert torch.equal(out, ops.paged_attention_decode(q.cuda(), kc.cuda(), vc.cuda(), fixed.cuda(), cl.cuda()))
+
+
+def test_ops_reject_tensors_on_different_devices(ops):
+    print("case: mixed devices", flush=True)
+    q = rnd(1, 2, 16, 64, seed=1).cuda()
+    with pytest.raises(ValueError):
+        ops.flash_attn_prefill(q, q.cpu(), q)
