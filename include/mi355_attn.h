@@ -162,11 +162,12 @@ int mi355_paged_decode_chunk_tokens(int max_ctx);
  * token not cached; NULL slot_mapping: rotate q only... k/v are then ignored).
  * The scatter has no counterpart in the reference (it has no KV cache).
  *   q_in/q_out (T,Hq,D), k_in/v_in (T,Hkv,D) bf16, heads contiguous, token strides in elements;
- *   positions int32 (T), each < context_length; k_cache/v_cache (num_blocks,Hkv,16,D) bf16.
+ *   positions int32 (T), each < context_length (a position outside the table is clamped into it);
+ *   k_cache/v_cache (num_blocks,Hkv,16,D) bf16; a slot outside [0, num_blocks*16) is not written.
  */
 int mi355_rope_and_cache(const void* q_in, const void* k_in, const void* v_in, void* q_out,
                          void* k_cache, void* v_cache, const float* freq_cache,
-                         const int32_t* positions, const int64_t* slot_mapping,
+                         const int32_t* positions, const int64_t* slot_mapping, int64_t num_blocks,
                          int T, int Hq, int Hkv, int D, int context_length,
                          int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
                          int64_t q_out_token_stride, void* stream);

@@ -18,6 +18,7 @@ struct RopeCacheParams {
     const int64_t* slots;         // (T): block * 16 + offset, negative = do not write the cache
     int64_t q_tok, k_tok, v_tok, qo_tok;   // token strides (elements); heads are contiguous (stride D)
     int T, Hq, Hkv, D, ctx_len;
+    int64_t n_slots;               // num_blocks * 16: slots outside [0, n_slots) are not written
 };
 
 // One thread per (token, head slot, pair of adjacent elements).  Head slots: Hq query heads,
@@ -32,8 +33,9 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeCacheParams p) 
         const int i = (int)(idx % half);
         const int hs = (int)((idx / half) % slots_per_tok);
         const int t = (int)(idx / ((int64_t)half * slots_per_tok));
-        const int pos = p.positions[t];
-        const int64_t slot = p.slots ? p.slots[t] : -1;
+        const int pos = min(max(p.positions[t], 0), p.ctx_len - 1);     // a position outside the table is clamped into it
+        int64_t slot = p.slots ? p.slots[t] : -1;
+        if (slot >= p.n_slots) slot = -1;
         if (hs < p.Hq) {
             const uint32_t raw = *reinterpret_cast<const uint32_t*>(p.q_in + t * p.q_tok + (int64_t)hs * p.D + 2 * i);
             const bf16x2 x = __builtin_bit_cast(bf16x2, raw);
@@ -74,7 +76,8 @@ __global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParam
         const int c = (int)(idx % groups);
         const int hs = (int)((idx / groups) % slots_per_tok);
         const int t = (int)(idx / ((int64_t)groups * slots_per_tok));
-        const int64_t slot = p.slots ? p.slots[t] : -1;
+        int64_t slot = p.slots ? p.slots[t] : -1;
+        if (slot >= p.n_slots) slot = -1;
         const bool is_q = hs < p.Hq;
         if (!is_q && slot < 0) continue;
         const bool is_v = hs >= p.Hq + p.Hkv;
@@ -83,7 +86,7 @@ __global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParam
                                  : (is_v ? p.v_in + t * p.v_tok : p.k_in + t * p.k_tok) + (int64_t)hk * p.D;
         u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 8 * c));
         if (!is_v) {
-            const int pos = p.positions[t];
+            const int pos = min(max(p.positions[t], 0), p.ctx_len - 1);
             const f32x4 cs = *reinterpret_cast<const f32x4*>(p.freq + (int64_t)pos * half + 4 * c);
             const f32x4 sn = *reinterpret_cast<const f32x4*>(p.freq + ((int64_t)p.ctx_len + pos) * half + 4 * c);
 #pragma unroll
@@ -150,13 +153,15 @@ using namespace mi355;
 
 extern "C" int mi355_rope_and_cache(const void* q_in, const void* k_in, const void* v_in, void* q_out, void* k_cache,
                                     void* v_cache, const float* freq_cache, const int32_t* positions,
-                                    const int64_t* slot_mapping, int T, int Hq, int Hkv, int D, int context_length,
+                                    const int64_t* slot_mapping, int64_t num_blocks, int T, int Hq, int Hkv, int D,
+                                    int context_length,
                                     int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
                                     int64_t q_out_token_stride, void* stream) {
     if (!q_in || !k_in || !v_in || !q_out || !freq_cache || !positions)
         return set_error(MI355_EINVAL, "rope_and_cache: null pointer argument");
     if (slot_mapping && (!k_cache || !v_cache))
         return set_error(MI355_EINVAL, "rope_and_cache: slot_mapping given without k_cache/v_cache");
+    if (slot_mapping && num_blocks <= 0) return set_error(MI355_EINVAL, "rope_and_cache: num_blocks must be positive");
     if (T < 0 || Hq <= 0 || Hkv <= 0 || context_length <= 0)
         return set_error(MI355_EINVAL, "rope_and_cache: T, Hq, Hkv, context_length out of range");
     if (D <= 0 || (D & 1)) return set_error(MI355_EINVAL, "rope_and_cache: head_dim must be even");
@@ -182,6 +187,7 @@ extern "C" int mi355_rope_and_cache(const void* q_in, const void* k_in, const vo
     p.Hkv = Hkv;
     p.D = D;
     p.ctx_len = context_length;
+    p.n_slots = slot_mapping ? num_blocks * 16 : 0;
     const auto aligned16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
     const bool vec8 = D % 8 == 0 && ((q_token_stride | k_token_stride | v_token_stride | q_out_token_stride) & 7) == 0 &&
                       aligned16(q_in) && aligned16(k_in) && aligned16(v_in) && aligned16(q_out) && aligned16(k_cache) &&

@@ -65,7 +65,7 @@ def load():
     lib.mi355_paged_decode_chunk_tokens.restype = i32
     lib.mi355_paged_decode_chunk_tokens.argtypes = [i32]
     lib.mi355_rope_and_cache.restype = i32
-    lib.mi355_rope_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32,
+    lib.mi355_rope_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32,
                                          i64, i64, i64, i64, vp]
     lib.mi355_quantize_kv_fp8.restype = i32
     lib.mi355_quantize_kv_fp8.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]

@@ -401,7 +401,7 @@ def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, s
             q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
             None if slot_mapping is None else k_cache.data_ptr(), None if slot_mapping is None else v_cache.data_ptr(),
             freq_cache.data_ptr(), positions.data_ptr(), None if slot_mapping is None else slot_mapping.data_ptr(),
-            T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0), stream)
+            0 if slot_mapping is None else k_cache.shape[0], T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0), stream)
     _lib.check(rc, "mi355_rope_and_cache")
     return q_out
 

@@ -75,6 +75,27 @@ def test_rope_and_cache_pair_path_and_out_argument(ops):
         ops.rope_and_cache(q, k, v, pos, fcg, kc_b, vc_b, slots, out=torch.empty(T, Hq, D + 8, dtype=torch.bfloat16, device="cuda"))
 
 
+def test_rope_and_cache_ignores_slots_outside_the_pool_and_clamps_positions(ops):
+    print("case: rope_and_cache bad slots / positions", flush=True)
+    T, Hq, Hkv, D, ctx, nb = 8, 2, 2, 64, 32, 3
+    q, k, v = rnd(T, Hq, D, seed=21).cuda(), rnd(T, Hkv, D, seed=22).cuda(), rnd(T, Hkv, D, seed=23).cuda()
+    fcg = ops.build_rope_cache(ctx, D)
+    pos = torch.tensor([0, 1, 2, 3, 31, 32, 1000, -5], dtype=torch.int32).cuda()
+    slots = torch.tensor([0, 1, nb * 16, 2 ** 40, 5, -1, 47, 46], dtype=torch.int64).cuda()
+    guard = torch.full((nb + 2, Hkv, 16, D), 7.0, dtype=torch.bfloat16, device="cuda")      # pool = blocks 1..nb of this buffer
+    kc, vc = guard[1:nb + 1], guard.clone()[1:nb + 1]
+    q_rot = ops.rope_and_cache(q, k, v, pos, fcg, kc, vc, slots)
+    torch.cuda.synchronize()
+    assert bool((guard[0] == 7).all()) and bool((guard[nb + 1] == 7).all())                  # nothing outside the pool was written
+    written = {0, 1, 5, 47, 46}
+    flat = kc.permute(0, 2, 1, 3).reshape(nb * 16, Hkv, D)
+    for s in range(nb * 16):
+        assert bool((flat[s] == 7).all()) != (s in written)
+    # positions outside the table behave like the nearest valid one
+    pos_ok = torch.tensor([0, 1, 2, 3, 31, 31, 31, 0], dtype=torch.int32).cuda()
+    assert torch.equal(q_rot, ops.rope_and_cache(q, k, v, pos_ok, fcg))
+
+
 @pytest.mark.parametrize("D", [32, 64, 128])
 def test_quantize_kv_fp8_is_bit_exact(ops, D):
     print(f"case: quantize D={D}", flush=True)
