@@ -340,8 +340,8 @@ def main():
                     help="only run the 1 GiB plain copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the path needs no exchange between GPUs; "
-              "see DESIGN.md for how it would shard). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this build measures one GPU only (attention needs no exchange between GPUs: it shards "
+              "by sequences or by kv heads, one process per GPU). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch
