@@ -99,17 +99,16 @@ int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out
  *                                    (dq like q, dk/dv like k/v, dout like out), each with its own strides
  *   lse   : as written by mi355_prefill_fwd_lse for the same inputs
  *   delta : fp32 scratch with lse's layout and size (receives rowsum(dout * out))
- *   total_q : rows of the packed query buffer (packed layout only; ignored for dense)
  * GQA: dk/dv of a kv head sum over its Hq/Hkv query heads.  Mask modes NONE / CAUSAL.
  * A causal query row that sees no key (Sq > Sk) gets dq = 0.  Three launches on `stream`
- * (delta, dk/dv, dq); no atomics, so the result is deterministic.
+ * (dv; dq, which also fills delta; dk); no atomics, so the result is deterministic.
  */
 int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout,
                       const float* lse, float* delta, void* dq, void* dk, void* dv,
                       const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
                       const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
                       const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[2],
-                      const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t total_q,
+                      const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
                       int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
                       float softmax_scale, int mask_mode, int dtype, void* stream);
 

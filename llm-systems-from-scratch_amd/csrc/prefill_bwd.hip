@@ -1,7 +1,7 @@
 // FlashAttention-style prefill backward for gfx950 (bf16, MFMA 32x32x16): dQ, dK, dV from
 // q, k, v, out, dout and the forward's log-sum-exp.  No atomics; results are deterministic.
 //
-//   delta_i = sum_d dO[i,d] * O[i,d]                       (bwd_delta_kernel)
+//   delta_i = sum_d dO[i,d] * O[i,d]                       (computed, and stored, by the dQ kernel)
 //   P_ij    = exp(scale * q_i.k_j - lse_i)                 (recomputed, never stored)
 //   dV_j    = sum_i P_ij dO_i
 //   dP_ij   = dO_i . v_j
@@ -25,7 +25,9 @@
 namespace mi355 {
 
 constexpr int kBwWaves = 4;
-constexpr int kBwCols = 32 * kBwWaves;   // columns (queries or keys) per workgroup
+constexpr int kBwCols = 32 * kBwWaves;   // query columns per workgroup of the dQ kernel
+constexpr int kBwKvWaves = 8;            // dK/dV kernels: 8 wavefronts = 256 key columns share every streamed Q/dO tile
+constexpr int kBwKvCols = 32 * kBwKvWaves;
 constexpr int kBwRows = 64;              // rows of a streamed LDS tile
 
 struct BwdParams {
@@ -50,12 +52,15 @@ struct BwdParams {
 
 // Loader of a 64-row tile (rows of D bf16, row stride `stride` elements) into swizzled LDS:
 // wavefront w, instruction j covers LDS chunks (w*NI + j)*64 .. +63; rows past `last` re-read row `last`.
-template <int D>
+template <int D, int NW>
 struct TileLoader {
     static constexpr int CPR = D / 8;
-    static constexpr int NI = kBwRows * CPR / 64 / kBwWaves;
+    static constexpr int TOTAL = kBwRows * CPR / 64;            // 1 KiB instructions per tile
+    static constexpr int NI = (TOTAL + NW - 1) / NW;            // per wavefront (the last wavefronts may have none)
     int row[NI], col[NI];
+    bool active;
     __device__ __forceinline__ void init(int wave, int lane) {
+        active = wave * NI < TOTAL;
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
             const int idx = (wave * NI + j) * 64 + lane;
@@ -64,44 +69,12 @@ struct TileLoader {
         }
     }
     __device__ __forceinline__ void issue(const __bf16* first_row, int stride, int last, uint32_t lds_wave_base) const {
+        if (!active) return;
 #pragma unroll
         for (int j = 0; j < NI; ++j)
             dma_to_lds_16(first_row, (uint32_t)(min(row[j], last) * stride * 2 + col[j]), lds_wave_base + j * 1024);
     }
 };
-
-// ---------------------------------------------------------------------------------------------
-// delta = rowsum(dO * O): 16 lanes per (row, head), 8 elements per lane and step.
-template <int D>
-__global__ __launch_bounds__(256) void bwd_delta_kernel(BwdParams p, int64_t total_rows) {
-    const int sub = threadIdx.x & 15;
-    const int64_t item = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;      // (b, h, i) flattened, i fastest
-    if (item >= total_rows * p.Hq) return;
-    const int h = (int)((item / total_rows) % p.Hq);
-    const int64_t r = item % total_rows;                                     // row inside the batch element / packed buffer
-    int64_t o_off, do_off, l_off;
-    if (p.cu_q) {
-        o_off = r * p.os[2] + (int64_t)h * p.os[1];
-        do_off = r * p.dos[2] + (int64_t)h * p.dos[1];
-        l_off = r + (int64_t)h * p.ls[1];
-    } else {
-        const int64_t b = r / p.Sq, i = r % p.Sq;
-        o_off = b * p.os[0] + (int64_t)h * p.os[1] + i * p.os[2];
-        do_off = b * p.dos[0] + (int64_t)h * p.dos[1] + i * p.dos[2];
-        l_off = b * p.ls[0] + (int64_t)h * p.ls[1] + i;
-    }
-    float acc = 0.f;
-#pragma unroll
-    for (int c = sub; c < D / 8; c += 16) {
-        const bf16x8 a = as_bf16x8(*reinterpret_cast<const u32x4*>(p.out + o_off + 8 * c));
-        const bf16x8 g = as_bf16x8(*reinterpret_cast<const u32x4*>(p.dout + do_off + 8 * c));
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)g[e];
-    }
-#pragma unroll
-    for (int off = 8; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (sub == 0) p.delta[l_off] = acc;
-}
 
 // Per-lane LDS offsets of the two read patterns of a swizzled 64 x D tile.
 template <int D>
@@ -131,6 +104,7 @@ struct TileReads {
 // Per wavefront: Q and dO fragments of its 32 query columns in registers (64), dQ^T accumulators (64).
 template <int D, bool CAUSAL>
 __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
+    constexpr int NWV = kBwWaves;
     using R = TileReads<D>;
     constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
     // [K buffer 0][K buffer 1][V buffer 0][V buffer 1]
@@ -150,11 +124,12 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
     const int b = lid / (n_pairs * p.Hq);
     const int hk = h / (p.Hq / p.Hkv);
     int sq, sk;
-    int64_t q_base, k_base, v_base, do_base, dq_base, l_base;
+    int64_t q_base, k_base, v_base, do_base, dq_base, l_base, o_base;
     if (p.cu_q) {
         const int q_start = p.cu_q[b], k_start = p.cu_k[b];
         sq = p.cu_q[b + 1] - q_start;
         sk = p.cu_k[b + 1] - k_start;
+        o_base = (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
         q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
         do_base = (int64_t)q_start * p.dos[2] + (int64_t)h * p.dos[1];
         dq_base = (int64_t)q_start * p.dqs[2] + (int64_t)h * p.dqs[1];
@@ -164,6 +139,7 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
     } else {
         sq = p.Sq;
         sk = p.Sk;
+        o_base = (int64_t)b * p.os[0] + (int64_t)h * p.os[1];
         q_base = (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
         do_base = (int64_t)b * p.dos[0] + (int64_t)h * p.dos[1];
         dq_base = (int64_t)b * p.dqs[0] + (int64_t)h * p.dqs[1];
@@ -179,11 +155,11 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
     const int n = lane & 31, kg = lane >> 5;
     const int coff = sk - sq;
 
-    TileLoader<D> ld;
+    TileLoader<D, NWV> ld;
     ld.init(wave, lane);
     R rd;
     rd.init(lane);
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D>::NI * 1024);
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D, NWV>::NI * 1024);
 
     for (int half = 0; half < 2; ++half) {
         const int qtile = half == 0 ? nq - 1 - pair : pair;
@@ -208,7 +184,19 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
         }
         // a padded query column gets lse = +inf, i.e. P = 0 everywhere
         const float lse2 = q_ok ? p.lse[l_base + qi] * kLog2e : INFINITY;
-        const float delta = q_ok ? p.delta[l_base + qi] : 0.f;
+        // delta = rowsum(dO * O) of this lane's query: each lane of the pair (kg = 0, 1) covers half of d.
+        // It is also written out: the dK kernel, launched after this one, reads it per row.
+        float delta = 0.f;
+        if (q_ok) {
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const bf16x8 o8 = as_bf16x8(*reinterpret_cast<const u32x4*>(p.out + o_base + (int64_t)qi * p.os[2] + 16 * s + 8 * kg));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) delta += (float)o8[e] * (float)dof[s][e];
+            }
+        }
+        delta = xor32_sum(delta);
+        if (q_ok && kg == 0) p.delta[l_base + qi] = delta;
 
         f32x16 dq[NDT];
 #pragma unroll
@@ -307,7 +295,9 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
 // one kernel that holds both accumulators keep each under 256 registers, i.e. two wavefronts per SIMD.
 // Per wavefront: K (and, for dK, V) fragments of its 32 key columns in registers, one accumulator set (64).
 template <int D, bool CAUSAL, bool WANT_DK>
-__global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dkv_kernel(BwdParams p) {
+__global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p) {
+    constexpr int NWV = kBwKvWaves;
+    constexpr int kCols = 32 * NWV;                                 // keys per workgroup
     using R = TileReads<D>;
     constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
     // [Q buffer 0][Q buffer 1][dO buffer 0][dO buffer 1]
@@ -343,7 +333,7 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dkv_kernel(BwdParams p) 
         v_base = (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
         o_base = WANT_DK ? (int64_t)b * p.dks[0] + (int64_t)hk * p.dks[1] : (int64_t)b * p.dvs[0] + (int64_t)hk * p.dvs[1];
     }
-    const int nk = (sk + kBwCols - 1) / kBwCols;
+    const int nk = (sk + kCols - 1) / kCols;
     if (sq <= 0 || 2 * pair >= nk) return;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -351,16 +341,16 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dkv_kernel(BwdParams p) 
     const int n = lane & 31, kg = lane >> 5;
     const int coff = sk - sq;
 
-    TileLoader<D> ld;
+    TileLoader<D, NWV> ld;
     ld.init(wave, lane);
     R rd;
     rd.init(lane);
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D>::NI * 1024);
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D, NWV>::NI * 1024);
 
     for (int half = 0; half < 2; ++half) {
         const int ktile = half == 0 ? pair : nk - 1 - pair;
         if (half == 1 && ktile == pair) break;                          // odd tile count: the middle tile has no partner
-        const int k0 = ktile * kBwCols;
+        const int k0 = ktile * kCols;
         const int kw0 = k0 + 32 * wave;
         const int kj = kw0 + n;
         const bool k_ok = kj < sk;
@@ -522,20 +512,17 @@ __global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dkv_kernel(BwdParams p) 
 }
 
 template <int D>
-static int launch_bwd(const BwdParams& p, bool causal, int64_t total_rows, hipStream_t stream) {
-    const int64_t delta_threads = total_rows * p.Hq * 16;
-    hipLaunchKernelGGL((bwd_delta_kernel<D>), dim3((unsigned)((delta_threads + 255) / 256)), dim3(256), 0, stream, p,
-                       total_rows);
-    const dim3 block(kBwWaves * 64);
+static int launch_bwd(const BwdParams& p, bool causal, hipStream_t stream) {
+    const dim3 block(kBwWaves * 64), block_kv(kBwKvWaves * 64);
     const dim3 grid_q((unsigned)((p.n_qtiles + 1) / 2 * p.Hq * p.B)), grid_k((unsigned)((p.n_ktiles + 1) / 2 * p.Hkv * p.B));
     if (causal) {
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, true, false>), grid_k, block, 0, stream, p);
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, true, true>), grid_k, block, 0, stream, p);
-        hipLaunchKernelGGL((bwd_dq_kernel<D, true>), grid_q, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, true, false>), grid_k, block_kv, 0, stream, p);     // dV
+        hipLaunchKernelGGL((bwd_dq_kernel<D, true>), grid_q, block, 0, stream, p);                // dQ, writes delta
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, true, true>), grid_k, block_kv, 0, stream, p);      // dK, reads delta
     } else {
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, false, false>), grid_k, block, 0, stream, p);
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, false, true>), grid_k, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, false, false>), grid_k, block_kv, 0, stream, p);
         hipLaunchKernelGGL((bwd_dq_kernel<D, false>), grid_q, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, false, true>), grid_k, block_kv, 0, stream, p);
     }
     return (int)hipGetLastError();
 }
@@ -549,7 +536,7 @@ extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, co
                                  const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
                                  const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
                                  const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[2],
-                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t total_q, int B, int Hq,
+                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int B, int Hq,
                                  int Hkv, int Sq_max, int Sk_max, int D, float softmax_scale, int mask_mode, int dtype,
                                  void* stream) {
     if (!q || !k || !v || !out || !dout || !lse || !delta || !dq || !dk || !dv)
@@ -566,7 +553,6 @@ extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, co
         return set_error(MI355_EINVAL, "prefill_bwd: cu_seqlens_q and cu_seqlens_k must be given together");
     if (mask_mode != MI355_MASK_NONE && mask_mode != MI355_MASK_CAUSAL)
         return set_error(MI355_EINVAL, "prefill_bwd: mask_mode must be MI355_MASK_NONE or MI355_MASK_CAUSAL");
-    if (cu_seqlens_q && total_q <= 0) return set_error(MI355_EINVAL, "prefill_bwd: total_q must be positive (packed layout)");
     const int64_t* all[8] = {q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides};
     for (const int64_t* st : all)
         for (int i = 0; i < 3; ++i)
@@ -612,16 +598,14 @@ extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, co
     p.scale = softmax_scale;
     p.scale_log2 = softmax_scale * kLog2e;
     p.n_qtiles = (Sq_max + kBwCols - 1) / kBwCols;
-    p.n_ktiles = (Sk_max + kBwCols - 1) / kBwCols;
+    p.n_ktiles = (Sk_max + kBwKvCols - 1) / kBwKvCols;
     if ((int64_t)p.n_qtiles * Hq * B > 0x7fffffffLL || (int64_t)p.n_ktiles * Hkv * B > 0x7fffffffLL)
         return set_error(MI355_EINVAL, "prefill_bwd: too many workgroups");
-    const int64_t total_rows = cu_seqlens_q ? total_q : (int64_t)B * Sq_max;
-    if (total_rows * Hq * 16 / 256 > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill_bwd: too many rows");
 
     hipStream_t s = (hipStream_t)stream;
     const bool causal = mask_mode == MI355_MASK_CAUSAL;
-    int rc = D == 128 ? launch_bwd<128>(p, causal, total_rows, s)
-                      : (D == 64 ? launch_bwd<64>(p, causal, total_rows, s) : launch_bwd<32>(p, causal, total_rows, s));
+    int rc = D == 128 ? launch_bwd<128>(p, causal, s)
+                      : (D == 64 ? launch_bwd<64>(p, causal, s) : launch_bwd<32>(p, causal, s));
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;
 }

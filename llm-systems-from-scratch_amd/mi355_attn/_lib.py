@@ -55,7 +55,7 @@ def load():
     lib.mi355_prefill_fwd_lse.argtypes = [vp, vp, vp, vp, vp, _i64x3, _i64x3, _i64x3, _i64x3, _i64x2, vp, vp,
                                           i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
     lib.mi355_prefill_bwd.restype = i32
-    lib.mi355_prefill_bwd.argtypes = [vp] * 10 + [_i64x3] * 8 + [_i64x2, vp, vp, i64,
+    lib.mi355_prefill_bwd.argtypes = [vp] * 10 + [_i64x3] * 8 + [_i64x2, vp, vp,
                                                                  i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
     lib.mi355_paged_decode_fwd.restype = i32
     lib.mi355_paged_decode_fwd.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, sz,

@@ -127,17 +127,17 @@ def _prefill_backward(q, k, v, out, dout, lse, cu_q, cu_k, Sq, Sk, scale, mode):
         return dq.zero_(), dk.zero_(), dv.zero_()
     delta = torch.empty_like(lse)
     if packed:
-        B, (T, Hq, D), Hkv = cu_q.numel() - 1, q.shape, k.shape[1]
+        B, (_, Hq, D), Hkv = cu_q.numel() - 1, q.shape, k.shape[1]
         ls = (0, lse.stride(0))
     else:
-        (B, Hq, _, D), Hkv, T = q.shape, k.shape[1], 0
+        (B, Hq, _, D), Hkv = q.shape, k.shape[1]
         ls = lse.stride()[:2]
     st = [_lib.strides3(_packed_or_dense_strides(t, packed)) for t in (q, k, v, out, dout, dq, dk, dv)]
     with _on(q, k, v, out, dout, lse, cu_q, cu_k) as stream:
         rc = _lib.load().mi355_prefill_bwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), *st, _lib.strides2(ls),
-            None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(), T,
+            None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(),
             B, Hq, Hkv, int(Sq), int(Sk), D, float(scale), mode, _lib.MI355_BF16, stream)
     _lib.check(rc, "mi355_prefill_bwd")
     return dq, dk, dv
