@@ -24,8 +24,8 @@
 
 namespace mi355 {
 
-constexpr int kBwWaves = 4;
-constexpr int kBwCols = 32 * kBwWaves;   // query columns per workgroup of the dQ kernel
+constexpr int kBwWaves = 8;
+constexpr int kBwCols = 32 * kBwWaves;   // query columns per workgroup of the dQ kernel (one workgroup of 8 wavefronts per CU)
 constexpr int kBwKvWaves = 8;            // dK/dV kernels: 8 wavefronts = 256 key columns share every streamed Q/dO tile
 constexpr int kBwKvCols = 32 * kBwKvWaves;
 constexpr int kBwRows = 64;              // rows of a streamed LDS tile
@@ -103,7 +103,7 @@ struct TileReads {
 // dQ: one workgroup per tile of 128 queries of one (batch, query head); K/V stream through LDS.
 // Per wavefront: Q and dO fragments of its 32 query columns in registers (64), dQ^T accumulators (64).
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(kBwWaves * 64, 2) void bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
     constexpr int NWV = kBwWaves;
     using R = TileReads<D>;
     constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
