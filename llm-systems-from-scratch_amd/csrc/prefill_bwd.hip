@@ -380,8 +380,9 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
         if (CAUSAL) first_tile = max(0, k0 - coff) / kBwRows;
         const int n_tiles = (sq + kBwRows - 1) / kBwRows;
         // The (query head, row tile) pairs of the GQA group form one stream of steps through the two LDS buffers.
-        // Row tiles are walked from the LAST one down: every key tile needs the last rows, so the workgroups of
-        // one (batch, kv head) start on the same Q/dO tiles and share them through the XCD's L2.
+        // Row tiles are walked from the LAST one down, the query heads of the group innermost: every key tile
+        // needs the last rows, so the workgroups of one (batch, kv head) walk the same Q/dO tiles at the same
+        // time and share them through the XCD's L2.
         const int tiles_per_head = max(0, n_tiles - first_tile);
         const int n_steps = G * tiles_per_head;
 
@@ -390,8 +391,8 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
         // so that waiting for them never sits in front of it.
         float pend_lse = 0.f, pend_delta = 0.f;
         const auto issue = [&](int st) {
-            const int h = hk * G + st / tiles_per_head;
-            const int r0 = (n_tiles - 1 - st % tiles_per_head) * kBwRows, buf = (st & 1) * kTile;
+            const int h = hk * G + st % G;
+            const int r0 = (n_tiles - 1 - st / G) * kBwRows, buf = (st & 1) * kTile;
             int64_t q_base, do_base, l_base;
             if (p.cu_q) {
                 q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
@@ -482,7 +483,7 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
         }
         for (int st = 0; st < n_steps; ++st) {
             const bool more = st + 1 < n_steps;
-            const int r0 = (n_tiles - 1 - st % tiles_per_head) * kBwRows;
+            const int r0 = (n_tiles - 1 - st / G) * kBwRows;
             wait_vmcnt<0>();                                   // this wavefront's share of the step's tiles has landed
             __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
             if (more) issue(st + 1);
