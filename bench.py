@@ -161,7 +161,26 @@ def bench_producers(args):
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS,
                      "device_ms": dev_ms, "traffic": _traffic("rope_and_cache")},
     }
-    del q, k, v, q_out, k_cache, v_cache
+    del k_cache, v_cache
+    # --- rope_and_cache_fp8: the same tokens into an fp8 pool with per-(block, kv head) scales (two launches:
+    # queries, then keys/values; 16 tokens per block arrive together, so no row is re-expressed)
+    k8 = torch.zeros(n_blocks, Hkv, 16, D, dtype=torch.uint8, device=dev)
+    v8 = torch.zeros_like(k8)
+    ks = torch.ones(n_blocks, Hkv, dtype=torch.float32, device=dev)
+    vs = torch.ones_like(ks)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.rope_and_cache_fp8(q, k, v, pos, freq, k8, v8, ks, vs, slots, out=q_out),
+                            args.steps, args.warmup)
+    nbytes = 2 * q.numel() * 2 + (k.numel() + v.numel()) * 3 + 2 * ks.numel() * 4 + T * 12 + freq.numel() * 4
+    res["rope_and_cache_fp8"] = {
+        "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 -> fp8-e4m3 (fp32 rotation)",
+        "config": {"workload": "RoPE + quantising write into an fp8 paged cache of configs[2]'s 32768 packed tokens "
+                               "(32 q / 8 kv heads, head_dim 128), blocks a random permutation", "algorithmic_bytes": nbytes},
+        "roofline": {"bound": "hbm", "kernel": "rope_and_cache_vec8_kernel + rope_and_cache_fp8_kernel",
+                     "achieved": nbytes / dev_ms / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS, "device_ms": dev_ms,
+                     "traffic": _traffic("rope_and_cache_fp8")},
+    }
+    del q, k, v, q_out, k8, v8
     # --- quantize_kv_fp8: a pool of configs[4]'s size (about 103k blocks x 8 kv heads x 16 x 128)
     nb = 103_000
     pool = torch.randn(nb, Hkv, 16, D, device=dev, generator=g).to(torch.bfloat16)

@@ -181,6 +181,28 @@ int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, float* scale,
                           int64_t num_blocks, int Hkv, int D, int block_size, void* stream);
 
 /*
+ * mi355_rope_and_cache with an fp8-e4m3 cache (the MI355_FP8_E4M3 format of
+ * mi355_paged_decode_fwd): RoPE as in llm-core/llm_core/model.py:93-104, then the rotated keys
+ * (rounded to bf16 first, as a bf16 cache would hold them) and the values are quantised into
+ * k_cache_fp8 / v_cache_fp8 (num_blocks,Hkv,16,D) bytes, and k_scale / v_scale (num_blocks,Hkv)
+ * fp32 are maintained so that a block's scale is always absmax/448 of its valid rows: writing
+ * at offset 0 starts the block afresh; writing at a later offset keeps the scale or, when the new
+ * rows raise it, re-expresses the rows already there in the new scale (fp8 -> fp32 -> fp8).
+ * Tokens that share a block must be adjacent in the packed order with consecutive slots (a run),
+ * and a block may receive one run per call (one sequence = one run per block, as a prefill or a
+ * decode step produces them).  Slots outside [0, 16*num_blocks) are skipped.  Needs 16-byte
+ * aligned tensors, token strides that are multiples of 8, D in {32, 64, 128}.  No reference
+ * counterpart (the reference has no KV cache).
+ */
+int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, const void* v_in, void* q_out,
+                             void* k_cache_fp8, void* v_cache_fp8, float* k_scale, float* v_scale,
+                             const float* freq_cache, const int32_t* positions,
+                             const int64_t* slot_mapping, int64_t num_blocks,
+                             int T, int Hq, int Hkv, int D, int context_length,
+                             int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
+                             int64_t q_out_token_stride, void* stream);
+
+/*
  * RMSNorm forward over the rows of a (n_rows, n_cols) bf16 matrix:
  *   y = weight * (h * rsqrt(mean(h^2) + eps)),  h = x, or h = bf16(x + residual)
  * fp32 math, one rounding to bf16 -- RMSNorm.forward, llm-core/llm_core/model.py:60-67, and the

@@ -147,6 +147,157 @@ __global__ __launch_bounds__(256) void quantize_kv_fp8_kernel(const __bf16* __re
     }
 }
 
+
+// ---- fused RoPE + write into an fp8 cache with per-(block, kv head) scales ------------------
+struct RopeCacheFp8Params {
+    const __bf16* k_in;
+    const __bf16* v_in;
+    unsigned char* k_cache;
+    unsigned char* v_cache;
+    float* k_scale;
+    float* v_scale;
+    const float* freq;
+    const int32_t* positions;
+    const int64_t* slots;
+    int64_t k_tok, v_tok;
+    int T, Hkv, ctx_len;
+    int64_t n_slots;
+};
+
+__device__ __forceinline__ void quantize8(const float (&x)[8], float sc, unsigned char* dst) {
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = fminf(fmaxf(x[e] / sc, -448.0f), 448.0f);
+    int w0 = 0, w1 = 0;
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], w0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], w1, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+    u32x2 out;
+    out[0] = (uint32_t)w0;
+    out[1] = (uint32_t)w1;
+    *reinterpret_cast<u32x2*>(dst) = out;
+}
+
+// One wavefront per (window of `win` consecutive tokens, kv head, K or V).  A RUN is a stretch of
+// consecutive tokens whose slots are consecutive inside one cache block; the wavefront writes every
+// run that STARTS in its window, whole (at most 16 rows), so exactly one wavefront touches a
+// (block, head) slab:
+//   scale' = max(scale of the rows already in the block, absmax(new rows) / 448)
+//   rows already in the block are re-expressed in scale' when it grew (fp8 -> fp32 -> fp8)
+//   new rows (keys rotated and rounded to bf16 first, as the bf16 cache would hold them) -> e4m3
+// The scale therefore always equals absmax/448 of the block's valid rows, as in quantize_kv_fp8_kernel.
+// A lane owns 8 adjacent elements of one row: D/8 lanes per row, 512/D rows per pass.
+// win = 16 for a packed prefill (one run per window when sequences start at block boundaries),
+// win = 1 for a decode step (every token is its own run; all of them proceed in parallel).
+template <int D>
+__global__ __launch_bounds__(256) void rope_and_cache_fp8_kernel(RopeCacheFp8Params p, int win, int n_windows) {
+    constexpr int LPR = D / 8, RPP = 64 / LPR, NP = 16 / RPP;
+    const int lane = threadIdx.x & 63;
+    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (w >= (int64_t)n_windows * 2 * p.Hkv) return;
+    const int window = (int)(w / (2 * p.Hkv));
+    const int rem = (int)(w % (2 * p.Hkv));
+    const bool is_v = rem >= p.Hkv;
+    const int hk = is_v ? rem - p.Hkv : rem;
+    const int c = lane % LPR, rip = lane / LPR;
+    const int half = D / 2;
+    // Lane i holds the slot of token base - 1 + i: lane 0 the token before the window, lanes 1..win the
+    // window, then 15 tokens of look-ahead (a run that starts in the window may end beyond it).
+    const int base = window * win;
+    const int64_t tok_i = (int64_t)base - 1 + lane;
+    int64_t my_slot = -1;
+    if (lane < win + 16 && tok_i >= 0 && tok_i < p.T) my_slot = p.slots[tok_i];
+    if (my_slot >= p.n_slots) my_slot = -1;
+    const int64_t prev_slot = __shfl_up(my_slot, 1, 64);
+    // a token continues the run of the token before it when both sit in the same block at consecutive offsets
+    const bool cont = lane >= 1 && my_slot >= 0 && (my_slot & 15) != 0 && prev_slot == my_slot - 1;
+    const uint64_t cont_mask = __builtin_amdgcn_ballot_w64(cont);
+    uint64_t head_mask = __builtin_amdgcn_ballot_w64(lane >= 1 && lane <= win && my_slot >= 0 && !cont);
+    while (head_mask != 0) {
+        const int h = __builtin_ctzll(head_mask);
+        head_mask &= head_mask - 1;
+        const int t = base - 1 + h;
+        const int64_t slot = __shfl(my_slot, h, 64);
+        const int off0 = (int)(slot & 15);
+        const int n = 1 + __builtin_ctzll(~(cont_mask >> (h + 1)));       // tokens of the run (at most 16 - off0)
+
+        const int64_t slab = (slot >> 4) * p.Hkv + hk;
+        unsigned char* cache = (is_v ? p.v_cache : p.k_cache) + slab * (16 * D);
+        float* scale = (is_v ? p.v_scale : p.k_scale) + slab;
+
+        float val[NP][8];
+        float amax = 0.f;
+#pragma unroll
+        for (int pi = 0; pi < NP; ++pi) {
+            const int j = pi * RPP + rip;                 // row of the block
+#pragma unroll
+            for (int e = 0; e < 8; ++e) val[pi][e] = 0.f;
+            if (j >= off0 && j < off0 + n) {
+                const int tok = t + j - off0;
+                const __bf16* src = (is_v ? p.v_in + tok * p.v_tok : p.k_in + tok * p.k_tok) + (int64_t)hk * D + 8 * c;
+                u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src));
+                if (!is_v) {
+                    const int pos = min(max(p.positions[tok], 0), p.ctx_len - 1);
+                    const f32x4 cs = *reinterpret_cast<const f32x4*>(p.freq + (int64_t)pos * half + 4 * c);
+                    const f32x4 sn = *reinterpret_cast<const f32x4*>(p.freq + ((int64_t)p.ctx_len + pos) * half + 4 * c);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t wd = raw[q];
+                        const bf16x2 x = __builtin_bit_cast(bf16x2, wd);
+                        const float x1 = (float)x[0], x2 = (float)x[1];
+                        raw[q] = pack_bf16(cs[q] * x1 - sn[q] * x2, sn[q] * x1 + cs[q] * x2);
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint32_t wd = raw[q];
+                    const bf16x2 x = __builtin_bit_cast(bf16x2, wd);
+                    val[pi][2 * q] = (float)x[0];
+                    val[pi][2 * q + 1] = (float)x[1];
+                    amax = fmaxf(amax, fmaxf(fabsf(val[pi][2 * q]), fabsf(val[pi][2 * q + 1])));
+                }
+            }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+
+        float sc;
+        if (off0 == 0) {
+            sc = amax > 0.f ? amax / 448.0f : 1.0f;      // a fresh block: whatever the slab held is dead
+        } else {
+            const float old = *scale;
+            sc = fmaxf(old, amax / 448.0f);
+            if (sc != old) {
+#pragma unroll
+                for (int pi = 0; pi < NP; ++pi) {
+                    const int j = pi * RPP + rip;
+                    if (j < off0) {
+                        unsigned char* row = cache + j * D + 8 * c;
+                        const u32x2 raw = *reinterpret_cast<const u32x2*>(row);
+                        const u32x2 lo = fp8x4_to_bf16x4(raw[0]), hi = fp8x4_to_bf16x4(raw[1]);
+                        const uint32_t wd[4] = {lo[0], lo[1], hi[0], hi[1]};
+                        float x[8];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const bf16x2 b = __builtin_bit_cast(bf16x2, wd[q]);
+                            x[2 * q] = (float)b[0] * old;
+                            x[2 * q + 1] = (float)b[1] * old;
+                        }
+                        quantize8(x, sc, row);
+                    }
+                }
+            }
+        }
+        if (lane == 0) *scale = sc;
+#pragma unroll
+        for (int pi = 0; pi < NP; ++pi) {
+            const int j = pi * RPP + rip;
+            if (j >= off0 && j < off0 + n) quantize8(val[pi], sc, cache + j * D + 8 * c);
+        }
+    }
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -224,6 +375,85 @@ extern "C" int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, fl
     else
         hipLaunchKernelGGL(quantize_kv_fp8_kernel<32>, dim3(grid), dim3(256), 0, s, (const __bf16*)cache_bf16,
                            (unsigned char*)cache_fp8, scale, n_slabs);
+    const int rc = (int)hipGetLastError();
+    if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
+}
+
+
+extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, const void* v_in, void* q_out,
+                                        void* k_cache_fp8, void* v_cache_fp8, float* k_scale, float* v_scale,
+                                        const float* freq_cache, const int32_t* positions, const int64_t* slot_mapping,
+                                        int64_t num_blocks, int T, int Hq, int Hkv, int D, int context_length,
+                                        int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
+                                        int64_t q_out_token_stride, void* stream) {
+    if (!q_in || !k_in || !v_in || !q_out || !freq_cache || !positions || !slot_mapping || !k_cache_fp8 || !v_cache_fp8 ||
+        !k_scale || !v_scale)
+        return set_error(MI355_EINVAL, "rope_and_cache_fp8: null pointer argument");
+    if (num_blocks <= 0) return set_error(MI355_EINVAL, "rope_and_cache_fp8: num_blocks must be positive");
+    if (T < 0 || Hq <= 0 || Hkv <= 0 || context_length <= 0)
+        return set_error(MI355_EINVAL, "rope_and_cache_fp8: T, Hq, Hkv, context_length out of range");
+    if (!(D == 32 || D == 64 || D == 128)) return set_error(MI355_EINVAL, "rope_and_cache_fp8: head_dim must be 32, 64 or 128");
+    const auto aligned16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+    if (((q_token_stride | k_token_stride | v_token_stride | q_out_token_stride) & 7) != 0 || !aligned16(q_in) ||
+        !aligned16(k_in) || !aligned16(v_in) || !aligned16(q_out) || !aligned16(k_cache_fp8) || !aligned16(v_cache_fp8) ||
+        !aligned16(freq_cache))
+        return set_error(MI355_EINVAL, "rope_and_cache_fp8: tensors must be 16-byte aligned with token strides that are multiples of 8");
+    if (T == 0) return MI355_OK;
+    hipStream_t s = (hipStream_t)stream;
+    // queries: the bf16 kernel with no key/value heads rotates q_in into q_out and touches nothing else
+    RopeCacheParams pq{};
+    pq.q_in = (const __bf16*)q_in;
+    pq.k_in = (const __bf16*)k_in;
+    pq.v_in = (const __bf16*)v_in;
+    pq.q_out = (__bf16*)q_out;
+    pq.freq = freq_cache;
+    pq.positions = positions;
+    pq.slots = nullptr;
+    pq.q_tok = q_token_stride;
+    pq.k_tok = k_token_stride;
+    pq.v_tok = v_token_stride;
+    pq.qo_tok = q_out_token_stride;
+    pq.T = T;
+    pq.Hq = Hq;
+    pq.Hkv = 0;
+    pq.D = D;
+    pq.ctx_len = context_length;
+    pq.n_slots = 0;
+    {
+        const int64_t total = (int64_t)T * Hq * (D / 8);
+        const int64_t blocks = (total + 255) / 256;
+        const unsigned grid = (unsigned)(blocks < 256 * 64 ? blocks : 256 * 64);
+        hipLaunchKernelGGL(rope_and_cache_vec8_kernel, dim3(grid), dim3(256), 0, s, pq);
+    }
+    RopeCacheFp8Params p;
+    p.k_in = (const __bf16*)k_in;
+    p.v_in = (const __bf16*)v_in;
+    p.k_cache = (unsigned char*)k_cache_fp8;
+    p.v_cache = (unsigned char*)v_cache_fp8;
+    p.k_scale = k_scale;
+    p.v_scale = v_scale;
+    p.freq = freq_cache;
+    p.positions = positions;
+    p.slots = slot_mapping;
+    p.k_tok = k_token_stride;
+    p.v_tok = v_token_stride;
+    p.T = T;
+    p.Hkv = Hkv;
+    p.ctx_len = context_length;
+    p.n_slots = num_blocks * 16;
+    // a decode step (few tokens, each its own run) spreads one token per wavefront; a packed prefill
+    // gives every wavefront a window of 16 tokens, which holds one run when sequences start on block boundaries
+    const int win = T >= 4096 ? 16 : 1;
+    const int n_windows = (T + win - 1) / win;
+    const int64_t wgs = ((int64_t)n_windows * 2 * Hkv + 3) / 4;
+    if (wgs > 0x7fffffff) return set_error(MI355_EINVAL, "rope_and_cache_fp8: too many tokens for one launch");
+    if (D == 128)
+        hipLaunchKernelGGL(rope_and_cache_fp8_kernel<128>, dim3((unsigned)wgs), dim3(256), 0, s, p, win, n_windows);
+    else if (D == 64)
+        hipLaunchKernelGGL(rope_and_cache_fp8_kernel<64>, dim3((unsigned)wgs), dim3(256), 0, s, p, win, n_windows);
+    else
+        hipLaunchKernelGGL(rope_and_cache_fp8_kernel<32>, dim3((unsigned)wgs), dim3(256), 0, s, p, win, n_windows);
     const int rc = (int)hipGetLastError();
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;

@@ -9,6 +9,7 @@ llm-core/llm_core/model.py:308-325 and the SDPA slot at model.py:382):
     paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, ...)
     rope_and_cache(q, k, v, positions, freq_cache, k_cache, v_cache, slot_mapping)   # cache producer
     quantize_kv_cache_fp8(cache)
+    rope_and_cache_fp8(q, k, v, positions, freq_cache, k_cache8, v_cache8, k_scale, v_scale, slot_mapping)
     rms_norm(x, weight, eps, residual=None)             # RMSNorm.forward / TritonRMSNorm forward
     silu_mul(gate, up)                                  # fused kernel of FusedSwiGLU
 
@@ -19,6 +20,7 @@ from .ops import (  # noqa: F401
     quantize_kv_cache_fp8,
     rms_norm,
     rope_and_cache,
+    rope_and_cache_fp8,
     silu_mul,
     flash_attn_prefill,
     flash_attn_varlen_prefill,

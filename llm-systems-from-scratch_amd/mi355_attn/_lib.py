@@ -24,6 +24,7 @@ EXPORTS = (
     "mi355_paged_decode_workspace_bytes",
     "mi355_paged_decode_chunk_tokens",
     "mi355_rope_and_cache",
+    "mi355_rope_and_cache_fp8",
     "mi355_quantize_kv_fp8",
     "mi355_rms_norm_fwd",
     "mi355_silu_mul_fwd",
@@ -67,6 +68,8 @@ def load():
     lib.mi355_rope_and_cache.restype = i32
     lib.mi355_rope_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32,
                                          i64, i64, i64, i64, vp]
+    lib.mi355_rope_and_cache_fp8.restype = i32
+    lib.mi355_rope_and_cache_fp8.argtypes = [vp] * 11 + [i64, i32, i32, i32, i32, i32, i64, i64, i64, i64, vp]
     lib.mi355_quantize_kv_fp8.restype = i32
     lib.mi355_quantize_kv_fp8.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
     lib.mi355_rms_norm_fwd.restype = i32

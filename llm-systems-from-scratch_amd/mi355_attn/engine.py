@@ -68,14 +68,24 @@ class DecodePlan:
 
 class PagedAttentionEngine:
     def __init__(self, num_blocks, n_q_heads, n_kv_heads, head_dim, context_length, *, rope_theta=10000.0,
-                 max_batch=256, num_layers=1, device="cuda:0"):
+                 max_batch=256, num_layers=1, kv_dtype="bf16", device="cuda:0"):
         self.device = torch.device(device)
         self.Hq, self.Hkv, self.D = n_q_heads, n_kv_heads, head_dim
         self.context_length = context_length
         self.num_layers = num_layers
-        self.k_caches = [torch.zeros(num_blocks, n_kv_heads, BLOCK, head_dim, dtype=torch.bfloat16, device=self.device)
+        if kv_dtype not in ("bf16", "fp8"):
+            raise ValueError("kv_dtype must be 'bf16' or 'fp8'")
+        if kv_dtype == "fp8" and head_dim not in (64, 128):
+            raise ValueError("an fp8 KV cache needs head_dim 64 or 128")
+        self.kv_dtype = kv_dtype
+        cache_dtype = torch.bfloat16 if kv_dtype == "bf16" else torch.uint8      # uint8 = e4m3 bit patterns
+        self.k_caches = [torch.zeros(num_blocks, n_kv_heads, BLOCK, head_dim, dtype=cache_dtype, device=self.device)
                          for _ in range(num_layers)]
         self.v_caches = [torch.zeros_like(k) for k in self.k_caches]
+        # per-(block, kv head) scales of an fp8 cache, maintained by the cache write
+        self.k_scales = [torch.ones(num_blocks, n_kv_heads, dtype=torch.float32, device=self.device)
+                         for _ in range(num_layers)] if kv_dtype == "fp8" else None
+        self.v_scales = [torch.ones_like(s) for s in self.k_scales] if kv_dtype == "fp8" else None
         self.freq_cache = ops.build_rope_cache(context_length, head_dim, rope_theta, self.device)
         self.allocator = BlockAllocator(num_blocks)
         self.blocks: dict[int, list[int]] = {}      # sequence id -> physical blocks
@@ -176,13 +186,21 @@ class PagedAttentionEngine:
                           torch.tensor([p + 1 for p in positions], dtype=torch.int32, device=dev), max_blk * BLOCK)
 
     # ---- attention calls (once per layer) -----------------------------------------
+    def _write_cache(self, layer: int, plan, q, k, v):
+        """RoPE on q and k, rotated k and v into layer `layer`'s cache (quantised when the cache is fp8);
+        returns the rotated q."""
+        kc, vc = self.k_caches[layer], self.v_caches[layer]
+        if self.kv_dtype == "bf16":
+            return ops.rope_and_cache(q, k, v, plan.positions, self.freq_cache, kc, vc, plan.slots)
+        return ops.rope_and_cache_fp8(q, k, v, plan.positions, self.freq_cache, kc, vc, self.k_scales[layer],
+                                      self.v_scales[layer], plan.slots)
+
     def attend_prefill(self, layer: int, plan: PrefillPlan, q, k, v):
         """q (T,Hq,D), k/v (T,Hkv,D) packed along dim 0 (token strides free, heads contiguous).  Writes
         rotated K and V of layer `layer` into its cache and returns causal attention output (T,Hq,D)."""
         if q.shape[0] != plan.positions.shape[0]:
             raise ValueError("the plan and the packed tensors disagree on the number of tokens")
-        kc, vc = self.k_caches[layer], self.v_caches[layer]
-        q_rot = ops.rope_and_cache(q, k, v, plan.positions, self.freq_cache, kc, vc, plan.slots)
+        q_rot = self._write_cache(layer, plan, q, k, v)
         k_rot = ops.rope_and_cache(k, k, v, plan.positions, self.freq_cache)   # rotated keys, packed, for the prefill kernel
         return ops.flash_attn_varlen_prefill(q_rot, k_rot, v, plan.cu_seqlens, plan.cu_seqlens, plan.max_len,
                                              plan.max_len, causal=True)
@@ -192,10 +210,11 @@ class PagedAttentionEngine:
         attention output (B,Hq,D)."""
         if q.shape[0] != plan.positions.shape[0]:
             raise ValueError("one query token per sequence expected")
-        kc, vc = self.k_caches[layer], self.v_caches[layer]
-        q_rot = ops.rope_and_cache(q, k, v, plan.positions, self.freq_cache, kc, vc, plan.slots)
-        return ops.paged_attention_decode(q_rot, kc, vc, plan.tables, plan.context_lens,
-                                          max_context=plan.max_context, workspace=self._workspace)
+        q_rot = self._write_cache(layer, plan, q, k, v)
+        scales = {} if self.kv_dtype == "bf16" else {"k_scale": self.k_scales[layer], "v_scale": self.v_scales[layer]}
+        return ops.paged_attention_decode(q_rot, self.k_caches[layer], self.v_caches[layer], plan.tables,
+                                          plan.context_lens, max_context=plan.max_context, workspace=self._workspace,
+                                          **scales)
 
     # ---- single-layer convenience ----------------------------------------------------
     def prefill(self, seq_ids, lens, q, k, v):

@@ -24,12 +24,13 @@ from .engine import BLOCK, PagedAttentionEngine
 
 class CachedTransformerLM:
     def __init__(self, config: dict, state_dict: dict, *, num_blocks: int | None = None, max_batch: int = 64,
-                 device="cuda:0"):
+                 kv_dtype: str = "bf16", device="cuda:0"):
         """config: the reference's constructor arguments (model.py:128-137: vocab_size, context_length,
         d_model, num_layers, num_heads, d_ff, rope_theta); state_dict: the reference's parameter names,
         with either the separate (ffn.gate_proj/up_proj/down_proj) or the merged (ffn.w_gate_up/w_down)
         feed-forward weights.  num_blocks sizes the KV pool of every layer (default: max_batch full
-        contexts)."""
+        contexts); kv_dtype "fp8" keeps the pool as e4m3 bytes with per-(block, head) scales (half the
+        cache bytes per decode step; d_head 64 or 128)."""
         self.config = dict(config)
         self.device = torch.device(device)
         self.vocab_size = config["vocab_size"]
@@ -67,7 +68,7 @@ class CachedTransformerLM:
             num_blocks = max_batch * ((self.context_length + BLOCK - 1) // BLOCK)
         self.engine = PagedAttentionEngine(num_blocks, H, H, self.d_head, self.context_length,
                                            rope_theta=config["rope_theta"], max_batch=max_batch, num_layers=L,
-                                           device=self.device)
+                                           kv_dtype=kv_dtype, device=self.device)
         self._next_id = 0
 
     @classmethod

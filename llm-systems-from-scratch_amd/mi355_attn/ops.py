@@ -406,6 +406,59 @@ def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, s
     return q_out
 
 
+def rope_and_cache_fp8(q, k, v, positions, freq_cache, k_cache, v_cache, k_scale, v_scale, slot_mapping, *, out=None):
+    """rope_and_cache into an fp8-e4m3 cache: k_cache, v_cache (num_blocks,Hkv,16,D) uint8 (or
+    float8_e4m3fn), k_scale, v_scale (num_blocks,Hkv) fp32, all updated in place.  A block's scale is
+    kept equal to absmax/448 of its valid rows; rows already in a block are re-expressed when new rows
+    raise the scale.  Tokens that share a block must be adjacent with consecutive slots, one such run
+    per block and call (what a prefill or a decode step produces).  Returns the rotated q."""
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        _require_gpu_bf16(n, t)
+        if t.dim() != 3 or t.stride(2) != 1 or t.stride(1) != t.shape[2]:
+            raise ValueError(f"{n} must be (tokens, heads, d_head) with contiguous heads")
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    if k.shape != v.shape or k.shape[0] != T or k.shape[2] != D:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if D not in (32, 64, 128):
+        raise ValueError("d_head must be 32, 64 or 128")
+    if freq_cache.dtype != torch.float32 or freq_cache.dim() != 3 or freq_cache.shape[0] != 2 \
+            or freq_cache.shape[2] * 2 != D or not freq_cache.is_contiguous() or not freq_cache.is_cuda:
+        raise ValueError("freq_cache must be a contiguous float32 GPU tensor (2, context_length, d_head/2)")
+    if positions.dtype != torch.int32 or positions.shape != (T,) or not positions.is_contiguous():
+        raise TypeError("positions must be a contiguous int32 (tokens,) tensor")
+    if slot_mapping.dtype != torch.int64 or slot_mapping.shape != (T,) or not slot_mapping.is_contiguous():
+        raise TypeError("slot_mapping must be a contiguous int64 (tokens,) tensor")
+    for n, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+        if c.dtype not in (torch.uint8, torch.float8_e4m3fn) or c.dim() != 4 or c.shape[1:] != (Hkv, _BLOCK, D) \
+                or not c.is_contiguous() or c.shape[0] != k_cache.shape[0]:
+            raise ValueError(f"{n} must be a contiguous uint8/float8_e4m3fn (num_blocks, {Hkv}, {_BLOCK}, {D}) tensor")
+    nb = k_cache.shape[0]
+    for n, c in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if c.dtype != torch.float32 or c.shape != (nb, Hkv) or not c.is_contiguous():
+            raise ValueError(f"{n} must be a contiguous float32 ({nb}, {Hkv}) tensor")
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        if t.stride(0) % 8 != 0 or t.data_ptr() % 16 != 0:
+            raise ValueError(f"{n} must be 16-byte aligned with a token stride that is a multiple of 8 elements")
+    if out is None:
+        q_out = torch.empty(T, Hq, D, dtype=q.dtype, device=q.device)
+    else:
+        q_out = out
+        _require_gpu_bf16("out", q_out)
+        if q_out.shape != q.shape or q_out.stride(2) != 1 or q_out.stride(1) != D or q_out.stride(0) % 8 != 0 \
+                or q_out.data_ptr() % 16 != 0:
+            raise ValueError("out must have q's shape with contiguous heads, 16-byte aligned")
+    if T == 0:
+        return q_out
+    with _on(q, k, v, q_out, freq_cache, positions, slot_mapping, k_cache, v_cache, k_scale, v_scale) as stream:
+        rc = _lib.load().mi355_rope_and_cache_fp8(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            k_scale.data_ptr(), v_scale.data_ptr(), freq_cache.data_ptr(), positions.data_ptr(), slot_mapping.data_ptr(),
+            nb, T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0), stream)
+    _lib.check(rc, "mi355_rope_and_cache_fp8")
+    return q_out
+
+
 def quantize_kv_cache_fp8(cache, *, out=None):
     """bf16 cache (num_blocks,Hkv,16,D) -> (uint8 e4m3 cache, fp32 scale (num_blocks,Hkv)), scale = absmax/448.
     `out` = (uint8 cache, fp32 scale) tensors to write into instead of new ones."""

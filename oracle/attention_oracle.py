@@ -302,6 +302,61 @@ def rope_and_cache_reference(q, k, v, positions, freq_cache, k_cache, v_cache, s
     return q_rot, kc, vc
 
 
+def _to_e4m3(x, scale):
+    return (x / scale).clamp(-FP8_E4M3_MAX, FP8_E4M3_MAX).to(torch.float8_e4m3fn)
+
+
+def append_rows_fp8(block8, scale, rows, offset):
+    """Appends `rows` (n,D) fp32 at row `offset` of ONE (block, head) slab: block8 (16,D) uint8 e4m3, scale a float.
+
+    The slab's scale stays absmax/448 of its valid rows: offset 0 starts afresh (1.0 for all-zero rows,
+    as quantize_kv_fp8); otherwise scale' = max(scale, absmax(rows)/448) and, when that raised the scale,
+    rows [0, offset) are re-expressed as e4m3((e4m3 value * scale) / scale').  Returns (block8, scale').
+    """
+    out = block8.clone()
+    amax = rows.abs().amax()
+    if offset == 0:
+        new = amax / FP8_E4M3_MAX if amax > 0 else torch.tensor(1.0)
+    else:
+        old = torch.tensor(float(scale), dtype=torch.float32)
+        new = torch.maximum(old, amax / FP8_E4M3_MAX)
+        if float(new) != float(old):
+            kept = out[:offset].view(torch.float8_e4m3fn).float() * old
+            out[:offset] = _to_e4m3(kept, new).view(torch.uint8)
+    out[offset:offset + rows.shape[0]] = _to_e4m3(rows.float(), new).view(torch.uint8)
+    return out, float(new)
+
+
+def rope_and_cache_fp8_reference(q, k, v, positions, freq_cache, k8, k_scale, v8, v_scale, slot_mapping):
+    """rope_and_cache_reference with fp8 caches (uint8 e4m3 (nb,Hkv,16,D) + fp32 scales (nb,Hkv)).
+
+    Rotated keys are rounded to bf16 (what a bf16 cache would hold) before quantisation.  Consecutive
+    tokens with consecutive slots inside one block form a run and are appended together.
+    Returns rotated q (fp32) and updated copies of (k8, k_scale, v8, v_scale).
+    """
+    pos = positions.long()
+    q_rot = rope_reference(q.float().transpose(0, 1), pos, freq_cache).transpose(0, 1)
+    k_rot = rope_reference(k.float().transpose(0, 1), pos, freq_cache).transpose(0, 1).to(torch.bfloat16).float()
+    k8, v8, k_scale, v_scale = k8.clone(), v8.clone(), k_scale.clone(), v_scale.clone()
+    T = q.shape[0]
+    t = 0
+    while t < T:
+        s = int(slot_mapping[t])
+        if s < 0 or s >= k8.shape[0] * 16:
+            t += 1
+            continue
+        n = 1
+        while t + n < T and (s + n) % 16 != 0 and int(slot_mapping[t + n]) == s + n:
+            n += 1
+        b, off = s // 16, s % 16
+        for h in range(k8.shape[1]):
+            k8[b, h], ks = append_rows_fp8(k8[b, h], k_scale[b, h], k_rot[t:t + n, h], off)
+            v8[b, h], vs = append_rows_fp8(v8[b, h], v_scale[b, h], v[t:t + n, h].float(), off)
+            k_scale[b, h], v_scale[b, h] = ks, vs
+        t += n
+    return q_rot, k8, k_scale, v8, v_scale
+
+
 # --------------------------------------------------------------------------
 # Independent brute force (float64 loops) used only to pin the functions above
 # --------------------------------------------------------------------------

@@ -143,3 +143,196 @@ def test_decode_loop_over_growing_cache_equals_causal_prefill(ops):
     pre = ops.flash_attn_prefill(q_rot[None].cuda(), k_rot[None].cuda(), v.transpose(0, 1)[None].cuda(), causal=True)[0]
     err = (pre.float().cpu() - ref).abs()
     assert bool((err <= 2e-2 + 1e-2 * ref.abs()).all()), float(err.max())
+
+
+def _ragged_prefill_case(lens, nb, seed):
+    """Packed tokens of sequences with `lens` tokens, blocks dealt from a seeded permutation of the pool."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(nb, generator=g).tolist()
+    slots, positions, tables = [], [], []
+    for n in lens:
+        blocks = [perm.pop() for _ in range((n + 15) // 16)]
+        tables.append(blocks)
+        slots += [blocks[t // 16] * 16 + t % 16 for t in range(n)]
+        positions += list(range(n))
+    return torch.tensor(slots, dtype=torch.int64), torch.tensor(positions, dtype=torch.int32), tables
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_rope_and_cache_fp8_prefill_then_decode_is_bit_exact_with_the_oracle(ops, D):
+    """A packed prefill (ragged runs, random blocks) and then single-token appends.  Values are copied, and
+    keys at position 0 rotate by the identity, so with all positions 0 both caches must equal the oracle's
+    bit for bit (scales included)."""
+    print(f"case: rope_and_cache_fp8 bit-exact D={D}", flush=True)
+    Hq, Hkv, ctx, nb = 4, 2, 64, 12
+    lens = [37, 1, 16, 5]
+    slots, _, tables = _ragged_prefill_case(lens, nb, seed=40 + D)
+    T = sum(lens)
+    pos0 = torch.zeros(T, dtype=torch.int32)
+    q, k, v = rnd(T, Hq, D, seed=41), rnd(T, Hkv, D, seed=42, scale=1.5), rnd(T, Hkv, D, seed=43, scale=0.8)
+    g = torch.Generator().manual_seed(44)
+    k8 = torch.randint(0, 255, (nb, Hkv, 16, D), generator=g).to(torch.uint8)       # a dirty pool: stale bytes and scales
+    v8 = torch.randint(0, 255, (nb, Hkv, 16, D), generator=g).to(torch.uint8)
+    ks, vs = torch.rand(nb, Hkv, generator=g) + 0.1, torch.rand(nb, Hkv, generator=g) + 0.1
+    fc = orc.build_rope_cache(ctx, D)
+    fcg = ops.build_rope_cache(ctx, D)
+    q_ref, k8r, ksr, v8r, vsr = orc.rope_and_cache_fp8_reference(q, k, v, pos0, fc, k8, ks, v8, vs, slots)
+    k8g, v8g, ksg, vsg = k8.cuda(), v8.cuda(), ks.cuda(), vs.cuda()
+    q_rot = ops.rope_and_cache_fp8(q.cuda(), k.cuda(), v.cuda(), pos0.cuda(), fcg, k8g, v8g, ksg, vsg, slots.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(q_rot.cpu(), q)
+    assert torch.equal(ksg.cpu(), ksr) and torch.equal(vsg.cpu(), vsr)
+    assert torch.equal(k8g.cpu(), k8r) and torch.equal(v8g.cpu(), v8r)
+    # decode steps: one token per sequence, growing amplitudes so that scales rise and rows are re-expressed
+    cur = list(lens)
+    for step in range(20):
+        slots_d, live = [], []
+        for i, blocks in enumerate(tables):
+            if cur[i] % 16 == 0:
+                if len(blocks) * 16 == cur[i]:
+                    free = sorted(set(range(nb)) - {b for tb in tables for b in tb})
+                    if not free:
+                        continue
+                    blocks.append(free[0])
+            slots_d.append(blocks[cur[i] // 16] * 16 + cur[i] % 16)
+            live.append(i)
+            cur[i] += 1
+        B = len(live)
+        amp = 0.5 + 0.25 * step
+        qd, kd, vd = rnd(B, Hq, D, seed=100 + step), rnd(B, Hkv, D, seed=200 + step, scale=amp), rnd(B, Hkv, D, seed=300 + step, scale=amp)
+        sd = torch.tensor(slots_d, dtype=torch.int64)
+        pd = torch.zeros(B, dtype=torch.int32)
+        _, k8r, ksr, v8r, vsr = orc.rope_and_cache_fp8_reference(qd, kd, vd, pd, fc, k8r, ksr, v8r, vsr, sd)
+        ops.rope_and_cache_fp8(qd.cuda(), kd.cuda(), vd.cuda(), pd.cuda(), fcg, k8g, v8g, ksg, vsg, sd.cuda())
+        torch.cuda.synchronize()
+        assert torch.equal(ksg.cpu(), ksr) and torch.equal(vsg.cpu(), vsr), step
+        assert torch.equal(k8g.cpu(), k8r) and torch.equal(v8g.cpu(), v8r), step
+
+
+def test_rope_and_cache_fp8_long_prefill_windows_are_bit_exact(ops):
+    """4096 tokens and more take the 16-token-window path; ragged lengths put run starts anywhere inside
+    the windows, and a second call appends mid-block chunks after them."""
+    print("case: rope_and_cache_fp8 long packed prefill", flush=True)
+    Hq, Hkv, D, ctx = 2, 2, 64, 4096
+    lens = [3001, 1000, 137, 7]
+    nb = sum((n + 15) // 16 for n in lens) + 300
+    slots, _, tables = _ragged_prefill_case(lens, nb, seed=45)
+    T = sum(lens)
+    pos0 = torch.zeros(T, dtype=torch.int32)
+    q, k, v = rnd(T, Hq, D, seed=46), rnd(T, Hkv, D, seed=47, scale=1.5), rnd(T, Hkv, D, seed=48, scale=0.8)
+    g = torch.Generator().manual_seed(49)
+    k8 = torch.randint(0, 255, (nb, Hkv, 16, D), generator=g).to(torch.uint8)
+    v8 = torch.randint(0, 255, (nb, Hkv, 16, D), generator=g).to(torch.uint8)
+    ks, vs = torch.rand(nb, Hkv, generator=g) + 0.1, torch.rand(nb, Hkv, generator=g) + 0.1
+    fc, fcg = orc.build_rope_cache(ctx, D), ops.build_rope_cache(ctx, D)
+    _, k8r, ksr, v8r, vsr = orc.rope_and_cache_fp8_reference(q, k, v, pos0, fc, k8, ks, v8, vs, slots)
+    k8g, v8g, ksg, vsg = k8.cuda(), v8.cuda(), ks.cuda(), vs.cuda()
+    ops.rope_and_cache_fp8(q.cuda(), k.cuda(), v.cuda(), pos0.cuda(), fcg, k8g, v8g, ksg, vsg, slots.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(ksg.cpu(), ksr) and torch.equal(vsg.cpu(), vsr)
+    assert torch.equal(k8g.cpu(), k8r) and torch.equal(v8g.cpu(), v8r)
+    # a chunk of 1100 more tokens per sequence, louder, starting mid-block: the old rows of the first block are re-expressed
+    used = {b for tb in tables for b in tb}
+    free = [b for b in range(nb) if b not in used]
+    more, slots2 = 1100, []
+    for i, n in enumerate(lens):
+        for t in range(n, n + more):
+            if t // 16 >= len(tables[i]):
+                tables[i].append(free.pop())
+            slots2.append(tables[i][t // 16] * 16 + t % 16)
+    T2 = more * len(lens)
+    q2, k2, v2 = rnd(T2, Hq, D, seed=56), rnd(T2, Hkv, D, seed=57, scale=3.0), rnd(T2, Hkv, D, seed=58, scale=2.0)
+    s2, p2 = torch.tensor(slots2, dtype=torch.int64), torch.zeros(T2, dtype=torch.int32)
+    _, k8r, ksr, v8r, vsr = orc.rope_and_cache_fp8_reference(q2, k2, v2, p2, fc, k8r, ksr, v8r, vsr, s2)
+    ops.rope_and_cache_fp8(q2.cuda(), k2.cuda(), v2.cuda(), p2.cuda(), fcg, k8g, v8g, ksg, vsg, s2.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(ksg.cpu(), ksr) and torch.equal(vsg.cpu(), vsr)
+    assert torch.equal(k8g.cpu(), k8r) and torch.equal(v8g.cpu(), v8r)
+
+
+def test_rope_and_cache_fp8_with_rotation_matches_the_oracle_within_one_rounding(ops):
+    """Real positions: the kernel's rotation may differ from the oracle's by one bf16 ulp before
+    quantisation, so compare dequantised keys: equal scales up to that ulp, values within one e4m3 step."""
+    print("case: rope_and_cache_fp8 rotation", flush=True)
+    Hq, Hkv, D, ctx, nb = 8, 2, 128, 256, 16
+    lens = [100, 33, 64]
+    slots, pos, _ = _ragged_prefill_case(lens, nb, seed=50)
+    T = sum(lens)
+    q, k, v = rnd(T, Hq, D, seed=51), rnd(T, Hkv, D, seed=52), rnd(T, Hkv, D, seed=53)
+    fc, fcg = orc.build_rope_cache(ctx, D), ops.build_rope_cache(ctx, D)
+    z8, ones = torch.zeros(nb, Hkv, 16, D, dtype=torch.uint8), torch.ones(nb, Hkv)
+    q_ref, k8r, ksr, v8r, vsr = orc.rope_and_cache_fp8_reference(q, k, v, pos, fc, z8, ones, z8, ones, slots)
+    k8g, v8g, ksg, vsg = z8.cuda(), z8.cuda(), ones.cuda(), ones.cuda()
+    q_rot = ops.rope_and_cache_fp8(q.cuda(), k.cuda(), v.cuda(), pos.cuda(), fcg, k8g, v8g, ksg, vsg, slots.cuda())
+    torch.cuda.synchronize()
+    torch.testing.assert_close(q_rot.float().cpu(), q_ref, atol=2 ** -7, rtol=2 ** -7)
+    assert torch.equal(v8g.cpu(), v8r) and torch.equal(vsg.cpu(), vsr)              # values: no rotation, exact
+    torch.testing.assert_close(ksg.cpu(), ksr, atol=0, rtol=2 ** -7)
+    got, ref = orc.dequantize_kv_fp8(k8g.cpu(), ksg.cpu()), orc.dequantize_kv_fp8(k8r, ksr)
+    assert bool(((got - ref).abs() <= 2 ** -3 * ref.abs() + ksr[:, :, None, None] * 2 ** -8).all())
+    assert float((k8g.cpu() != k8r).float().mean()) < 0.02                            # and almost all bytes agree
+
+
+def test_rope_and_cache_fp8_skips_bad_slots_and_rejects_bad_arguments(ops):
+    print("case: rope_and_cache_fp8 bad slots / arguments", flush=True)
+    T, Hq, Hkv, D, ctx, nb = 6, 2, 2, 64, 32, 3
+    q, k, v = rnd(T, Hq, D, seed=61).cuda(), rnd(T, Hkv, D, seed=62).cuda(), rnd(T, Hkv, D, seed=63).cuda()
+    fcg = ops.build_rope_cache(ctx, D)
+    pos = torch.tensor([0, 1, 2, 3, 40, -2], dtype=torch.int32).cuda()
+    slots = torch.tensor([16, 17, nb * 16, -1, 2 ** 40, 5], dtype=torch.int64).cuda()
+    guard = torch.full((nb + 2, Hkv, 16, D), 9, dtype=torch.uint8, device="cuda")
+    k8, v8 = guard[1:nb + 1], guard.clone()[1:nb + 1]
+    sguard = torch.full((nb + 2, Hkv), 3.0, device="cuda")
+    ks, vs = sguard[1:nb + 1], sguard.clone()[1:nb + 1]
+    ops.rope_and_cache_fp8(q, k, v, pos, fcg, k8, v8, ks, vs, slots)
+    torch.cuda.synchronize()
+    assert bool((guard[0] == 9).all()) and bool((guard[nb + 1] == 9).all())
+    assert bool((sguard[0] == 3).all()) and bool((sguard[nb + 1] == 3).all())
+    flat = k8.permute(0, 2, 1, 3).reshape(nb * 16, Hkv, D)
+    for s in range(nb * 16):
+        assert bool((flat[s] == 9).all()) != (s in {16, 17, 5})
+    assert bool((ks[2] == 3).all())                                                    # block 2 received nothing
+    with pytest.raises(ValueError):
+        ops.rope_and_cache_fp8(q, k, v, pos, fcg, k8, v8, ks[:2], vs, slots)           # scale shape
+    with pytest.raises(ValueError):
+        ops.rope_and_cache_fp8(q, k, v, pos, fcg, k8.to(torch.bfloat16), v8, ks, vs, slots)
+    with pytest.raises(TypeError):
+        ops.rope_and_cache_fp8(q, k, v, pos, fcg, k8, v8, ks, vs, slots.to(torch.int32))
+
+
+def test_fp8_engine_decode_loop_tracks_the_bf16_oracle(ops):
+    """PagedAttentionEngine with an fp8 cache: prefill + 40 decode steps of two sequences; every decode
+    output within the fp8 bound of the fp32 oracle on the unquantised keys and values."""
+    print("case: fp8 engine decode loop", flush=True)
+    Hq, Hkv, D, ctx = 8, 2, 128, 256
+    eng = ops.PagedAttentionEngine(24, Hq, Hkv, D, ctx, max_batch=4, kv_dtype="fp8")
+    lens = [50, 23]
+    steps = 40
+    total = [n + steps for n in lens]
+    qs = [rnd(n, Hq, D, seed=70 + i, scale=0.7) for i, n in enumerate(total)]
+    ks = [rnd(n, Hkv, D, seed=80 + i, scale=0.7) for i, n in enumerate(total)]
+    vs = [rnd(n, Hkv, D, seed=90 + i, scale=0.7) for i, n in enumerate(total)]
+    fc = orc.build_rope_cache(ctx, D)
+    refs = []
+    for i, n in enumerate(total):
+        p = torch.arange(n)
+        qr = orc.rope_reference(qs[i].float().transpose(0, 1), p, fc).to(torch.bfloat16)
+        kr = orc.rope_reference(ks[i].float().transpose(0, 1), p, fc).to(torch.bfloat16)
+        refs.append(orc.prefill_reference(qr[None], kr[None], vs[i].transpose(0, 1)[None], causal=True)[0])   # (Hq,n,D)
+    for i in range(2):
+        eng.add_sequence(i)
+    cat = lambda xs: torch.cat([x[:n] for x, n in zip(xs, lens)]).cuda()
+    out = eng.prefill([0, 1], lens, cat(qs), cat(ks), cat(vs))
+    torch.cuda.synchronize()
+    ref = torch.cat([r[:, :n].transpose(0, 1) for r, n in zip(refs, lens)])
+    err = (out.float().cpu() - ref).abs()
+    assert bool((err <= 2e-2 + 1e-2 * ref.abs()).all())                                # prefill attends the bf16 tensors
+    worst = 0.0
+    for s in range(steps):
+        row = lambda xs: torch.stack([x[n + s] for x, n in zip(xs, lens)]).cuda()
+        o = eng.decode_step([0, 1], row(qs), row(ks), row(vs)).float().cpu()
+        r = torch.stack([refs[i][:, lens[i] + s] for i in range(2)])
+        err = (o - r).abs()
+        worst = max(worst, float(err.max()))
+        assert bool((err <= 0.15 + 2 ** -4 * r.abs()).all()), (s, float(err.max()))
+    print(f"fp8 engine decode: worst abs err {worst:.4f}", flush=True)

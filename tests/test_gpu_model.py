@@ -155,6 +155,41 @@ def test_cached_decode_equals_full_forward_and_oracle(ops):
     assert model.engine.allocator.num_free == model.engine.allocator.num_blocks
 
 
+def test_cached_decode_with_fp8_kv_cache_tracks_the_oracle(ops):
+    """The same decode loop over an fp8 KV pool (fused quantising cache write + fp8 decode kernel).
+    e4m3 keeps 4 significant bits, so the logits carry quantisation noise on top of the bf16 path's: the
+    bound asserted is 0.15 + 5e-2 |ref| against the fp32 oracle (observed 0.07), and the mean absolute
+    error must stay below 0.03."""
+    print("case: cached decode, fp8 KV", flush=True)
+    cfg = dict(CFG, num_layers=3, num_heads=2, d_model=128)          # d_head 64
+    params = _bf16_params(cfg, seed=13)
+    model = ops.CachedTransformerLM(cfg, params, max_batch=4, kv_dtype="fp8")
+    assert model.engine.k_caches[0].dtype == torch.uint8
+    g = torch.Generator().manual_seed(14)
+    seqs = [torch.randint(0, cfg["vocab_size"], (n,), generator=g) for n in (50, 33)]
+    n_prompt = [17, 30]
+    sids = [model.new_sequence() for _ in seqs]
+    logits = model.prefill(sids, [s[:n] for s, n in zip(seqs, n_prompt)])
+    per_seq = [[logits[i]] for i in range(2)]
+    live, pos = [0, 1], list(n_prompt)
+    while live:
+        lg = model.decode([sids[i] for i in live], [int(seqs[i][pos[i]]) for i in live])
+        for j, i in enumerate(live):
+            per_seq[i].append(lg[j])
+            pos[i] += 1
+        live = [i for i in live if pos[i] < len(seqs[i])]
+    for i, s in enumerate(seqs):
+        got = torch.stack(per_seq[i]).float().cpu()
+        ref = mo.transformer_lm_reference(params, cfg, s[None])[0, n_prompt[i] - 1:]
+        err = (got - ref).abs()
+        print(f"fp8 KV logits: max err {float(err.max()):.4f} mean {float(err.mean()):.4f}", flush=True)
+        assert bool((err <= 0.15 + 5e-2 * ref.abs()).all()), float(err.max())
+        assert float(err.mean()) < 0.03
+    for s in sids:
+        model.free_sequence(s)
+    assert model.engine.allocator.num_free == model.engine.allocator.num_blocks
+
+
 def _check_greedy(params, cfg, prompt, toks, margin=0.15):
     """Every generated token must be (nearly) the oracle's argmax given the tokens before it, with the
     reference's sliding window (model.py:215)."""

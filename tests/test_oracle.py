@@ -339,6 +339,94 @@ def test_rope_and_cache_reference_scatters_to_slots():
     assert kc2.abs().sum(dim=(1, 3)).count_nonzero() == 4                       # token 3 (slot -1) was not written
 
 
+def test_fp8_append_whole_block_equals_block_quantiser():
+    """One run that fills a block from offset 0 is exactly quantize_kv_fp8 of that block (scale and bytes)."""
+    g = torch.Generator().manual_seed(31)
+    rows = (torch.randn(16, 64, generator=g) * 3).to(torch.bfloat16).float()
+    junk = torch.randint(0, 255, (16, 64), generator=g).to(torch.uint8)
+    got8, got_scale = orc.append_rows_fp8(junk, 123.0, rows, 0)           # what the slab held before is dead
+    ref8, ref_scale = orc.quantize_kv_fp8(rows.view(1, 1, 16, 64))
+    assert torch.equal(got8, ref8[0, 0]) and got_scale == float(ref_scale[0, 0])
+    z8, z_scale = orc.append_rows_fp8(junk, 5.0, torch.zeros(3, 64), 0)   # all-zero rows: guarded scale
+    assert z_scale == 1.0 and torch.equal(z8[:3], torch.zeros(3, 64, dtype=torch.uint8)) and torch.equal(z8[3:], junk[3:])
+
+
+def test_fp8_append_keeps_scale_equal_to_block_absmax_and_bounds_the_error():
+    """Token-by-token appends: the scale is always absmax(valid rows)/448 (what the block quantiser
+    gives); rows written under an unchanged scale keep their bytes; every re-expression costs at most
+    one more e4m3 rounding (relative 2^-4 on normals, half a subnormal step below)."""
+    g = torch.Generator().manual_seed(32)
+    rows = (torch.randn(16, 128, generator=g) * torch.linspace(0.3, 2.0, 16)[:, None]).to(torch.bfloat16).float()
+    block8 = torch.zeros(16, 128, dtype=torch.uint8)
+    scale, raises = 0.0, 0
+    for t in range(16):
+        before, old = block8.clone(), scale
+        block8, scale = orc.append_rows_fp8(block8, scale, rows[t:t + 1], t)
+        assert scale == float(rows[:t + 1].abs().amax() / orc.FP8_E4M3_MAX)
+        if t and scale == old:
+            assert torch.equal(block8[:t], before[:t])
+        elif t:
+            raises += 1
+        deq = block8[:t + 1].view(torch.float8_e4m3fn).float() * scale
+        step = scale * 2.0 ** -9                                           # e4m3 subnormal spacing, in real units
+        bound = (raises + 1) * (2.0 ** -4 * rows[:t + 1].abs() + step)
+        assert bool(((deq - rows[:t + 1]).abs() <= bound).all())
+    assert raises >= 2                                                     # the growing rows did raise the scale
+
+
+def test_fp8_append_reexpression_is_exact_for_power_of_two_scale_changes():
+    """When the scale doubles, bytes well inside the normal range just lose one exponent step: the
+    re-expressed value equals the old one whenever it stays representable."""
+    rows0 = torch.tensor([[448.0, 224.0, 112.0, 3.5, -28.0, 0.0, 1.75, 56.0]])        # scale 1.0
+    b8, s = orc.append_rows_fp8(torch.zeros(16, 8, dtype=torch.uint8), 0.0, rows0, 0)
+    assert s == 1.0
+    b8, s = orc.append_rows_fp8(b8, s, torch.full((1, 8), 896.0), 1)                   # scale 2.0
+    assert s == 2.0
+    assert torch.equal(b8[0].view(torch.float8_e4m3fn).float() * s, rows0[0])
+    assert torch.equal(b8[1].view(torch.float8_e4m3fn).float() * s, torch.full((8,), 896.0))
+
+
+def test_rope_and_cache_fp8_reference_runs_and_layout():
+    """With whole-block runs the fp8 cache equals quantize_kv_fp8 of the bf16 cache that
+    rope_and_cache_reference builds; decode-style single-token appends keep scale = absmax/448."""
+    g = torch.Generator().manual_seed(33)
+    T, Hq, Hkv, D, ctx, nb = 48, 4, 2, 32, 64, 5
+    q = torch.randn(T, Hq, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(T, Hkv, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(T, Hkv, D, generator=g).to(torch.bfloat16)
+    fc = orc.build_rope_cache(ctx, D)
+    pos = torch.arange(T, dtype=torch.int32) % ctx
+    blocks = [3, 0, 4]                                                     # three full blocks of one sequence
+    slots = torch.tensor([blocks[t // 16] * 16 + t % 16 for t in range(T)], dtype=torch.int64)
+    k8 = torch.randint(0, 255, (nb, Hkv, 16, D), generator=g).to(torch.uint8)
+    v8 = torch.randint(0, 255, (nb, Hkv, 16, D), generator=g).to(torch.uint8)
+    ks, vs = torch.rand(nb, Hkv, generator=g), torch.rand(nb, Hkv, generator=g)
+    q_rot, k8n, ksn, v8n, vsn = orc.rope_and_cache_fp8_reference(q, k, v, pos, fc, k8, ks, v8, vs, slots)
+    q_ref, kc, vc = orc.rope_and_cache_reference(q, k, v, pos, fc, torch.zeros(nb, Hkv, 16, D), torch.zeros(nb, Hkv, 16, D), slots)
+    assert torch.equal(q_rot, q_ref)
+    rk8, rks = orc.quantize_kv_fp8(kc.to(torch.bfloat16))
+    rv8, rvs = orc.quantize_kv_fp8(vc)
+    for b in blocks:
+        assert torch.equal(k8n[b], rk8[b]) and torch.equal(ksn[b], rks[b])
+        assert torch.equal(v8n[b], rv8[b]) and torch.equal(vsn[b], rvs[b])
+    for b in (1, 2):                                                       # untouched blocks keep bytes and scales
+        assert torch.equal(k8n[b], k8[b]) and torch.equal(ksn[b], ks[b]) and torch.equal(v8n[b], v8[b])
+    # the same tokens one call at a time (a decode loop): scales end up identical, bytes differ only by re-expression
+    k8d, v8d, ksd, vsd = k8.clone(), v8.clone(), ks.clone(), vs.clone()
+    for t in range(T):
+        _, k8d, ksd, v8d, vsd = orc.rope_and_cache_fp8_reference(q[t:t + 1], k[t:t + 1], v[t:t + 1], pos[t:t + 1], fc,
+                                                                 k8d, ksd, v8d, vsd, slots[t:t + 1])
+    for b in blocks:
+        assert torch.equal(ksd[b], rks[b]) and torch.equal(vsd[b], rvs[b])
+        err = (orc.dequantize_kv_fp8(v8d, vsd)[b] - vc[b]).abs()
+        assert bool((err <= 16 * (2.0 ** -4 * vc[b].abs() + vsd[b][:, None, None] * 2.0 ** -9)).all())
+    # a slot outside the pool or negative is skipped
+    bad = slots.clone()
+    bad[0], bad[1] = -1, nb * 16
+    _, k8b, _, _, _ = orc.rope_and_cache_fp8_reference(q[:2], k[:2], v[:2], pos[:2], fc, k8, ks, v8, vs, bad[:2])
+    assert torch.equal(k8b, k8)
+
+
 # ---------------------------------------------------------------------------------------------
 # backward oracle
 # ---------------------------------------------------------------------------------------------
