@@ -379,12 +379,16 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
         int first_tile = 0;
         if (CAUSAL) first_tile = max(0, k0 - coff) / kBwRows;
         const int n_tiles = (sq + kBwRows - 1) / kBwRows;
-        // The (query head, row tile) pairs of the GQA group form one stream of steps through the two LDS buffers.
-        // Row tiles are walked from the LAST one down, the query heads of the group innermost: every key tile
-        // needs the last rows, so the workgroups of one (batch, kv head) walk the same Q/dO tiles at the same
-        // time and share them through the XCD's L2.
+        // The (query head, row tile) pairs of the GQA group form one stream of steps through the two LDS buffers,
+        // the query heads of the group innermost.  The workgroups of one (batch, kv head) should walk the same
+        // Q/dO tiles at the same time, so that they share them through the XCD's L2: the first key tile of
+        // the pair (the one with more rows) is walked from the LAST row tile down - every key tile needs the
+        // last rows, and the workgroups start together; the second from its FIRST row tile up - a workgroup
+        // whose first key tile needed n_tiles - 4*pair row tiles then starts at row tile n_tiles - 4*(pair+1)
+        // ... exactly where the workgroups that finished earlier have arrived by then.
         const int tiles_per_head = max(0, n_tiles - first_tile);
         const int n_steps = G * tiles_per_head;
+        const auto row0 = [&](int st) { return (half == 0 ? n_tiles - 1 - st / G : first_tile + st / G) * kBwRows; };
 
         // lse (pre-multiplied by log2 e) and delta of the step's 64 rows: loaded into registers by the first
         // wavefront when the step's tiles are issued, stored to LDS only after the current step's arithmetic,
@@ -392,7 +396,7 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
         float pend_lse = 0.f, pend_delta = 0.f;
         const auto issue = [&](int st) {
             const int h = hk * G + st % G;
-            const int r0 = (n_tiles - 1 - st / G) * kBwRows, buf = (st & 1) * kTile;
+            const int r0 = row0(st), buf = (st & 1) * kTile;
             int64_t q_base, do_base, l_base;
             if (p.cu_q) {
                 q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
@@ -483,7 +487,7 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
         }
         for (int st = 0; st < n_steps; ++st) {
             const bool more = st + 1 < n_steps;
-            const int r0 = (n_tiles - 1 - st / G) * kBwRows;
+            const int r0 = row0(st);
             wait_vmcnt<0>();                                   // this wavefront's share of the step's tiles has landed
             __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
             if (more) issue(st + 1);

@@ -1,0 +1,182 @@
+"""The benchmark configurations at their full stated shapes (configs[2], [3], [4]).
+
+The CPU oracle cannot cover these shapes whole in test time, so each case combines
+  * the oracle on a sample that it finishes in seconds (whole sequences of the decode batches, whole
+    heads of the prefill), and
+  * properties that do not depend on size and involve every output element:
+    decode   - the result does not depend on where the blocks live: after moving every block to a
+               new physical position (and rewriting the tables) the output is identical bit for bit;
+               a sequence served alone equals its row of the batch; outputs lie inside the range of
+               the values attended;
+    prefill  - causality: the rows of a prefix of every sequence are reproduced (bit for bit when the
+               prefix is a whole number of query tiles) when the kernel is given only that prefix;
+               constant values come back as that constant; a first token returns its own value row;
+    backward - linearity in dO for a power-of-two factor (exact), plus the oracle's gradients on all
+               query heads of one (sequence, kv head) group.
+Tolerance where the oracle is involved: |got - ref| <= 2e-2 + 1e-2 |ref| (bf16 paths); fp8 KV is
+checked against the oracle on the dequantised cache with the same bound.
+"""
+import pytest
+import torch
+
+from oracle import attention_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import mi355_attn
+    mi355_attn.load()
+    return mi355_attn
+
+
+def _close(got, ref, atol=2e-2, rtol=1e-2):
+    err = (got.float().cpu() - ref).abs()
+    assert bool((err <= atol + rtol * ref.abs()).all()), f"max err {float(err.max()):.4f}"
+
+
+def _oracle_rows(case, rows):
+    """Oracle output for the sequences `rows` of a decode case: their blocks are gathered into a small pool."""
+    ctx = case.context_lens_host[rows]
+    nblk = (ctx + 15) // 16
+    ids = torch.cat([case.block_tables[b, :int(n)] for b, n in zip(rows, nblk)]).long()
+    kc, vc = case.k_cache[ids].cpu(), case.v_cache[ids].cpu()
+    ks = case.k_scale[ids].cpu() if case.k_scale is not None else None
+    vs = case.v_scale[ids].cpu() if case.v_scale is not None else None
+    bt = torch.zeros(len(rows), int(nblk.max()), dtype=torch.int32)
+    off = 0
+    for i, n in enumerate(nblk):
+        bt[i, :int(n)] = torch.arange(off, off + int(n), dtype=torch.int32)
+        off += int(n)
+    return orc.paged_decode_reference(case.q[rows].cpu(), kc, vc, bt, ctx, k_scale=ks, v_scale=vs)
+
+
+@pytest.mark.parametrize("cfg", [3, 4])
+def test_decode_full_size(ops, cfg):
+    from mi355_attn import workloads
+    print(f"case: decode configs[{cfg}] full size", flush=True)
+    case = workloads.decode_config(cfg, seed=0)
+    B = case.q.shape[0]
+    scales = {} if case.k_scale is None else {"k_scale": case.k_scale, "v_scale": case.v_scale}
+    out = ops.paged_attention_decode(case.q, case.k_cache, case.v_cache, case.block_tables, case.context_lens,
+                                     max_context=case.max_context, **scales)
+    torch.cuda.synchronize()
+    assert out.shape == case.q.shape and bool(torch.isfinite(out.float()).all())
+
+    # oracle on the shortest, the longest and six more sequences
+    order = torch.argsort(case.context_lens_host)
+    rows = sorted({int(order[0]), int(order[-1]), int(order[B // 2])} | {int(i) for i in order[torch.arange(5, B, B // 6)]})
+    _close(out[rows], _oracle_rows(case, rows))
+
+    # every output lies between the smallest and the largest value it can average (per sequence, kv head, dim)
+    b = int(order[B // 3])
+    n = int((case.context_lens_host[b] + 15) // 16)
+    ids = case.block_tables[b, :n].long()
+    vals = case.v_cache[ids]
+    vals = (vals.view(torch.float8_e4m3fn).float() * case.v_scale[ids][:, :, None, None]) if case.k_scale is not None else vals.float()
+    vals = vals.permute(1, 0, 2, 3).reshape(vals.shape[1], n * 16, -1)[:, :int(case.context_lens_host[b])]     # (Hkv, ctx, D)
+    G = case.q.shape[1] // vals.shape[0]
+    lo = vals.amin(1).repeat_interleave(G, 0)
+    hi = vals.amax(1).repeat_interleave(G, 0)
+    o = out[b].float()
+    assert bool((o >= lo - 2e-2 - 1e-2 * lo.abs()).all()) and bool((o <= hi + 2e-2 + 1e-2 * hi.abs()).all())
+
+    # a sequence alone equals its row in the batch (other chunking: within rounding, not bitwise)
+    b = int(order[-1])
+    alone = ops.paged_attention_decode(case.q[b:b + 1], case.k_cache, case.v_cache, case.block_tables[b:b + 1],
+                                       case.context_lens[b:b + 1], **scales)
+    _close(alone, out[b:b + 1].float().cpu(), atol=1e-2, rtol=1e-2)
+
+    # move every block to a new physical position: the output must not change at all
+    nb = case.k_cache.shape[0]
+    perm = torch.randperm(nb, generator=torch.Generator().manual_seed(7)).cuda()        # new position of old block i
+    for name in ("k_cache", "v_cache", "k_scale", "v_scale"):
+        t = getattr(case, name)
+        if t is not None:
+            moved = torch.empty_like(t)
+            moved[perm] = t
+            setattr(case, name, moved)
+            del t, moved
+    tables = perm[case.block_tables.long()].to(torch.int32)
+    scales = {} if case.k_scale is None else {"k_scale": case.k_scale, "v_scale": case.v_scale}
+    out2 = ops.paged_attention_decode(case.q, case.k_cache, case.v_cache, tables, case.context_lens,
+                                      max_context=case.max_context, **scales)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
+def test_prefill_and_backward_full_size(ops):
+    from mi355_attn import workloads
+    print("case: prefill configs[2] full size", flush=True)
+    case = workloads.prefill_config(2, seed=0)
+    S, B = case.seqlen, case.batch
+    Hq, Hkv, D = case.q.shape[1], case.k.shape[1], case.q.shape[2]
+    out = ops.flash_attn_varlen_prefill(case.q, case.k, case.v, case.cu_seqlens, case.cu_seqlens, S, S, causal=True)
+    torch.cuda.synchronize()
+    assert out.shape == case.q.shape and bool(torch.isfinite(out.float()).all())
+
+    # oracle on whole heads: (sequence, query head) samples
+    for b, h in ((0, 0), (3, 13), (7, 31)):
+        hk = h // (Hq // Hkv)
+        rows = slice(b * S, (b + 1) * S)
+        q = case.q[rows, h][None, None].cpu()
+        k = case.k[rows, hk][None, None].cpu()
+        v = case.v[rows, hk][None, None].cpu()
+        _close(out[rows, h][None, None], orc.prefill_reference(q, k, v, causal=True))
+    # the first token of every sequence attends only itself
+    first = torch.arange(B, device="cuda") * S
+    assert torch.equal(out[first], case.v[first].repeat_interleave(Hq // Hkv, 1))
+
+    # causality: given only the first n tokens of every sequence, the kernel reproduces those rows - bit for bit
+    # when n is a multiple of the 256-query tile (same tiles, same wavefronts), within rounding otherwise
+    # (the rescaling decisions of a wavefront then see different neighbour rows)
+    for n in (1536, 1500):
+        idx = (torch.arange(B, device="cuda")[:, None] * S + torch.arange(n, device="cuda")[None]).reshape(-1)
+        cu = (torch.arange(B + 1, dtype=torch.int32) * n).cuda()
+        part = ops.flash_attn_varlen_prefill(case.q[idx], case.k[idx], case.v[idx], cu, cu, n, n, causal=True)
+        torch.cuda.synchronize()
+        if n % 256 == 0:
+            assert torch.equal(part, out[idx])
+        else:
+            _close(part, out[idx].float().cpu(), atol=1e-2, rtol=1e-2)
+
+    # constant values come back unchanged
+    vconst = torch.full_like(case.v, 0.375)
+    oc = ops.flash_attn_varlen_prefill(case.q, case.k, vconst, case.cu_seqlens, case.cu_seqlens, S, S, causal=True)
+    torch.cuda.synchronize()
+    assert float((oc.float() - 0.375).abs().max()) <= 2 ** -8
+    del oc, vconst, part
+
+    print("case: backward configs[2] full size", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    dout = (torch.randn(case.q.shape, generator=g, device="cuda") * 0.5).to(torch.bfloat16)
+
+    def grads(do):
+        q, k, v = (t.detach().clone().requires_grad_() for t in (case.q, case.k, case.v))
+        ops.flash_attn_varlen_prefill(q, k, v, case.cu_seqlens, case.cu_seqlens, S, S, causal=True).backward(do)
+        torch.cuda.synchronize()
+        return q.grad, k.grad, v.grad
+
+    dq, dk, dv = grads(dout)
+    for t in (dq, dk, dv):
+        assert bool(torch.isfinite(t.float()).all())
+    # exactly linear in dO for a power-of-two factor
+    dq4, dk4, dv4 = grads(dout * 4)
+    assert torch.equal(dq4, dq * 4) and torch.equal(dk4, dk * 4) and torch.equal(dv4, dv * 4)
+    del dq4, dk4, dv4
+    # the oracle's gradients on one (sequence, kv head) group: all its query heads, full length
+    b, hk = 5, 3
+    G = Hq // Hkv
+    rows = slice(b * S, (b + 1) * S)
+    q = case.q[rows, hk * G:(hk + 1) * G].transpose(0, 1)[None].cpu()
+    k = case.k[rows, hk:hk + 1].transpose(0, 1)[None].cpu()
+    v = case.v[rows, hk:hk + 1].transpose(0, 1)[None].cpu()
+    do = dout[rows, hk * G:(hk + 1) * G].transpose(0, 1)[None].cpu()
+    rq, rk, rv, _ = orc.prefill_backward_reference(q, k, v, do, causal=True)
+    for name, got, ref in (("dq", dq[rows, hk * G:(hk + 1) * G].transpose(0, 1)[None], rq),
+                           ("dk", dk[rows, hk:hk + 1].transpose(0, 1)[None], rk),
+                           ("dv", dv[rows, hk:hk + 1].transpose(0, 1)[None], rv)):
+        err = (got.float().cpu() - ref).abs()
+        bound = 2e-2 * float(ref.abs().max()) + 2e-2 * ref.abs()
+        assert bool((err <= bound).all()), f"{name}: max err {float(err.max()):.4g} (max |ref| {float(ref.abs().max()):.4g})"
