@@ -13,7 +13,7 @@ The CPU baseline is the oracle (a restatement of the reference's PyTorch attenti
 timed on the host cores over a bounded sample of the same inputs; its outputs also
 check the GPU results of that sample.
 
-usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|fp8|backward|producers|layer]
+usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|fp8|backward|producers|layer|loop]
                        [--no-cpu]
 """
 from __future__ import annotations
@@ -236,6 +236,56 @@ def bench_layer_ops(args):
     return res
 
 
+def bench_decode_loop(args):
+    """Decode steps of the KV-cached decoder at the reference's sample model (configures/sample.yaml:
+    vocab 10000, context 256, d_model 512, 4 layers, 16 heads, d_ff 1344; random weights), batch 8:
+    launched eagerly (about ten launches per layer from Python) and replayed from a captured HIP graph."""
+    import torch
+    import mi355_attn
+
+    cfg = dict(vocab_size=10000, context_length=256, d_model=512, num_layers=4, num_heads=16, d_ff=1344,
+               rope_theta=10000.0)
+    g = torch.Generator().manual_seed(args.seed)
+    d, ff, V = cfg["d_model"], cfg["d_ff"], cfg["vocab_size"]
+
+    def w(*shape, std):
+        return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16)
+
+    sd = {"token_embeddings.weight": w(V, d, std=1.0), "lm_head.weight": w(V, d, std=d ** -0.5),
+          "final_norm.weight": torch.ones(d)}
+    for i in range(cfg["num_layers"]):
+        pre = f"layers.{i}."
+        for n in ("q_proj", "k_proj", "v_proj", "output_proj"):
+            sd[pre + f"attn.{n}.weight"] = w(d, d, std=d ** -0.5)
+        sd[pre + "ffn.gate_proj.weight"] = w(ff, d, std=d ** -0.5)
+        sd[pre + "ffn.up_proj.weight"] = w(ff, d, std=d ** -0.5)
+        sd[pre + "ffn.down_proj.weight"] = w(d, ff, std=ff ** -0.5)
+        sd[pre + "attn_norm.weight"] = torch.ones(d)
+        sd[pre + "ffn_norm.weight"] = torch.ones(d)
+    B, prompt_len, n_steps = 8, 32, min(200, cfg["context_length"] - 33)
+    res = {"config": {"workload": f"decode steps of the KV-cached decoder, reference sample model {cfg}, batch {B}, "
+                                  f"prompt {prompt_len}, {n_steps} timed steps, greedy tokens fed back on the device side "
+                                  "of the host loop", "model": "random weights"}}
+    for name, graphs in (("eager", False), ("hip_graph", True)):
+        model = mi355_attn.CachedTransformerLM(cfg, sd, max_batch=B, decode_graphs=graphs)
+        sids = [model.new_sequence() for _ in range(B)]
+        prompts = [torch.randint(0, V, (prompt_len,), generator=g) for _ in range(B)]
+        logits = model.prefill(sids, prompts)
+        toks = logits.argmax(-1).tolist()
+        for _ in range(5):                                   # warm-up steps (the first graphed one captures)
+            toks = model.decode(sids, toks).argmax(-1).tolist()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_steps):
+            toks = model.decode(sids, toks).argmax(-1).tolist()     # .tolist() synchronises: a real sampling loop
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / n_steps
+        res[name] = {"ms_per_step": dt * 1e3, "tokens_per_s": B / dt}
+        del model
+    res["speedup"] = res["eager"]["ms_per_step"] / res["hip_graph"]["ms_per_step"]
+    return res
+
+
 def _timed_repeats(fn, min_seconds=10.0, max_reps=20):
     """Run fn until min_seconds of wall time have been spent; returns (last result, seconds per call, calls)."""
     total, reps, out = 0.0, 0, None
@@ -353,7 +403,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", choices=["decode", "prefill", "fp8", "backward", "producers", "layer"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "fp8", "backward", "producers", "layer", "loop"], default=None)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the 1 GiB plain copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
@@ -429,6 +479,8 @@ def main():
         line["cache_producers"] = bench_producers(args)
     if args.only in (None, "layer"):
         line["layer_ops"] = bench_layer_ops(args)
+    if args.only in (None, "loop"):
+        line["decode_loop"] = bench_decode_loop(args)
     print(json.dumps(line))
 
 

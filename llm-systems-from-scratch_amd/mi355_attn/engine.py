@@ -66,6 +66,44 @@ class DecodePlan:
     max_context: int
 
 
+class StaticDecodeStep:
+    """Device tensors of one decode step at fixed addresses, refreshed from the host by one copy.
+
+    Layout of the int32 buffer: token ids (int64), slots (int64), positions, context lengths,
+    block tables (batch x max_blocks)."""
+
+    def __init__(self, batch: int, max_blocks: int, device):
+        B, M = batch, max_blocks
+        self.batch, self.max_blocks = B, M
+        n = 6 * B + B * M
+        self._dev = torch.zeros(n, dtype=torch.int32, device=device)
+        self._host = torch.zeros(n, dtype=torch.int32, pin_memory=True)
+        self._copied = torch.cuda.Event()
+        self._pending = False
+        self.tokens = self._dev[0:2 * B].view(torch.int64)
+        slots = self._dev[2 * B:4 * B].view(torch.int64)
+        positions = self._dev[4 * B:5 * B]
+        context_lens = self._dev[5 * B:6 * B]
+        tables = self._dev[6 * B:].view(B, M)
+        self.plan = DecodePlan(positions, slots, tables, context_lens, M * BLOCK)
+        h = self._host
+        self._h_tokens, self._h_slots = h[0:2 * B].view(torch.int64), h[2 * B:4 * B].view(torch.int64)
+        self._h_positions, self._h_ctx, self._h_tables = h[4 * B:5 * B], h[5 * B:6 * B], h[6 * B:].view(B, M)
+
+    def fill(self, tokens, slots, positions, context_lens, block_lists) -> None:
+        if self._pending:
+            self._copied.synchronize()              # the previous copy has left the staging buffer
+        self._h_tokens.copy_(torch.tensor(tokens, dtype=torch.int64))
+        self._h_slots.copy_(torch.tensor(slots, dtype=torch.int64))
+        self._h_positions.copy_(torch.tensor(positions, dtype=torch.int32))
+        self._h_ctx.copy_(torch.tensor(context_lens, dtype=torch.int32))
+        for i, blocks in enumerate(block_lists):
+            self._h_tables[i, :len(blocks)] = torch.tensor(blocks, dtype=torch.int32)
+        self._dev.copy_(self._host, non_blocking=True)
+        self._copied.record()
+        self._pending = True
+
+
 class PagedAttentionEngine:
     def __init__(self, num_blocks, n_q_heads, n_kv_heads, head_dim, context_length, *, rope_theta=10000.0,
                  max_batch=256, num_layers=1, kv_dtype="bf16", device="cuda:0"):
@@ -155,8 +193,8 @@ class PagedAttentionEngine:
                            torch.tensor(cu, dtype=torch.int32, device=dev), max(lens),
                            torch.tensor([c - 1 for c in cu[1:]], dtype=torch.int64, device=dev))
 
-    def plan_decode(self, seq_ids) -> DecodePlan:
-        """Reserves the slot of one new token for each running sequence in `seq_ids`."""
+    def _reserve_decode(self, seq_ids):
+        """Host side of a decode step: checks, reserves one slot per sequence.  Returns (positions, slots)."""
         B = len(seq_ids)
         if B == 0 or B > self.max_batch:
             raise ValueError(f"batch {B} must be in 1..{self.max_batch}")
@@ -172,6 +210,12 @@ class PagedAttentionEngine:
             raise OutOfBlocks(f"decode step needs {need} blocks, {self.allocator.num_free} free")
         positions = [self.lengths[s] for s in seq_ids]
         slots = [self._reserve(s, 1)[0] for s in seq_ids]
+        return positions, slots
+
+    def plan_decode(self, seq_ids) -> DecodePlan:
+        """Reserves the slot of one new token for each running sequence in `seq_ids`."""
+        B = len(seq_ids)
+        positions, slots = self._reserve_decode(seq_ids)
         dev = self.device
         max_len = max(self.lengths[s] for s in seq_ids)
         max_blk = (max_len + BLOCK - 1) // BLOCK
@@ -184,6 +228,25 @@ class PagedAttentionEngine:
         return DecodePlan(torch.tensor(positions, dtype=torch.int32, device=dev),
                           torch.tensor(slots, dtype=torch.int64, device=dev), tables,
                           torch.tensor([p + 1 for p in positions], dtype=torch.int32, device=dev), max_blk * BLOCK)
+
+    def make_static_decode(self, batch: int) -> "StaticDecodeStep":
+        """Fixed device tensors for decode steps of `batch` sequences (what a captured HIP graph needs:
+        the same addresses and shapes on every replay)."""
+        if batch < 1 or batch > self.max_batch:
+            raise ValueError(f"batch {batch} must be in 1..{self.max_batch}")
+        return StaticDecodeStep(batch, self.max_blocks_per_seq, self.device)
+
+    def plan_decode_into(self, seq_ids, tokens, static: "StaticDecodeStep") -> DecodePlan:
+        """plan_decode whose tensors (and the new token ids) are written into `static`: one pinned staging
+        buffer, one asynchronous copy on the current stream.  Tables have their full width and
+        max_context is the context length, so nothing about the step's shapes depends on the data."""
+        B = len(seq_ids)
+        if B != static.batch or len(tokens) != B:
+            raise ValueError("seq_ids, tokens and the static buffers disagree on the batch size")
+        positions, slots = self._reserve_decode(seq_ids)
+        static.fill([int(t) for t in tokens], slots, positions, [p + 1 for p in positions],
+                    [self.blocks[s] for s in seq_ids])
+        return static.plan
 
     # ---- attention calls (once per layer) -----------------------------------------
     def _write_cache(self, layer: int, plan, q, k, v):

@@ -24,13 +24,15 @@ from .engine import BLOCK, PagedAttentionEngine
 
 class CachedTransformerLM:
     def __init__(self, config: dict, state_dict: dict, *, num_blocks: int | None = None, max_batch: int = 64,
-                 kv_dtype: str = "bf16", device="cuda:0"):
+                 kv_dtype: str = "bf16", decode_graphs: bool = False, device="cuda:0"):
         """config: the reference's constructor arguments (model.py:128-137: vocab_size, context_length,
         d_model, num_layers, num_heads, d_ff, rope_theta); state_dict: the reference's parameter names,
         with either the separate (ffn.gate_proj/up_proj/down_proj) or the merged (ffn.w_gate_up/w_down)
         feed-forward weights.  num_blocks sizes the KV pool of every layer (default: max_batch full
         contexts); kv_dtype "fp8" keeps the pool as e4m3 bytes with per-(block, head) scales (half the
-        cache bytes per decode step; d_head 64 or 128)."""
+        cache bytes per decode step; d_head 64 or 128).  decode_graphs=True replays every decode step
+        after the first of a batch size from a captured HIP graph (about ten launches per layer become one
+        graph launch; the step's tensors then live at fixed addresses and tables have their full width)."""
         self.config = dict(config)
         self.device = torch.device(device)
         self.vocab_size = config["vocab_size"]
@@ -70,6 +72,8 @@ class CachedTransformerLM:
                                            rope_theta=config["rope_theta"], max_batch=max_batch, num_layers=L,
                                            kv_dtype=kv_dtype, device=self.device)
         self._next_id = 0
+        self.decode_graphs = decode_graphs
+        self._graphs = {}                      # batch size -> [static step tensors, captured graph, its logits]
 
     @classmethod
     def from_pretrained(cls, config_path: str, checkpoint_path: str, **kwargs) -> "CachedTransformerLM":
@@ -124,11 +128,36 @@ class CachedTransformerLM:
 
     def decode(self, seq_ids, tokens):
         """Appends one token to each running sequence; returns the next-token logits (n_seq, vocab) fp32."""
-        plan = self.engine.plan_decode(list(seq_ids))
+        seq_ids = list(seq_ids)
+        if self.decode_graphs:
+            return self._decode_graphed(seq_ids, torch.as_tensor(tokens).reshape(-1).tolist())
         ids = torch.as_tensor(tokens, dtype=torch.int64).reshape(-1).to(self.device)
         if ids.numel() != len(seq_ids):
             raise ValueError("one token per sequence expected")
+        plan = self.engine.plan_decode(seq_ids)
         return self._forward(ids, plan, self.engine.attend_decode)
+
+    def _decode_graphed(self, seq_ids, tokens):
+        """The decode step through a HIP graph.  The first step of a batch size runs eagerly on the static
+        step tensors (which also initialises every library the graph will call) and is then captured; later
+        steps refresh the static tensors with one copy and replay."""
+        B = len(seq_ids)
+        if len(tokens) != B:
+            raise ValueError("one token per sequence expected")
+        entry = self._graphs.get(B)
+        if entry is None:
+            entry = self._graphs[B] = [self.engine.make_static_decode(B), None, None]
+        static = entry[0]
+        plan = self.engine.plan_decode_into(seq_ids, tokens, static)
+        if entry[1] is None:
+            logits = self._forward(static.tokens, plan, self.engine.attend_decode)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                entry[2] = self._forward(static.tokens, plan, self.engine.attend_decode)
+            entry[1] = graph
+            return logits
+        entry[1].replay()
+        return entry[2].clone()
 
     def forward(self, token_ids):
         """Logits (batch, seq, vocab) of whole sequences, as TransformerLM.forward returns them

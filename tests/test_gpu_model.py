@@ -190,6 +190,53 @@ def test_cached_decode_with_fp8_kv_cache_tracks_the_oracle(ops):
     assert model.engine.allocator.num_free == model.engine.allocator.num_blocks
 
 
+@pytest.mark.parametrize("kv_dtype", ["bf16", "fp8"])
+def test_decode_steps_replayed_from_a_hip_graph_equal_eager_steps(ops, kv_dtype):
+    """decode_graphs=True: the first step of a batch size runs eagerly and is captured, later steps are
+    replays.  Every step of a graphed model is compared with the same step of an eager twin (whose own
+    launches and synchronisations sit between the replays); sequences cross block boundaries, one leaves
+    (a second batch size, a second graph) and a new one joins."""
+    print(f"case: decode graphs, {kv_dtype} KV", flush=True)
+    cfg = dict(CFG, num_layers=3, num_heads=2, d_model=128)          # d_head 64
+    params = _bf16_params(cfg, seed=21)
+    eager = ops.CachedTransformerLM(cfg, params, max_batch=4, kv_dtype=kv_dtype)
+    graphed = ops.CachedTransformerLM(cfg, params, max_batch=4, kv_dtype=kv_dtype, decode_graphs=True)
+    g = torch.Generator().manual_seed(22)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g) for n in (13, 30)]
+    stream = torch.randint(0, cfg["vocab_size"], (40, 2), generator=g)
+    se = [eager.new_sequence() for _ in prompts]
+    sg = [graphed.new_sequence() for _ in prompts]
+    torch.testing.assert_close(graphed.prefill(sg, prompts), eager.prefill(se, prompts))
+
+    def step(ids_e, ids_g, toks):
+        a = eager.decode(ids_e, toks)
+        torch.cuda.synchronize()
+        b = graphed.decode(ids_g, toks)
+        torch.cuda.synchronize()
+        err = (a - b).abs()
+        assert bool((err <= 2e-2 + 2e-2 * a.abs()).all()), float(err.max())     # same kernels; the attention chunking differs
+        return b
+
+    for t in range(20):                                               # 13 -> 33 and 30 -> 50 tokens: new blocks on the way
+        step(se, sg, stream[t].tolist())
+    assert set(graphed._graphs) == {2} and graphed._graphs[2][1] is not None
+    eager.free_sequence(se[0])
+    graphed.free_sequence(sg[0])
+    for t in range(20, 26):                                           # one sequence left: batch size 1
+        step(se[1:], sg[1:], stream[t, 1:].tolist())
+    ne, ng = eager.new_sequence(), graphed.new_sequence()             # a newcomer: back to batch size 2, its graph is reused
+    p3 = torch.randint(0, cfg["vocab_size"], (5,), generator=g)
+    torch.testing.assert_close(graphed.prefill([ng], [p3]), eager.prefill([ne], [p3]))
+    for t in range(26, 34):
+        last = step([se[1], ne], [sg[1], ng], stream[t].tolist())
+    assert set(graphed._graphs) == {1, 2}
+    # and against the oracle: the last step of the long sequence
+    hist = torch.cat([prompts[1], stream[:26, 1], stream[26:34, 0]])    # what that sequence was fed
+    ref = mo.transformer_lm_reference(params, cfg, hist[None])[0, -1]
+    err = (last[0].float().cpu() - ref).abs()
+    assert bool((err <= (0.15 if kv_dtype == "fp8" else 8e-2) + 5e-2 * ref.abs()).all()), float(err.max())
+
+
 def _check_greedy(params, cfg, prompt, toks, margin=0.15):
     """Every generated token must be (nearly) the oracle's argmax given the tokens before it, with the
     reference's sliding window (model.py:215)."""
