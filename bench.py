@@ -97,7 +97,7 @@ def bench_decode(cfg, args, with_cpu):
 
 
 def bench_prefill_backward(cfg, args):
-    """dq, dk, dv at configs[cfg] (the three backward launches: delta, dk/dv, dq).  FLOPs by the usual
+    """dq, dk, dv at configs[cfg] (the two backward launches: dq with delta, then dk and dv).  FLOPs by the usual
     convention: 2.5 x the forward's (five GEMMs against two), causal = half."""
     import torch
     from mi355_attn import ops, workloads
@@ -120,7 +120,7 @@ def bench_prefill_backward(cfg, args):
         "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
         "algorithmic_flops": flops,
         "config": {"workload": f"configs[{cfg}] backward: dq, dk, dv of the causal prefill (seed {args.seed})"},
-        "roofline": {"bound": "mfma", "kernel": "bwd_dkv_kernel + bwd_dq_kernel (+ bwd_delta_kernel)",
+        "roofline": {"bound": "mfma", "kernel": "bwd_dq_kernel + bwd_dkv_kernel",
                      "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms,
                      "traffic": _traffic(f"prefill_bwd_cfg{cfg}")},

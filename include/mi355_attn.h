@@ -100,8 +100,8 @@ int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out
  *   lse   : as written by mi355_prefill_fwd_lse for the same inputs
  *   delta : fp32 scratch with lse's layout and size (receives rowsum(dout * out))
  * GQA: dk/dv of a kv head sum over its Hq/Hkv query heads.  Mask modes NONE / CAUSAL.
- * A causal query row that sees no key (Sq > Sk) gets dq = 0.  Three launches on `stream`
- * (dv; dq, which also fills delta; dk); no atomics, so the result is deterministic.
+ * A causal query row that sees no key (Sq > Sk) gets dq = 0.  Two launches on `stream`
+ * (dq, which also fills delta; then dk and dv together); no atomics, so the result is deterministic.
  */
 int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout,
                       const float* lse, float* delta, void* dq, void* dk, void* dv,

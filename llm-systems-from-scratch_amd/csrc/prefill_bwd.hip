@@ -3,19 +3,19 @@
 //
 //   delta_i = sum_d dO[i,d] * O[i,d]                       (computed, and stored, by the dQ kernel)
 //   P_ij    = exp(scale * q_i.k_j - lse_i)                 (recomputed, never stored)
-//   dV_j    = sum_i P_ij dO_i
-//   dP_ij   = dO_i . v_j
-//   dS_ij   = P_ij (dP_ij - delta_i)
+//   dV_j    = sum_i P_ij dO_i                              (bwd_dkv_kernel: one workgroup per key tile,
+//   dP_ij   = dO_i . v_j                                    summing over the query heads of a GQA group;
+//   dS_ij   = P_ij (dP_ij - delta_i)                        dV on half of its wavefronts, dK on the other half)
+//   dK_j    = scale * sum_i dS_ij q_i
 //   dQ_i    = scale * sum_j dS_ij k_j                      (bwd_dq_kernel: one workgroup per query tile)
-//   dK_j    = scale * sum_i dS_ij q_i                      (bwd_dkv_kernel: one workgroup per key tile,
-//                                                           summing over the query heads of a GQA group)
 //
-// Both main kernels work on transposed problems, like the forward: the wavefront owns 32
-// columns (queries in the dQ kernel, keys in the dK/dV kernel) whose operand fragments stay in
+// Both kernels work on transposed problems, like the forward: the wavefront owns 32 columns
+// (queries in the dQ kernel, keys in the dK/dV kernel) whose operand fragments stay in
 // registers; the other side streams through LDS tiles of 64 rows.  The accumulator of the first
-// MFMA pair (S and dP, column = lane) is, converted to bf16, directly the B operand of the
-// second (dQ^T += K^T dS^T; dV^T += dO^T P, dK^T += Q^T dS), and the matching A operand is a
-// transposed LDS read (ds_read_b64_tr_b16) of the streamed tile with the same row permutation.
+// MFMA (S or dP, column = lane) is, converted to bf16, directly the B operand of the second
+// (dQ^T += K^T dS^T; dV^T += dO^T P, dK^T += Q^T dS), and the matching A operand is a transposed
+// LDS read (ds_read_b64_tr_b16) of the streamed tile with the same row permutation.
+// 7 GEMM-sized products are executed (S and dP in both kernels) where 5 are needed.
 #include <type_traits>
 
 #include "common.hpp"
@@ -26,8 +26,6 @@ namespace mi355 {
 
 constexpr int kBwWaves = 8;
 constexpr int kBwCols = 32 * kBwWaves;   // query columns per workgroup of the dQ kernel (one workgroup of 8 wavefronts per CU)
-constexpr int kBwKvWaves = 8;            // dK/dV kernels: 8 wavefronts = 256 key columns share every streamed Q/dO tile
-constexpr int kBwKvCols = 32 * kBwKvWaves;
 constexpr int kBwRows = 64;              // rows of a streamed LDS tile
 
 struct BwdParams {
@@ -214,53 +212,67 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
             ld.issue(p.k + k_base + (int64_t)r0 * p.ks[2], (int)p.ks[2], sk - 1 - r0, dst + buf);
             ld.issue(p.v + v_base + (int64_t)r0 * p.vs[2], (int)p.vs[2], sk - 1 - r0, dst + 2 * kTile + buf);
         };
+        // The LDS fragments of every MFMA are read kDepth MFMAs ahead, in program order, fenced by scheduling
+        // barriers: left alone the compiler puts each read, and a full wait, directly in front of its MFMA,
+        // and the wavefront then sits through the LDS latency once per MFMA.
+        constexpr int kDepth = 2;
+        // (32 rows of the tile at a_lds) x (this lane's query column, fragments b)
+        const auto scores = [&](const unsigned char* a_lds, const bf16x8 (&bfr)[NS]) {
+            u32x4 a[NS];
+#pragma unroll
+            for (int s = 0; s < kDepth && s < NS; ++s) a[s] = *reinterpret_cast<const u32x4*>(a_lds + rd.row_off[s]);
+            f32x16 r = zero16;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                if (s + kDepth < NS) a[s + kDepth] = *reinterpret_cast<const u32x4*>(a_lds + rd.row_off[s + kDepth]);
+                r = mfma32(as_bf16x8(a[s]), bfr[s], r);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            return r;
+        };
         const auto step = [&](auto masked_c, int tile) {
             constexpr bool MASKED = decltype(masked_c)::value;
             const int k0 = tile * kBwRows;
             const unsigned char* k_lds = lds + (tile & 1) * kTile;
             const unsigned char* v_lds = k_lds + 2 * kTile;
             const int key_lim = last_key - k0 - 4 * kg;      // element (t,i) is kept iff its tile-relative key index <= key_lim
-            f32x16 s_acc[2], dp_acc[2];
+            u32x4 ds[4];
+            // one 32-key half at a time: element i of this lane is key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                for (int s = 0; s < NS; ++s) {
-                    const u32x4 kf = *reinterpret_cast<const u32x4*>(k_lds + t * 32 * kRow + rd.row_off[s]);
-                    s_acc[t] = mfma32(as_bf16x8(kf), qf[s], s == 0 ? zero16 : s_acc[t]);
-                }
-#pragma unroll
-                for (int s = 0; s < NS; ++s) {
-                    const u32x4 vf = *reinterpret_cast<const u32x4*>(v_lds + t * 32 * kRow + rd.row_off[s]);
-                    dp_acc[t] = mfma32(as_bf16x8(vf), dof[s], s == 0 ? zero16 : dp_acc[t]);
-                }
-            }
-            // element (t,i) of this lane: key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
+                const f32x16 s_acc = scores(k_lds + t * 32 * kRow, qf);
+                const f32x16 dp_acc = scores(v_lds + t * 32 * kRow, dof);
+                float x[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float pr = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -lse2));
-                    float ds = pr * (dp_acc[t][i] - delta);                        // dS (without the scale factor)
+                    const float pr = fast_exp2(fmaf(s_acc[i], p.scale_log2, -lse2));
+                    x[i] = pr * (dp_acc[i] - delta);                                   // dS (without the scale factor)
                     if constexpr (MASKED) {
                         // key index relative to the tile (compile-time part) against this lane's last visible key
-                        ds = (32 * t + 8 * (i >> 2) + (i & 3) <= key_lim) ? ds : 0.f;
+                        x[i] = (32 * t + 8 * (i >> 2) + (i & 3) <= key_lim) ? x[i] : 0.f;
                     }
-                    s_acc[t][i] = ds;
                 }
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    ds[2 * t][w] = pack_bf16(x[2 * w], x[2 * w + 1]);
+                    ds[2 * t + 1][w] = pack_bf16(x[8 + 2 * w], x[8 + 2 * w + 1]);
+                }
+            }
             // dQ^T (D x 32 queries) += K^T . dS^T, 16 keys at a time
+            constexpr int NC = 4 * NDT;
+            i16x4 lo[NC], hi[NC];
+            const auto read = [&](int c) {
+                const int u = c / NDT, dt = c % NDT;
+                lo[c] = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[0][dt]);
+                hi[c] = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[1][dt]);
+            };
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int t = u >> 1, e0 = 8 * (u & 1);
-                u32x4 pw;
+            for (int c = 0; c < kDepth && c < NC; ++c) read(c);
 #pragma unroll
-                for (int w = 0; w < 4; ++w) pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
-                const bf16x8 pf = as_bf16x8(pw);
-#pragma unroll
-                for (int dt = 0; dt < NDT; ++dt) {
-                    const i16x4 lo = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[0][dt]);
-                    const i16x4 hi = lds_read_tr16(k_lds + 16 * u * kRow + rd.tr_off[1][dt]);
-                    dq[dt] = mfma32(join_bf16x8(lo, hi), pf, dq[dt]);
-                }
+            for (int c = 0; c < NC; ++c) {
+                if (c + kDepth < NC) read(c + kDepth);
+                dq[c % NDT] = mfma32(join_bf16x8(lo[c], hi[c]), as_bf16x8(ds[c / NDT]), dq[c % NDT]);
+                __builtin_amdgcn_sched_barrier(0);
             }
         };
 
@@ -290,23 +302,32 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// dK (WANT_DK) or dV: one workgroup per tile of 128 keys of one (batch, kv head); Q/dO of every query
-// head of the GQA group stream through LDS together with their lse (and delta).  Two launches instead of
-// one kernel that holds both accumulators keep each under 256 registers, i.e. two wavefronts per SIMD.
-// Per wavefront: K (and, for dK, V) fragments of its 32 key columns in registers, one accumulator set (64).
-template <int D, bool CAUSAL, bool WANT_DK>
-__global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p) {
-    constexpr int NWV = kBwKvWaves;
-    constexpr int kCols = 32 * NWV;                                 // keys per workgroup
+// dK and dV in one kernel, the two roles on different wavefronts: a workgroup owns 128 keys of one
+// (batch, kv head); wavefronts 0-3 (role A) hold the K fragments of 32 keys each and the dV
+// accumulators, wavefronts 4-7 (role B) hold the V fragments of the same keys and the dK accumulators
+// (each role fits 256 registers, so two wavefronts share a SIMD - an A and a B wavefront).  Per step
+// (64 query rows of one query head):
+//   A:  S = Q K^T,  P = exp2(S c - lse)  -> LDS (fp32, for B) and registers (bf16),  dV^T += dO^T P
+//   B:  dP = dO V^T,  dS = P (dP - delta)  with A's P from LDS,                        dK^T += Q^T dS
+// so S is computed once for both gradients (4 GEMM-sized products per step instead of 2 + 3 in two
+// kernels).  A runs one step ahead of B with its P: at iteration i, A produces P(i+1) while B consumes
+// P(i), and the only synchronisation is the one workgroup barrier per iteration that the tile stream
+// needs anyway.  Q tiles therefore live for three iterations (landing, read by A, read by B): a ring
+// of three; dO tiles, read by both roles in the same iteration, alternate between two buffers.
+constexpr int kFuPairs = 4;
+constexpr int kFuCols = 32 * kFuPairs;
+
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams p) {
+    constexpr int NWV = 2 * kFuPairs;
     using R = TileReads<D>;
     constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
-    // [Q buffer 0][Q buffer 1][dO buffer 0][dO buffer 1]
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kTile];
+    constexpr int kPSlab = 64 * 32 * 4;                              // one wavefront's P of one step, fp32
+    // [Q ring 0..2][dO buffer 0..1][P: 2 x kFuPairs slabs]
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[5 * kTile + 2 * kFuPairs * kPSlab];
     __shared__ __attribute__((aligned(16))) float lse_lds2[2 * kBwRows];
     __shared__ __attribute__((aligned(16))) float delta_lds2[2 * kBwRows];
 
-    // equal work per workgroup and one XCD per contiguous id range, as in the dQ kernel: a workgroup takes
-    // the key-tile PAIR (i, nk-1-i)
     const int n_wg = gridDim.x;
     int lid = blockIdx.x;
     if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
@@ -316,7 +337,7 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
     const int b = lid / (n_pairs * p.Hkv);
     const int G = p.Hq / p.Hkv;
     int sq, sk, q_start = 0;
-    int64_t k_base, v_base, o_base;
+    int64_t k_base, v_base, dk_base, dv_base;
     if (p.cu_q) {
         q_start = p.cu_q[b];
         const int k_start = p.cu_k[b];
@@ -324,20 +345,23 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
         sk = p.cu_k[b + 1] - k_start;
         k_base = (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
         v_base = (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
-        o_base = WANT_DK ? (int64_t)k_start * p.dks[2] + (int64_t)hk * p.dks[1]
-                         : (int64_t)k_start * p.dvs[2] + (int64_t)hk * p.dvs[1];
+        dk_base = (int64_t)k_start * p.dks[2] + (int64_t)hk * p.dks[1];
+        dv_base = (int64_t)k_start * p.dvs[2] + (int64_t)hk * p.dvs[1];
     } else {
         sq = p.Sq;
         sk = p.Sk;
         k_base = (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
         v_base = (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
-        o_base = WANT_DK ? (int64_t)b * p.dks[0] + (int64_t)hk * p.dks[1] : (int64_t)b * p.dvs[0] + (int64_t)hk * p.dvs[1];
+        dk_base = (int64_t)b * p.dks[0] + (int64_t)hk * p.dks[1];
+        dv_base = (int64_t)b * p.dvs[0] + (int64_t)hk * p.dvs[1];
     }
-    const int nk = (sk + kCols - 1) / kCols;
+    const int nk = (sk + kFuCols - 1) / kFuCols;
     if (sq <= 0 || 2 * pair >= nk) return;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool role_b = wave >= kFuPairs;
+    const int pw = wave & (kFuPairs - 1);
     const int n = lane & 31, kg = lane >> 5;
     const int coff = sk - sq;
 
@@ -346,58 +370,47 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
     R rd;
     rd.init(lane);
     const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + wave * TileLoader<D, NWV>::NI * 1024);
+    unsigned char* const p_lds = lds + 5 * kTile + pw * kPSlab + lane * 16;       // + parity * kFuPairs * kPSlab + 1024 * vector
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     for (int half = 0; half < 2; ++half) {
         const int ktile = half == 0 ? pair : nk - 1 - pair;
         if (half == 1 && ktile == pair) break;                          // odd tile count: the middle tile has no partner
-        const int k0 = ktile * kCols;
-        const int kw0 = k0 + 32 * wave;
+        const int k0 = ktile * kFuCols;
+        const int kw0 = k0 + 32 * pw;
         const int kj = kw0 + n;
         const bool k_ok = kj < sk;
         __syncthreads();                                                // the previous half's readers are done with the LDS buffers
 
-        // fragments of this lane's key column: step s covers d = 16s + 8kg + j
-        bf16x8 kf[NS], vf[WANT_DK ? NS : 1];
+        // fragments of this lane's key column (K for role A, V for role B): step s covers d = 16s + 8kg + j
+        bf16x8 frag[NS];
+        {
+            const __bf16* src = role_b ? p.v + v_base + (int64_t)kj * p.vs[2] : p.k + k_base + (int64_t)kj * p.ks[2];
 #pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            u32x4 a = {0u, 0u, 0u, 0u}, g = {0u, 0u, 0u, 0u};
-            if (k_ok) {
-                a = *reinterpret_cast<const u32x4*>(p.k + k_base + (int64_t)kj * p.ks[2] + 16 * s + 8 * kg);
-                if (WANT_DK) g = *reinterpret_cast<const u32x4*>(p.v + v_base + (int64_t)kj * p.vs[2] + 16 * s + 8 * kg);
+            for (int s = 0; s < NS; ++s) {
+                u32x4 a = {0u, 0u, 0u, 0u};
+                if (k_ok) a = *reinterpret_cast<const u32x4*>(src + 16 * s + 8 * kg);
+                frag[s] = as_bf16x8(a);
             }
-            kf[s] = as_bf16x8(a);
-            if (WANT_DK) vf[s] = as_bf16x8(g);
         }
         f32x16 acc[NDT];
 #pragma unroll
-        for (int i = 0; i < NDT; ++i)
-#pragma unroll
-            for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
-        const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < NDT; ++i) acc[i] = zero16;
 
-        // causal: key kj is seen by queries i >= kj - coff; the first row tile that can see key k0
         int first_tile = 0;
         if (CAUSAL) first_tile = max(0, k0 - coff) / kBwRows;
         const int n_tiles = (sq + kBwRows - 1) / kBwRows;
-        // The (query head, row tile) pairs of the GQA group form one stream of steps through the two LDS buffers,
-        // the query heads of the group innermost.  The workgroups of one (batch, kv head) should walk the same
-        // Q/dO tiles at the same time, so that they share them through the XCD's L2: the first key tile of
-        // the pair (the one with more rows) is walked from the LAST row tile down - every key tile needs the
-        // last rows, and the workgroups start together; the second from its FIRST row tile up - a workgroup
-        // whose first key tile needed n_tiles - 4*pair row tiles then starts at row tile n_tiles - 4*(pair+1)
-        // ... exactly where the workgroups that finished earlier have arrived by then.
-        const int tiles_per_head = max(0, n_tiles - first_tile);
-        const int n_steps = G * tiles_per_head;
+        // Steps: (query head of the group, row tile), heads innermost; the first key tile of the pair walks
+        // its row tiles from the last one down, the second from its first one up, which keeps all workgroups
+        // of a (batch, kv head) on the same Q/dO tiles at the same time (they share them through the L2).
+        const int n_steps = G * max(0, n_tiles - first_tile);
         const auto row0 = [&](int st) { return (half == 0 ? n_tiles - 1 - st / G : first_tile + st / G) * kBwRows; };
+        // a step whose rows all lie above this wavefront's first key column has nothing for it (uniform)
+        const auto idle = [&](int st) { return CAUSAL && kw0 > row0(st) + kBwRows - 1 + coff; };
 
-        // lse (pre-multiplied by log2 e) and delta of the step's 64 rows: loaded into registers by the first
-        // wavefront when the step's tiles are issued, stored to LDS only after the current step's arithmetic,
-        // so that waiting for them never sits in front of it.
         float pend_lse = 0.f, pend_delta = 0.f;
-        const auto issue = [&](int st) {
+        const auto bases = [&](int st, int64_t& q_base, int64_t& do_base, int64_t& l_base) {
             const int h = hk * G + st % G;
-            const int r0 = row0(st), buf = (st & 1) * kTile;
-            int64_t q_base, do_base, l_base;
             if (p.cu_q) {
                 q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
                 do_base = (int64_t)q_start * p.dos[2] + (int64_t)h * p.dos[1];
@@ -407,102 +420,149 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
                 do_base = (int64_t)b * p.dos[0] + (int64_t)h * p.dos[1];
                 l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
             }
-            ld.issue(p.q + q_base + (int64_t)r0 * p.qs[2], (int)p.qs[2], sq - 1 - r0, dst + buf);
-            ld.issue(p.dout + do_base + (int64_t)r0 * p.dos[2], (int)p.dos[2], sq - 1 - r0, dst + 2 * kTile + buf);
-            if (tid < kBwRows) {                               // a padded query row gets lse = +inf, i.e. P = 0
-                const bool ok = r0 + tid < sq;
-                pend_lse = ok ? p.lse[l_base + r0 + tid] * kLog2e : INFINITY;
-                if (WANT_DK) pend_delta = ok ? p.delta[l_base + r0 + tid] : 0.f;
-            }
         };
-        const auto publish = [&](int st) {
-            if (tid < kBwRows) {
-                lse_lds2[(st & 1) * kBwRows + tid] = pend_lse;
-                if (WANT_DK) delta_lds2[(st & 1) * kBwRows + tid] = pend_delta;
-            }
+        // Q tile of step st into ring slot `slot`; its lse into a register
+        const auto issue_q = [&](int st, int slot) {
+            int64_t q_base, do_base, l_base;
+            bases(st, q_base, do_base, l_base);
+            const int r0 = row0(st);
+            ld.issue(p.q + q_base + (int64_t)r0 * p.qs[2], (int)p.qs[2], sq - 1 - r0, dst + slot * kTile);
+            const float* rows = p.lse + l_base + r0;                                   // uniform base, 32-bit lane offset
+            if (tid < kBwRows) pend_lse = rows[(unsigned)min(tid, sq - 1 - r0)];                 // consumed only by publish_lse
         };
-        const auto step = [&](auto masked_c, int st, int r0) {
-            constexpr bool MASKED = decltype(masked_c)::value;
-            const unsigned char* q_lds = lds + (st & 1) * kTile;
-            const unsigned char* do_lds = q_lds + 2 * kTile;
-            const float* lse_lds = lse_lds2 + (st & 1) * kBwRows;
-            const float* delta_lds = delta_lds2 + (st & 1) * kBwRows;
-            const int row_lim = CAUSAL ? kj - coff - r0 - 4 * kg : -1;
-            f32x16 s_acc[2], dp_acc[WANT_DK ? 2 : 1];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                for (int s = 0; s < NS; ++s) {
-                    const u32x4 a = *reinterpret_cast<const u32x4*>(q_lds + t * 32 * kRow + rd.row_off[s]);
-                    s_acc[t] = mfma32(as_bf16x8(a), kf[s], s == 0 ? zero16 : s_acc[t]);
-                }
-                if constexpr (WANT_DK) {
-#pragma unroll
-                    for (int s = 0; s < NS; ++s) {
-                        const u32x4 a = *reinterpret_cast<const u32x4*>(do_lds + t * 32 * kRow + rd.row_off[s]);
-                        dp_acc[t] = mfma32(as_bf16x8(a), vf[s], s == 0 ? zero16 : dp_acc[t]);
-                    }
-                }
-            }
-            // element (t,i) of this lane: query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int rl = 32 * t + 8 * j + 4 * kg;                        // local row of element i = 4j
-                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_lds + rl);
-                    f32x4 d4 = {0.f, 0.f, 0.f, 0.f};
-                    if constexpr (WANT_DK) d4 = *reinterpret_cast<const f32x4*>(delta_lds + rl);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int i = 4 * j + r;
-                        float x = fast_exp2(fmaf(s_acc[t][i], p.scale_log2, -l4[r]));     // P
-                        if constexpr (WANT_DK) x *= dp_acc[t][i] - d4[r];                  // dS (without the scale factor)
-                        // kept iff kj <= r0 + rl + r + coff, i.e. the tile-relative row (compile-time part) >= row_lim
-                        if constexpr (MASKED) x = (32 * t + 8 * j + r >= row_lim) ? x : 0.f;
-                        s_acc[t][i] = x;
-                    }
-                }
-            // dV^T (D x 32 keys) += dO^T . P   or   dK^T += Q^T . dS, 16 query rows at a time
-            const unsigned char* a_lds = WANT_DK ? q_lds : do_lds;
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int t = u >> 1, e0 = 8 * (u & 1);
-                u32x4 pw;
-#pragma unroll
-                for (int w = 0; w < 4; ++w) pw[w] = pack_bf16(s_acc[t][e0 + 2 * w], s_acc[t][e0 + 2 * w + 1]);
-                const bf16x8 pf = as_bf16x8(pw);
-#pragma unroll
-                for (int dt = 0; dt < NDT; ++dt) {
-                    const i16x4 lo = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[0][dt]);
-                    const i16x4 hi = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[1][dt]);
-                    acc[dt] = mfma32(join_bf16x8(lo, hi), pf, acc[dt]);
-                }
-            }
+        const auto issue_do = [&](int st) {
+            int64_t q_base, do_base, l_base;
+            bases(st, q_base, do_base, l_base);
+            const int r0 = row0(st);
+            ld.issue(p.dout + do_base + (int64_t)r0 * p.dos[2], (int)p.dos[2], sq - 1 - r0, dst + (3 + (st & 1)) * kTile);
+            const float* rows = p.delta + l_base + r0;
+            if (tid < kBwRows) pend_delta = rows[(unsigned)min(tid, sq - 1 - r0)];
+        };
+        // (the values are scaled and masked here, not where they are loaded: consuming them there would put a
+        // wait for all outstanding loads - the tiles just issued - in front of the step's arithmetic)
+        const auto publish_lse = [&](int st) {
+            if (tid < kBwRows) lse_lds2[(st & 1) * kBwRows + tid] = row0(st) + tid < sq ? pend_lse * kLog2e : INFINITY;
+        };
+        const auto publish_delta = [&](int st) {
+            if (tid < kBwRows) delta_lds2[(st & 1) * kBwRows + tid] = row0(st) + tid < sq ? pend_delta : 0.f;
         };
 
-        if (n_steps > 0) {
-            issue(0);
-            publish(0);
-        }
-        for (int st = 0; st < n_steps; ++st) {
-            const bool more = st + 1 < n_steps;
-            const int r0 = row0(st);
-            wait_vmcnt<0>();                                   // this wavefront's share of the step's tiles has landed
-            __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
-            if (more) issue(st + 1);
-            // nothing to do when the tile lies wholly above this wavefront's diagonal (its first key column is
-            // not seen by the tile's last row); no mask when the tile's first row sees the last key column
-            if (!(CAUSAL && kw0 > r0 + kBwRows - 1 + coff)) {
-                step(std::true_type{}, st, r0);
+        // second GEMM of either role: acc^T (D x 32 keys) += tile^T . W, 16 query rows at a time.
+        // The transposed fragments are read kDepth MFMAs ahead, in this order, fenced by scheduling barriers:
+        // left alone the compiler puts each pair of reads, and a full wait, directly in front of its MFMA.
+        constexpr int kDepth = 2;
+        const auto update = [&](const unsigned char* a_lds, const u32x4 (&w)[4]) {
+            constexpr int NC = 4 * NDT;
+            i16x4 lo[NC], hi[NC];
+            const auto read = [&](int c) {
+                const int u = c / NDT, dt = c % NDT;
+                lo[c] = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[0][dt]);
+                hi[c] = lds_read_tr16(a_lds + 16 * u * kRow + rd.tr_off[1][dt]);
+            };
+#pragma unroll
+            for (int c = 0; c < kDepth && c < NC; ++c) read(c);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                if (c + kDepth < NC) read(c + kDepth);
+                acc[c % NDT] = mfma32(join_bf16x8(lo[c], hi[c]), as_bf16x8(w[c / NDT]), acc[c % NDT]);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            if (more) publish(st + 1);
+        };
+        // first GEMM of either role: (32 rows of the tile at a_lds) x (this lane's key column), fragments read ahead likewise
+        const auto scores = [&](const unsigned char* a_lds) {
+            u32x4 a[NS];
+#pragma unroll
+            for (int s = 0; s < kDepth && s < NS; ++s) a[s] = *reinterpret_cast<const u32x4*>(a_lds + rd.row_off[s]);
+            f32x16 r = zero16;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                if (s + kDepth < NS) a[s + kDepth] = *reinterpret_cast<const u32x4*>(a_lds + rd.row_off[s + kDepth]);
+                r = mfma32(as_bf16x8(a[s]), frag[s], r);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            return r;
+        };
+        // role A: P of step st from the Q tile in ring slot `slot`: fp32 to LDS for role B, bf16 into p_cur
+        u32x4 p_cur[4];
+        const auto make_p = [&](int st, int slot) {
+            const unsigned char* q_lds = lds + slot * kTile;
+            const float* lse_lds = lse_lds2 + (st & 1) * kBwRows;
+            unsigned char* out = p_lds + (st & 1) * (kFuPairs * kPSlab);
+            const int row_lim = CAUSAL ? kj - coff - row0(st) - 4 * kg : -1;
+            // one 32-row half at a time: element i of this lane is query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const f32x16 s_acc = scores(q_lds + t * 32 * kRow);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_lds + 32 * t + 8 * j + 4 * kg);
+                    f32x4 x4;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float x = fast_exp2(fmaf(s_acc[4 * j + r], p.scale_log2, -l4[r]));
+                        // kept iff kj <= row + coff, i.e. the tile-relative row (compile-time part) >= row_lim
+                        if (CAUSAL) x = (32 * t + 8 * j + r >= row_lim) ? x : 0.f;
+                        x4[r] = x;
+                    }
+                    *reinterpret_cast<f32x4*>(out + (4 * t + j) * 1024) = x4;
+                    p_cur[2 * t + (j >> 1)][2 * (j & 1)] = pack_bf16(x4[0], x4[1]);
+                    p_cur[2 * t + (j >> 1)][2 * (j & 1) + 1] = pack_bf16(x4[2], x4[3]);
+                }
+            }
+        };
+        // role B: dS of step st (Q tile in ring slot `slot`), dK^T += Q^T dS
+        const auto step_b = [&](int st, int slot) {
+            const unsigned char* q_lds = lds + slot * kTile;
+            const unsigned char* do_lds = lds + (3 + (st & 1)) * kTile;
+            const float* delta_lds = delta_lds2 + (st & 1) * kBwRows;
+            const unsigned char* in = p_lds + (st & 1) * (kFuPairs * kPSlab);
+            u32x4 ds[4];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const f32x16 dp_acc = scores(do_lds + t * 32 * kRow);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const f32x4 p4 = *reinterpret_cast<const f32x4*>(in + (4 * t + j) * 1024);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_lds + 32 * t + 8 * j + 4 * kg);
+                    float x[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) x[r] = p4[r] * (dp_acc[4 * j + r] - d4[r]);      // dS without the scale factor
+                    ds[2 * t + (j >> 1)][2 * (j & 1)] = pack_bf16(x[0], x[1]);
+                    ds[2 * t + (j >> 1)][2 * (j & 1) + 1] = pack_bf16(x[2], x[3]);
+                }
+            }
+            update(q_lds, ds);
+        };
+
+        // iteration i = -1 .. n_steps-1; ring slots: Q(i) in s_b, Q(i+1) in s_a, Q(i+2) lands in s_l
+        if (n_steps > 0) {
+            issue_q(0, 0);
+            publish_lse(0);
+        }
+        int s_b = 2, s_a = 0, s_l = 1;
+        for (int i = -1; i < n_steps; ++i) {
+            wait_vmcnt<0>();                                   // this wavefront's share of the tiles issued one iteration ago has landed
+            __syncthreads();                                   // ... and everybody's; P(i), lse(i+1), delta(i) are visible; older buffers are free
+            if (i + 2 < n_steps) issue_q(i + 2, s_l);
+            if (i + 1 < n_steps) issue_do(i + 1);
+            if (!role_b) {
+                if (i >= 0 && !idle(i)) update(lds + (3 + (i & 1)) * kTile, p_cur);      // dV^T += dO(i)^T P(i)
+                if (i + 1 < n_steps && !idle(i + 1)) make_p(i + 1, s_a);
+            } else {
+                if (i >= 0 && !idle(i)) step_b(i, s_b);
+            }
+            if (i + 2 < n_steps) publish_lse(i + 2);
+            if (i + 1 < n_steps) publish_delta(i + 1);
+            const int t3 = s_b;
+            s_b = s_a;
+            s_a = s_l;
+            s_l = t3;
         }
 
         // store: lane owns key kj, d = 32dt + 8(i/4) + 4kg + i%4
         if (k_ok) {
-            const float f = WANT_DK ? p.scale : 1.0f;
-            __bf16* row = (WANT_DK ? p.dk + (int64_t)kj * p.dks[2] : p.dv + (int64_t)kj * p.dvs[2]) + o_base;
+            const float f = role_b ? p.scale : 1.0f;
+            __bf16* row = role_b ? p.dk + dk_base + (int64_t)kj * p.dks[2] : p.dv + dv_base + (int64_t)kj * p.dvs[2];
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
@@ -518,16 +578,14 @@ __global__ __launch_bounds__(kBwKvWaves * 64, 1) void bwd_dkv_kernel(BwdParams p
 
 template <int D>
 static int launch_bwd(const BwdParams& p, bool causal, hipStream_t stream) {
-    const dim3 block(kBwWaves * 64), block_kv(kBwKvWaves * 64);
+    const dim3 block(kBwWaves * 64), block_kv(2 * kFuPairs * 64);
     const dim3 grid_q((unsigned)((p.n_qtiles + 1) / 2 * p.Hq * p.B)), grid_k((unsigned)((p.n_ktiles + 1) / 2 * p.Hkv * p.B));
     if (causal) {
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, true, false>), grid_k, block_kv, 0, stream, p);     // dV
         hipLaunchKernelGGL((bwd_dq_kernel<D, true>), grid_q, block, 0, stream, p);                // dQ, writes delta
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, true, true>), grid_k, block_kv, 0, stream, p);      // dK, reads delta
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, true>), grid_k, block_kv, 0, stream, p);      // dK and dV, reads delta
     } else {
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, false, false>), grid_k, block_kv, 0, stream, p);
         hipLaunchKernelGGL((bwd_dq_kernel<D, false>), grid_q, block, 0, stream, p);
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, false, true>), grid_k, block_kv, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, false>), grid_k, block_kv, 0, stream, p);
     }
     return (int)hipGetLastError();
 }
@@ -603,7 +661,7 @@ extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, co
     p.scale = softmax_scale;
     p.scale_log2 = softmax_scale * kLog2e;
     p.n_qtiles = (Sq_max + kBwCols - 1) / kBwCols;
-    p.n_ktiles = (Sk_max + kBwKvCols - 1) / kBwKvCols;
+    p.n_ktiles = (Sk_max + kFuCols - 1) / kFuCols;
     if ((int64_t)p.n_qtiles * Hq * B > 0x7fffffffLL || (int64_t)p.n_ktiles * Hkv * B > 0x7fffffffLL)
         return set_error(MI355_EINVAL, "prefill_bwd: too many workgroups");
 
