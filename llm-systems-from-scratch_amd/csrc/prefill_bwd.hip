@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
         l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
     }
     const int nq = (sq + kBwCols - 1) / kBwCols;
-    if (sk <= 0 || 2 * pair >= nq) return;
+    if (2 * pair >= nq) return;                                         // (a sequence without keys still gets dq = 0 written)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -356,7 +356,7 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
         dv_base = (int64_t)b * p.dvs[0] + (int64_t)hk * p.dvs[1];
     }
     const int nk = (sk + kFuCols - 1) / kFuCols;
-    if (sq <= 0 || 2 * pair >= nk) return;
+    if (2 * pair >= nk) return;                                         // (a sequence without queries still gets dk = dv = 0 written)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -444,7 +444,10 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             if (tid < kBwRows) lse_lds2[(st & 1) * kBwRows + tid] = row0(st) + tid < sq ? pend_lse * kLog2e : INFINITY;
         };
         const auto publish_delta = [&](int st) {
-            if (tid < kBwRows) delta_lds2[(st & 1) * kBwRows + tid] = row0(st) + tid < sq ? pend_delta : 0.f;
+            // a causal row that sees no key has out = NaN, hence delta = NaN, and P = 0 everywhere: any finite
+            // delta gives the dS = 0 it must have
+            if (tid < kBwRows)
+                delta_lds2[(st & 1) * kBwRows + tid] = (row0(st) + tid < sq && pend_delta == pend_delta) ? pend_delta : 0.f;
         };
 
         // second GEMM of either role: acc^T (D x 32 keys) += tile^T . W, 16 query rows at a time.

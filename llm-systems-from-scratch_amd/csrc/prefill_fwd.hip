@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     // Causal work grows with the query-tile index, so a workgroup takes the tiles
     // (nq-1-pair) and (pair): every workgroup of a sequence then carries the same load.
     const int nq = (sq + kBM - 1) / kBM;
-    if (sk <= 0 || 2 * pair >= nq) return;
+    if (2 * pair >= nq) return;          // (a sequence without keys still gets its rows written: no key kept -> NaN)
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;

@@ -157,3 +157,48 @@ def test_no_grad_path_and_errors(ops):
     assert out.requires_grad
     out.sum().backward()
     assert q.grad is not None and k.grad is None
+
+
+def test_backward_rows_without_keys_and_empty_sequences(ops):
+    """Causal with more queries than keys: the first Sq - Sk rows see no key (forward: NaN rows, like the
+    reference softmax of an all-masked row); they must get dq = 0 and leave dk, dv untouched, i.e. the
+    gradients equal those of the problem restricted to the rows that do see keys.  Packed batch with a
+    sequence that has keys but no queries, and one with queries but no keys: every gradient row is
+    written (zeros where nothing contributes)."""
+    print("case: backward rows without keys / empty sequences", flush=True)
+    B, Hq, Hkv, Sq, Sk, D = 1, 4, 2, 200, 130, 64
+    q, k, v, dout = rnd(B, Hq, Sq, D, seed=90), rnd(B, Hkv, Sk, D, seed=91), rnd(B, Hkv, Sk, D, seed=92), rnd(B, Hq, Sq, D, seed=93)
+    qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+    out = ops.flash_attn_prefill(qg, kg, vg, causal=True)
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    dead = Sq - Sk
+    assert bool(torch.isnan(out[:, :, :dead].float()).all()) and bool(torch.isfinite(out[:, :, dead:].float()).all())
+    dq_ref, dk_ref, dv_ref, _ = orc.prefill_backward_reference(q[:, :, dead:], k, v, dout[:, :, dead:], causal=True)
+    assert bool((qg.grad[:, :, :dead] == 0).all())
+    check_grad("dq", qg.grad[:, :, dead:], dq_ref)
+    check_grad("dk", kg.grad, dk_ref)
+    check_grad("dv", vg.grad, dv_ref)
+
+    lens_q, lens_k = [70, 0, 33, 40], [70, 50, 33, 0]
+    Hq, Hkv, D = 4, 2, 128
+    cu_q = torch.tensor([0] + torch.tensor(lens_q).cumsum(0).tolist(), dtype=torch.int32)
+    cu_k = torch.tensor([0] + torch.tensor(lens_k).cumsum(0).tolist(), dtype=torch.int32)
+    Tq, Tk = sum(lens_q), sum(lens_k)
+    q, k, v, dout = rnd(Tq, Hq, D, seed=94), rnd(Tk, Hkv, D, seed=95), rnd(Tk, Hkv, D, seed=96), rnd(Tq, Hq, D, seed=97)
+    qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+    out = ops.flash_attn_varlen_prefill(qg, kg, vg, cu_q.cuda(), cu_k.cuda(), max(lens_q), max(lens_k), causal=False)
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    dq_ref, dk_ref, dv_ref = torch.zeros(Tq, Hq, D), torch.zeros(Tk, Hkv, D), torch.zeros(Tk, Hkv, D)
+    for b in range(len(lens_q)):
+        sq, sk = slice(int(cu_q[b]), int(cu_q[b + 1])), slice(int(cu_k[b]), int(cu_k[b + 1]))
+        if lens_q[b] == 0 or lens_k[b] == 0:
+            continue                                                   # nothing attends / nothing to attend: zero gradients
+        args = [q[sq].transpose(0, 1)[None], k[sk].transpose(0, 1)[None], v[sk].transpose(0, 1)[None], dout[sq].transpose(0, 1)[None]]
+        a, bb, c, _ = orc.prefill_backward_reference(*args, causal=False)
+        dq_ref[sq], dk_ref[sk], dv_ref[sk] = a[0].transpose(0, 1), bb[0].transpose(0, 1), c[0].transpose(0, 1)
+    assert bool(torch.isnan(out[int(cu_q[3]):].float()).all())        # queries without keys: NaN rows, as for any row that keeps no key
+    check_grad("dq", qg.grad, dq_ref)
+    check_grad("dk", kg.grad, dk_ref)
+    check_grad("dv", vg.grad, dv_ref)
