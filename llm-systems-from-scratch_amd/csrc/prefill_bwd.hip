@@ -404,13 +404,26 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
         // its row tiles from the last one down, the second from its first one up, which keeps all workgroups
         // of a (batch, kv head) on the same Q/dO tiles at the same time (they share them through the L2).
         const int n_steps = G * max(0, n_tiles - first_tile);
-        const auto row0 = [&](int st) { return (half == 0 ? n_tiles - 1 - st / G : first_tile + st / G) * kBwRows; };
+        // position of a step: first row of its tile and query head within the group; advanced incrementally
+        // (steps i, i+1 and i+2 are in flight at any time; no division per step)
+        struct Pos {
+            int r0, hq;
+        };
+        const int r_step = half == 0 ? -kBwRows : kBwRows;
+        const auto advance = [&](Pos ps) {
+            ++ps.hq;
+            if (ps.hq == G) {
+                ps.hq = 0;
+                ps.r0 += r_step;
+            }
+            return ps;
+        };
         // a step whose rows all lie above this wavefront's first key column has nothing for it (uniform)
-        const auto idle = [&](int st) { return CAUSAL && kw0 > row0(st) + kBwRows - 1 + coff; };
+        const auto idle = [&](Pos ps) { return CAUSAL && kw0 > ps.r0 + kBwRows - 1 + coff; };
 
         float pend_lse = 0.f, pend_delta = 0.f;
-        const auto bases = [&](int st, int64_t& q_base, int64_t& do_base, int64_t& l_base) {
-            const int h = hk * G + st % G;
+        const auto bases = [&](Pos ps, int64_t& q_base, int64_t& do_base, int64_t& l_base) {
+            const int h = hk * G + ps.hq;
             if (p.cu_q) {
                 q_base = (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
                 do_base = (int64_t)q_start * p.dos[2] + (int64_t)h * p.dos[1];
@@ -421,33 +434,33 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
                 l_base = (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1];
             }
         };
-        // Q tile of step st into ring slot `slot`; its lse into a register
-        const auto issue_q = [&](int st, int slot) {
+        // Q tile of step st (at ps) into ring slot `slot`; its lse into a register
+        const auto issue_q = [&](Pos ps, int slot) {
             int64_t q_base, do_base, l_base;
-            bases(st, q_base, do_base, l_base);
-            const int r0 = row0(st);
+            bases(ps, q_base, do_base, l_base);
+            const int r0 = ps.r0;
             ld.issue(p.q + q_base + (int64_t)r0 * p.qs[2], (int)p.qs[2], sq - 1 - r0, dst + slot * kTile);
             const float* rows = p.lse + l_base + r0;                                   // uniform base, 32-bit lane offset
-            if (tid < kBwRows) pend_lse = rows[(unsigned)min(tid, sq - 1 - r0)];                 // consumed only by publish_lse
+            if (tid < kBwRows) pend_lse = rows[(unsigned)min(tid, sq - 1 - r0)];       // consumed only by publish_lse
         };
-        const auto issue_do = [&](int st) {
+        const auto issue_do = [&](int st, Pos ps) {
             int64_t q_base, do_base, l_base;
-            bases(st, q_base, do_base, l_base);
-            const int r0 = row0(st);
+            bases(ps, q_base, do_base, l_base);
+            const int r0 = ps.r0;
             ld.issue(p.dout + do_base + (int64_t)r0 * p.dos[2], (int)p.dos[2], sq - 1 - r0, dst + (3 + (st & 1)) * kTile);
             const float* rows = p.delta + l_base + r0;
             if (tid < kBwRows) pend_delta = rows[(unsigned)min(tid, sq - 1 - r0)];
         };
         // (the values are scaled and masked here, not where they are loaded: consuming them there would put a
         // wait for all outstanding loads - the tiles just issued - in front of the step's arithmetic)
-        const auto publish_lse = [&](int st) {
-            if (tid < kBwRows) lse_lds2[(st & 1) * kBwRows + tid] = row0(st) + tid < sq ? pend_lse * kLog2e : INFINITY;
+        const auto publish_lse = [&](int st, Pos ps) {
+            if (tid < kBwRows) lse_lds2[(st & 1) * kBwRows + tid] = ps.r0 + tid < sq ? pend_lse * kLog2e : INFINITY;
         };
-        const auto publish_delta = [&](int st) {
+        const auto publish_delta = [&](int st, Pos ps) {
             // a causal row that sees no key has out = NaN, hence delta = NaN, and P = 0 everywhere: any finite
             // delta gives the dS = 0 it must have
             if (tid < kBwRows)
-                delta_lds2[(st & 1) * kBwRows + tid] = (row0(st) + tid < sq && pend_delta == pend_delta) ? pend_delta : 0.f;
+                delta_lds2[(st & 1) * kBwRows + tid] = (ps.r0 + tid < sq && pend_delta == pend_delta) ? pend_delta : 0.f;
         };
 
         // second GEMM of either role: acc^T (D x 32 keys) += tile^T . W, 16 query rows at a time.
@@ -487,11 +500,11 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
         };
         // role A: P of step st from the Q tile in ring slot `slot`: fp32 to LDS for role B, bf16 into p_cur
         u32x4 p_cur[4];
-        const auto make_p = [&](int st, int slot) {
+        const auto make_p = [&](int st, Pos ps, int slot) {
             const unsigned char* q_lds = lds + slot * kTile;
             const float* lse_lds = lse_lds2 + (st & 1) * kBwRows;
             unsigned char* out = p_lds + (st & 1) * (kFuPairs * kPSlab);
-            const int row_lim = CAUSAL ? kj - coff - row0(st) - 4 * kg : -1;
+            const int row_lim = CAUSAL ? kj - coff - ps.r0 - 4 * kg : -1;
             // one 32-row half at a time: element i of this lane is query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
@@ -537,29 +550,35 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             update(q_lds, ds);
         };
 
-        // iteration i = -1 .. n_steps-1; ring slots: Q(i) in s_b, Q(i+1) in s_a, Q(i+2) lands in s_l
+        // iteration i = -1 .. n_steps-1; ring slots: Q(i) in s_b, Q(i+1) in s_a, Q(i+2) lands in s_l;
+        // positions: ps0 of step i, ps1 of step i+1, ps2 of step i+2
+        Pos ps1 = {(half == 0 ? n_tiles - 1 : first_tile) * kBwRows, 0};
+        Pos ps0 = ps1, ps2 = advance(ps1);
         if (n_steps > 0) {
-            issue_q(0, 0);
-            publish_lse(0);
+            issue_q(ps1, 0);
+            publish_lse(0, ps1);
         }
         int s_b = 2, s_a = 0, s_l = 1;
         for (int i = -1; i < n_steps; ++i) {
             wait_vmcnt<0>();                                   // this wavefront's share of the tiles issued one iteration ago has landed
             __syncthreads();                                   // ... and everybody's; P(i), lse(i+1), delta(i) are visible; older buffers are free
-            if (i + 2 < n_steps) issue_q(i + 2, s_l);
-            if (i + 1 < n_steps) issue_do(i + 1);
+            if (i + 2 < n_steps) issue_q(ps2, s_l);
+            if (i + 1 < n_steps) issue_do(i + 1, ps1);
             if (!role_b) {
-                if (i >= 0 && !idle(i)) update(lds + (3 + (i & 1)) * kTile, p_cur);      // dV^T += dO(i)^T P(i)
-                if (i + 1 < n_steps && !idle(i + 1)) make_p(i + 1, s_a);
+                if (i >= 0 && !idle(ps0)) update(lds + (3 + (i & 1)) * kTile, p_cur);      // dV^T += dO(i)^T P(i)
+                if (i + 1 < n_steps && !idle(ps1)) make_p(i + 1, ps1, s_a);
             } else {
-                if (i >= 0 && !idle(i)) step_b(i, s_b);
+                if (i >= 0 && !idle(ps0)) step_b(i, s_b);
             }
-            if (i + 2 < n_steps) publish_lse(i + 2);
-            if (i + 1 < n_steps) publish_delta(i + 1);
+            if (i + 2 < n_steps) publish_lse(i + 2, ps2);
+            if (i + 1 < n_steps) publish_delta(i + 1, ps1);
             const int t3 = s_b;
             s_b = s_a;
             s_a = s_l;
             s_l = t3;
+            ps0 = ps1;
+            ps1 = ps2;
+            ps2 = advance(ps2);
         }
 
         // store: lane owns key kj, d = 32dt + 8(i/4) + 4kg + i%4
