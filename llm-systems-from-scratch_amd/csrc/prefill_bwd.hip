@@ -559,17 +559,14 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             publish_lse(0, ps1);
         }
         int s_b = 2, s_a = 0, s_l = 1;
-        for (int i = -1; i < n_steps; ++i) {
+        // what every wavefront does around its role's work in an iteration (the same number of barriers in both loops)
+        const auto open_iteration = [&](int i) {
             wait_vmcnt<0>();                                   // this wavefront's share of the tiles issued one iteration ago has landed
             __syncthreads();                                   // ... and everybody's; P(i), lse(i+1), delta(i) are visible; older buffers are free
             if (i + 2 < n_steps) issue_q(ps2, s_l);
             if (i + 1 < n_steps) issue_do(i + 1, ps1);
-            if (!role_b) {
-                if (i >= 0 && !idle(ps0)) update(lds + (3 + (i & 1)) * kTile, p_cur);      // dV^T += dO(i)^T P(i)
-                if (i + 1 < n_steps && !idle(ps1)) make_p(i + 1, ps1, s_a);
-            } else {
-                if (i >= 0 && !idle(ps0)) step_b(i, s_b);
-            }
+        };
+        const auto close_iteration = [&](int i) {
             if (i + 2 < n_steps) publish_lse(i + 2, ps2);
             if (i + 1 < n_steps) publish_delta(i + 1, ps1);
             const int t3 = s_b;
@@ -579,6 +576,22 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             ps0 = ps1;
             ps1 = ps2;
             ps2 = advance(ps2);
+        };
+        // One loop per role: in a shared loop the accumulators of the two branches meet again after every
+        // iteration, and the compiler then copies all 64 of them, and more, each time round.
+        if (!role_b) {
+            for (int i = -1; i < n_steps; ++i) {
+                open_iteration(i);
+                if (i >= 0 && !idle(ps0)) update(lds + (3 + (i & 1)) * kTile, p_cur);      // dV^T += dO(i)^T P(i)
+                if (i + 1 < n_steps && !idle(ps1)) make_p(i + 1, ps1, s_a);
+                close_iteration(i);
+            }
+        } else {
+            for (int i = -1; i < n_steps; ++i) {
+                open_iteration(i);
+                if (i >= 0 && !idle(ps0)) step_b(i, s_b);
+                close_iteration(i);
+            }
         }
 
         // store: lane owns key kj, d = 32dt + 8(i/4) + 4kg + i%4
