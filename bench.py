@@ -264,8 +264,8 @@ def bench_decode_loop(args):
         sd[pre + "ffn_norm.weight"] = torch.ones(d)
     B, prompt_len, n_steps = 8, 32, min(200, cfg["context_length"] - 33)
     res = {"config": {"workload": f"decode steps of the KV-cached decoder, reference sample model {cfg}, batch {B}, "
-                                  f"prompt {prompt_len}, {n_steps} timed steps, greedy tokens fed back on the device side "
-                                  "of the host loop", "model": "random weights"}}
+                                  f"prompt {prompt_len}, {n_steps} timed steps, greedy tokens fed back through the host",
+                       "weights": "random"}}
     for name, graphs in (("eager", False), ("hip_graph", True)):
         model = mi355_attn.CachedTransformerLM(cfg, sd, max_batch=B, decode_graphs=graphs)
         sids = [model.new_sequence() for _ in range(B)]
