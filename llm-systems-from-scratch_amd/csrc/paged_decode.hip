@@ -24,6 +24,8 @@
 // chunk is normalised and written straight to `out`, otherwise the chunk's
 // partial goes to the workspace and the combine kernel finishes it:
 //   o = sum_c 2^(m_c - m) o_c / sum_c 2^(m_c - m) l_c      (m = max_c m_c).
+#include <type_traits>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -192,9 +194,11 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
         load_v(0);
         load_k(0);
     }
-    for (int it = 0; it < n_iter; ++it) {
+    // One step; TAIL selects the code that blanks the keys past the end of the range (only the last step
+    // of a wavefront can need it, so the other steps carry no compare/select per element).
+    const auto step = [&](int it, auto tail_c) {
+        constexpr bool tail = decltype(tail_c)::value;
         const int kbase = t0 + it * kStage;
-        const bool tail = kbase + kStage > t1;
 
         // ---- V: registers -> wavefront-private LDS tile (bf16, row = key) --
 #pragma unroll
@@ -320,6 +324,11 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
         // optimiser turns "phi of loads" into "load of phi" and the loads land at the top of
         // the NEXT iteration, i.e. the prefetch is undone.
         asm volatile("" ::: "memory");
+    };
+    for (int it = 0; it + 1 < n_iter; ++it) step(it, std::false_type{});
+    if (n_iter > 0) {
+        if ((t1 - t0) % kStage == 0) step(n_iter - 1, std::false_type{});
+        else step(n_iter - 1, std::true_type{});
     }
 
     // ---- merge the four wavefronts ------------------------------------------
