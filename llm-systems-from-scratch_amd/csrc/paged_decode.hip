@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
         }
     };
 
-    float m_run = -INFINITY;      // running max (log2 domain) of this lane's query column
+    float m_run = -INFINITY;      // exponent reference (log2 domain) of this lane's query column: >= its running max - slack
     float l_run = 0.0f;           // this lane's share of the running sum
     f32x4 o[NT];
 #pragma unroll
@@ -292,18 +292,25 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void paged_decode_split_kernel(D
             }
         }
         mx = xor_max_16_32(mx);
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = fast_exp2(m_run - m_new);
-        m_run = m_new;
+        // Lazy rescaling: m_run is the exponent reference, not the running maximum; it moves only when some
+        // query's maximum outgrows it by more than 2^kSlack (weights up to 2^kSlack are exact in the fp32
+        // sums and harmless in bf16), so the common step neither multiplies O nor touches l.
+        constexpr float kSlack = 8.0f;
+        if (__builtin_amdgcn_ballot_w64(!(mx - m_run <= kSlack)) != 0) {       // also taken while m_run = -inf
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = m_new == -INFINITY ? 1.0f : fast_exp2(m_run - m_new);   // 0 the first time a key is seen
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int i = 0; i < NT; ++i) o[i] *= alpha;
+        }
         float psum = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            x[i] = fast_exp2(x[i] - m_new);
+            x[i] = fast_exp2(x[i] - m_run);
             psum += x[i];
         }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int i = 0; i < NT; ++i) o[i] *= alpha;
+        l_run += psum;
         u32x4 pp;
         pp[0] = pack_bf16(x[0] * vs2[0], x[1] * vs2[0]);
         pp[1] = pack_bf16(x[2] * vs2[0], x[3] * vs2[0]);
