@@ -46,7 +46,7 @@ __device__ __forceinline__ void load_weight8(const RmsNormParams& p, int col, fl
 // One wavefront per row, the row held in registers: NCHUNK chunks of 512 elements (8 per lane).
 // Requires n_cols % 8 == 0, n_cols <= 512 * NCHUNK, 16-byte aligned rows.
 template <int NCHUNK>
-__global__ __launch_bounds__(256) void rms_norm_rows_kernel(RmsNormParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void rms_norm_rows_kernel(RmsNormParams p) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= p.n_rows) return;
