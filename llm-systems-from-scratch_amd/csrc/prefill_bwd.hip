@@ -202,11 +202,16 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
 #pragma unroll
             for (int j = 0; j < 16; ++j) dq[i][j] = 0.f;
         const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        // dP - delta comes straight out of the MFMAs: -delta (one value per lane: its query) is their C operand
+        f32x16 neg_delta16;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) neg_delta16[j] = -delta;
 
         int kv_end = sk;
         if (CAUSAL) kv_end = max(0, min(sk, min(sq, q0 + kBwCols) + coff));
         const int n_tiles = (kv_end + kBwRows - 1) / kBwRows;
         const int last_key = CAUSAL ? min(sk - 1, qi + coff) : sk - 1;      // last key this lane's query sees
+        const int wave_last_key = CAUSAL ? min(sk - 1, qw0 + coff) : sk - 1;   // ... and the last one ALL queries of the wavefront see
         const auto issue = [&](int tile) {
             const int r0 = tile * kBwRows, buf = (tile & 1) * kTile;
             ld.issue(p.k + k_base + (int64_t)r0 * p.ks[2], (int)p.ks[2], sk - 1 - r0, dst + buf);
@@ -217,11 +222,11 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
         // and the wavefront then sits through the LDS latency once per MFMA.
         constexpr int kDepth = 2;
         // (32 rows of the tile at a_lds) x (this lane's query column, fragments b)
-        const auto scores = [&](const unsigned char* a_lds, const bf16x8 (&bfr)[NS]) {
+        const auto scores = [&](const unsigned char* a_lds, const bf16x8 (&bfr)[NS], const f32x16& c0) {
             u32x4 a[NS];
 #pragma unroll
             for (int s = 0; s < kDepth && s < NS; ++s) a[s] = *reinterpret_cast<const u32x4*>(a_lds + rd.row_off[s]);
-            f32x16 r = zero16;
+            f32x16 r = c0;
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 if (s + kDepth < NS) a[s + kDepth] = *reinterpret_cast<const u32x4*>(a_lds + rd.row_off[s + kDepth]);
@@ -240,13 +245,13 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
             // one 32-key half at a time: element i of this lane is key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                const f32x16 s_acc = scores(k_lds + t * 32 * kRow, qf);
-                const f32x16 dp_acc = scores(v_lds + t * 32 * kRow, dof);
+                const f32x16 s_acc = scores(k_lds + t * 32 * kRow, qf, zero16);
+                const f32x16 dp_acc = scores(v_lds + t * 32 * kRow, dof, neg_delta16);             // dP - delta
                 float x[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const float pr = fast_exp2(fmaf(s_acc[i], p.scale_log2, -lse2));
-                    x[i] = pr * (dp_acc[i] - delta);                                   // dS (without the scale factor)
+                    x[i] = pr * dp_acc[i];                                             // dS (without the scale factor)
                     if constexpr (MASKED) {
                         // key index relative to the tile (compile-time part) against this lane's last visible key
                         x[i] = (32 * t + 8 * (i >> 2) + (i & 3) <= key_lim) ? x[i] : 0.f;
@@ -276,10 +281,20 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
             }
         };
 
+        // Two loops over the tile stream: first the tiles that every query of the wavefront sees in full, then
+        // those that reach past wave_last_key (the diagonal, a ragged end), which run the instantiation with the
+        // per-element compare/select.  (Two loops, not a branch in one: each loop body is scheduled on its own.)
+        const int n_full = min(n_tiles, max(0, wave_last_key + 1) / kBwRows);
         if (n_tiles > 0) issue(0);
-        for (int tile = 0; tile < n_tiles; ++tile) {
+        for (int tile = 0; tile < n_full; ++tile) {
             wait_vmcnt<0>();                                   // this wavefront's share of tile `tile` has landed
             __syncthreads();                                   // ... and everybody's; all are done reading the other buffer
+            if (tile + 1 < n_tiles) issue(tile + 1);
+            step(std::false_type{}, tile);
+        }
+        for (int tile = n_full; tile < n_tiles; ++tile) {
+            wait_vmcnt<0>();
+            __syncthreads();
             if (tile + 1 < n_tiles) issue(tile + 1);
             if (CAUSAL && tile * kBwRows > qw0 + 31 + coff) continue;      // wholly above this wavefront's diagonal (uniform)
             step(std::true_type{}, tile);
@@ -421,7 +436,7 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
         // a step whose rows all lie above this wavefront's first key column has nothing for it (uniform)
         const auto idle = [&](Pos ps) { return CAUSAL && kw0 > ps.r0 + kBwRows - 1 + coff; };
 
-        float pend_lse = 0.f, pend_delta = 0.f;
+        float pend_lse = 0.f, pend_delta = 0.f;      // (delta_lds2 holds -delta)
         const auto bases = [&](Pos ps, int64_t& q_base, int64_t& do_base, int64_t& l_base) {
             const int h = hk * G + ps.hq;
             if (p.cu_q) {
@@ -460,7 +475,7 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             // a causal row that sees no key has out = NaN, hence delta = NaN, and P = 0 everywhere: any finite
             // delta gives the dS = 0 it must have
             if (tid < kBwRows)
-                delta_lds2[(st & 1) * kBwRows + tid] = (ps.r0 + tid < sq && pend_delta == pend_delta) ? pend_delta : 0.f;
+                delta_lds2[(st & 1) * kBwRows + tid] = (ps.r0 + tid < sq && pend_delta == pend_delta) ? -pend_delta : 0.f;
         };
 
         // second GEMM of either role: acc^T (D x 32 keys) += tile^T . W, 16 query rows at a time.
@@ -485,11 +500,11 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             }
         };
         // first GEMM of either role: (32 rows of the tile at a_lds) x (this lane's key column), fragments read ahead likewise
-        const auto scores = [&](const unsigned char* a_lds) {
+        const auto scores = [&](const unsigned char* a_lds, const f32x16& c0) {
             u32x4 a[NS];
 #pragma unroll
             for (int s = 0; s < kDepth && s < NS; ++s) a[s] = *reinterpret_cast<const u32x4*>(a_lds + rd.row_off[s]);
-            f32x16 r = zero16;
+            f32x16 r = c0;
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
                 if (s + kDepth < NS) a[s + kDepth] = *reinterpret_cast<const u32x4*>(a_lds + rd.row_off[s + kDepth]);
@@ -500,7 +515,8 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
         };
         // role A: P of step st from the Q tile in ring slot `slot`: fp32 to LDS for role B, bf16 into p_cur
         u32x4 p_cur[4];
-        const auto make_p = [&](int st, Pos ps, int slot) {
+        const auto make_p = [&](auto masked_c, int st, Pos ps, int slot) {
+            constexpr bool MASKED = decltype(masked_c)::value;
             const unsigned char* q_lds = lds + slot * kTile;
             const float* lse_lds = lse_lds2 + (st & 1) * kBwRows;
             unsigned char* out = p_lds + (st & 1) * (kFuPairs * kPSlab);
@@ -508,7 +524,7 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             // one 32-row half at a time: element i of this lane is query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                const f32x16 s_acc = scores(q_lds + t * 32 * kRow);
+                const f32x16 s_acc = scores(q_lds + t * 32 * kRow, zero16);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_lds + 32 * t + 8 * j + 4 * kg);
@@ -517,7 +533,7 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
                     for (int r = 0; r < 4; ++r) {
                         float x = fast_exp2(fmaf(s_acc[4 * j + r], p.scale_log2, -l4[r]));
                         // kept iff kj <= row + coff, i.e. the tile-relative row (compile-time part) >= row_lim
-                        if (CAUSAL) x = (32 * t + 8 * j + r >= row_lim) ? x : 0.f;
+                        if constexpr (MASKED) x = (32 * t + 8 * j + r >= row_lim) ? x : 0.f;
                         x4[r] = x;
                     }
                     *reinterpret_cast<f32x4*>(out + (4 * t + j) * 1024) = x4;
@@ -535,14 +551,21 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             u32x4 ds[4];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                const f32x16 dp_acc = scores(do_lds + t * 32 * kRow);
+                // dP - delta comes straight out of the MFMAs: the -delta of the rows (as published) is their C operand
+                f32x16 c0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_lds + 32 * t + 8 * j + 4 * kg);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) c0[4 * j + r] = d4[r];
+                }
+                const f32x16 dp_acc = scores(do_lds + t * 32 * kRow, c0);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const f32x4 p4 = *reinterpret_cast<const f32x4*>(in + (4 * t + j) * 1024);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_lds + 32 * t + 8 * j + 4 * kg);
                     float x[4];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) x[r] = p4[r] * (dp_acc[4 * j + r] - d4[r]);      // dS without the scale factor
+                    for (int r = 0; r < 4; ++r) x[r] = p4[r] * dp_acc[4 * j + r];                 // dS without the scale factor
                     ds[2 * t + (j >> 1)][2 * (j & 1)] = pack_bf16(x[0], x[1]);
                     ds[2 * t + (j >> 1)][2 * (j & 1) + 1] = pack_bf16(x[2], x[3]);
                 }
@@ -583,7 +606,7 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             for (int i = -1; i < n_steps; ++i) {
                 open_iteration(i);
                 if (i >= 0 && !idle(ps0)) update(lds + (3 + (i & 1)) * kTile, p_cur);      // dV^T += dO(i)^T P(i)
-                if (i + 1 < n_steps && !idle(ps1)) make_p(i + 1, ps1, s_a);
+                if (i + 1 < n_steps && !idle(ps1)) make_p(std::integral_constant<bool, CAUSAL>{}, i + 1, ps1, s_a);
                 close_iteration(i);
             }
         } else {
