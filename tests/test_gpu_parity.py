@@ -96,6 +96,39 @@ def test_decode_long_contexts_multi_chunk(ops, fp8):
     check(got, ref, what=f"long contexts fp8={fp8}")
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("slope", [0.4, 0.02, -0.02, -0.4])
+def test_decode_scores_that_ramp_along_the_context(ops, fp8, slope):
+    """Scores that rise (or fall) steadily with the token position, by much more or much less per 32-key step than
+    the slack of the kernel's lazily moved exponent reference, plus one isolated spike in the middle: the output
+    must follow the oracle whether the reference moves every step, every few steps or never."""
+    ctx = [40, 700, 2500, 5000]
+    D, Hq, Hkv = 128, 4, 2
+    print(f"case: decode ramp slope={slope} fp8={fp8}", flush=True)
+    q, kc, vc, bt, cl = orc.make_paged_case(batch=len(ctx), n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                            context_lens=ctx, pool_factor=1.2, seed=31, dtype=torch.bfloat16)
+    q = (q.float() * 0.05)
+    q[:, :, 0] = math.sqrt(D)                     # score of token t = K[t, 0] + small noise (scale 1/sqrt(D))
+    q[:, 1::2, 0] = -math.sqrt(D)                 # every other query head sees the ramp the other way round
+    q = q.to(torch.bfloat16)
+    for b, n in enumerate(ctx):
+        t = torch.arange(n, dtype=torch.float32)
+        col = slope * t
+        col[n // 2] += 30.0 if slope > 0 else -30.0            # a spike (for the odd heads: a dip)
+        for j in range((n + 15) // 16):
+            rows = col[16 * j:16 * j + 16]
+            kc[int(bt[b, j]), :, :rows.numel(), 0] = rows.to(torch.bfloat16)[None]
+    if fp8:
+        k8, ks = orc.quantize_kv_fp8(kc)
+        v8, vs = orc.quantize_kv_fp8(vc)
+        got = run_decode(ops, q, k8, v8, bt, cl, k_scale=ks, v_scale=vs)
+        ref = orc.paged_decode_reference(q, k8, v8, bt, cl, k_scale=ks, v_scale=vs)
+    else:
+        got = run_decode(ops, q, kc, vc, bt, cl)
+        ref = orc.paged_decode_reference(q, kc, vc, bt, cl)
+    check(got, ref, what=f"ramp slope={slope} fp8={fp8}")
+
+
 def test_decode_ignores_pool_garbage_and_table_tail(ops):
     """NaN/Inf bit patterns in unused blocks, in the tail of the last block and junk table entries are never used."""
     ctx = [5, 40, 100, 1030]
