@@ -390,33 +390,47 @@ void paged_decode_split_kernel(DecodeParams p) {
     }
 }
 
+// Combine: one thread per (row = sequence x query head, 4 adjacent d), 256 / (D / 4) rows per workgroup.
+constexpr int kCombineThreads = 256;
+
 template <int D>
-__global__ __launch_bounds__(D) void paged_decode_combine_kernel(DecodeParams p) {
-    const int row = blockIdx.x;                  // b * Hq + h
+__global__ __launch_bounds__(kCombineThreads) void paged_decode_combine_kernel(DecodeParams p) {
+    constexpr int kLanesPerRow = D / 4;
+    const int row = blockIdx.x * (kCombineThreads / kLanesPerRow) + threadIdx.x / kLanesPerRow;      // b * Hq + h
+    if (row >= p.B * p.Hq) return;
     const int b = row / p.Hq;
     const int ctx = min(p.context_lens[b], p.max_ctx);
     const int chunk_tokens = kDecodeWaves * p.tokens_per_wave;
     const int n_chunks = (ctx + chunk_tokens - 1) / chunk_tokens;
     if (n_chunks <= 1) return;                   // written by the split pass (or empty)
-    const int d = threadIdx.x;
+    const int d = (threadIdx.x % kLanesPerRow) * 4;
     const int64_t base = (int64_t)row * p.max_chunks;
     float M = -INFINITY;
     for (int c = 0; c < n_chunks; ++c) M = fmaxf(M, p.ws_m[base + c]);
-    float num = 0.f, den = 0.f;
+    f32x4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
     for (int c = 0; c < n_chunks; ++c) {
         const float f = fast_exp2(p.ws_m[base + c] - M);
-        num += f * p.ws_o[(base + c) * D + d];
+        const f32x4 o = *reinterpret_cast<const f32x4*>(p.ws_o + (base + c) * D + d);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) num[i] += f * o[i];
         den += f * p.ws_l[base + c];
     }
-    p.out[(int64_t)row * D + d] = (__bf16)(num / den);
+    u32x2 w;
+    w[0] = pack_bf16(num[0] / den, num[1] / den);
+    w[1] = pack_bf16(num[2] / den, num[3] / den);
+    *reinterpret_cast<u32x2*>(p.out + (int64_t)row * D + d) = w;
 }
 
 template <int D, bool FP8>
 static int launch_decode(const DecodeParams& p, hipStream_t stream) {
     dim3 grid((unsigned)p.max_chunks * p.Hkv * p.B);
     hipLaunchKernelGGL((paged_decode_split_kernel<D, FP8>), grid, dim3(kDecodeWaves * 64), 0, stream, p);
-    if (p.max_chunks > 1)
-        hipLaunchKernelGGL((paged_decode_combine_kernel<D>), dim3(p.B * p.Hq), dim3(D), 0, stream, p);
+    if (p.max_chunks > 1) {
+        const int rows_per_wg = kCombineThreads / (D / 4);
+        hipLaunchKernelGGL((paged_decode_combine_kernel<D>), dim3((p.B * p.Hq + rows_per_wg - 1) / rows_per_wg),
+                           dim3(kCombineThreads), 0, stream, p);
+    }
     return (int)hipGetLastError();
 }
 
