@@ -348,3 +348,28 @@ def test_ops_reject_tensors_on_different_devices(ops):
     q = rnd(1, 2, 16, 64, seed=1).cuda()
     with pytest.raises(ValueError):
         ops.flash_attn_prefill(q, q.cpu(), q)
+
+
+def test_ops_run_on_the_current_stream(ops):
+    """The wrappers hand torch's CURRENT stream to the library: inside `torch.cuda.stream(s)` the kernels are ordered
+    after the work already queued on s (here a chain of matrix products that takes milliseconds and whose result the
+    inputs depend on) and give exactly what the default stream gives."""
+    print("case: non-default stream", flush=True)
+    dev = "cuda:0"
+    q, k, v = (rnd(2, 4, 300, 64, seed=s, scale=0.5).to(dev) for s in (1, 2, 3))
+    dq, kc, vc, bt, cl = (t.to(dev) for t in orc.make_paged_case(batch=3, n_q_heads=8, n_kv_heads=2, head_dim=128, block_size=16,
+                                                                 context_lens=[700, 5000, 33], seed=9, dtype=torch.bfloat16))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        a = torch.randn(2048, 2048, device=dev)
+        for _ in range(30):
+            a = torch.tanh(a @ a)
+        zero = (a[0, 0] * 0).to(torch.bfloat16)          # 0, available only when the chain has finished
+        out_p = ops.flash_attn_prefill(q + zero, k, v, causal=True)
+        out_d = ops.paged_attention_decode(dq + zero, kc, vc, bt, cl)
+    side.synchronize()
+    ref_p = ops.flash_attn_prefill(q, k, v, causal=True)
+    ref_d = ops.paged_attention_decode(dq, kc, vc, bt, cl)
+    torch.cuda.synchronize()
+    assert torch.equal(out_p, ref_p) and torch.equal(out_d, ref_d)
