@@ -65,6 +65,12 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
 
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kTile];
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kTile];
+    // Staging of the query rows on their way in and of the output rows on their way out, one private slab per
+    // wavefront (32 rows of D bf16, rows padded by 16 bytes): fragments and accumulators hold a query per lane,
+    // so direct accesses would touch 16- or 8-byte pieces of 32 different rows per instruction; through the
+    // slab every global instruction moves whole 2*D-byte rows (+2.4 % for the stores alone at D = 128).
+    constexpr int kORow = D * 2 + 16;
+    __shared__ __attribute__((aligned(16))) unsigned char o_lds[kPfWaves * 32 * kORow];
 
     // Workgroup ids are dealt round-robin to the 8 XCDs, each with a private L2.  The id is
     // remapped so that every XCD works through a contiguous range of the logical order
@@ -186,13 +192,31 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
         if (causal) kv_end = max(0, min(sk, min(sq, q0 + kBM) + coff));
         const int n_tiles = (kv_end + kBN - 1) / kBN;
 
+        // the first K/V tile is requested before the query rows, so that the two latencies overlap
+        __syncthreads();                     // the previous query tile's readers are done with the LDS buffers
+        if (n_tiles > 0) issue_tile(0, 0);
+
         // ---- Q^T fragments: step s covers d = 16s + 8kg + j ----------------------
+        // rows come in whole (CPR lanes per row) and go through the wavefront's slab (private, and LDS operations
+        // of a wavefront execute in order: no barrier); rows past the end of the sequence are zero
         bf16x8 qf[NS];
+        {
+            unsigned char* slab = o_lds + wave * (32 * kORow);
+            constexpr int kRowsPerPass = 64 / CPR;
+            const int c = lane % CPR, r0 = lane / CPR;
+            u32x4 rows[32 / kRowsPerPass];
 #pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            u32x4 t = {0u, 0u, 0u, 0u};
-            if (q_ok) t = *reinterpret_cast<const u32x4*>(qb + (int64_t)qi * p.qs[2] + 16 * s + 8 * kg);
-            qf[s] = as_bf16x8(t);
+            for (int i = 0; i < 32 / kRowsPerPass; ++i) {
+                const int r = i * kRowsPerPass + r0;
+                rows[i] = u32x4{0u, 0u, 0u, 0u};
+                if (qw0 + r < sq) rows[i] = *reinterpret_cast<const u32x4*>(qb + (int64_t)(qw0 + r) * p.qs[2] + c * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 32 / kRowsPerPass; ++i)
+                *reinterpret_cast<u32x4*>(slab + (i * kRowsPerPass + r0) * kORow + c * 16) = rows[i];
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                qf[s] = as_bf16x8(*reinterpret_cast<const u32x4*>(slab + n * kORow + (16 * s + 8 * kg) * 2));
         }
 
         f32x16 o[NDT];
@@ -336,8 +360,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
             }
         };
 
-        __syncthreads();                     // the previous query tile's readers are done with the LDS buffers
-        if (n_tiles > 0) issue_tile(0, 0);
         run_tiles(std::false_type{}, 0, n_plain);
         run_tiles(std::true_type{}, n_plain, n_tiles);
         if (n_tiles & 1) flip();             // leave the offsets pointing at buffer 0 for the next query tile
@@ -348,8 +370,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
         // sum_j exp(scale * s_j) = 2^(m_ref * scale_log2) * l  ->  lse = ln2 * (m_ref * scale_log2 + log2 l)
         if (lb && q_ok && kg == 0)
             lb[qi] = l_run > 0.f ? 0.69314718056f * (m_ref * p.scale_log2 + __log2f(l_run)) : -INFINITY;
-        if (q_ok) {
-            __bf16* orow = ob + (int64_t)qi * p.os[2];
+        {
+            // (the slab is private to the wavefront and LDS operations of a wavefront execute in order: no barrier)
+            unsigned char* slab = o_lds + wave * (32 * kORow);
+            unsigned char* mine = slab + n * kORow + 8 * kg;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
@@ -357,8 +381,17 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
                     u32x2 w;
                     w[0] = pack_bf16(o[dt][4 * g + 0] * inv, o[dt][4 * g + 1] * inv);
                     w[1] = pack_bf16(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
-                    *reinterpret_cast<u32x2*>(orow + 32 * dt + 8 * g + 4 * kg) = w;
+                    *reinterpret_cast<u32x2*>(mine + (32 * dt + 8 * g) * 2) = w;
                 }
+            // read back row-wise: 16-byte chunk c of row r, CPR lanes per row
+            constexpr int kRowsPerPass = 64 / CPR;
+            const int c = lane % CPR, r0 = lane / CPR;
+#pragma unroll
+            for (int i = 0; i < 32 / kRowsPerPass; ++i) {
+                const int r = i * kRowsPerPass + r0;
+                const u32x4 w = *reinterpret_cast<const u32x4*>(slab + r * kORow + c * 16);
+                if (qw0 + r < sq) *reinterpret_cast<u32x4*>(ob + (int64_t)(qw0 + r) * p.os[2] + c * 8) = w;
+            }
         }
     }
 }
