@@ -43,10 +43,15 @@ def _traffic(key):
         return None
 
 
-def timed(fn, steps, warmup):
-    """Returns (wall ms/step, device ms/step): K launches between two syncs, HIP events on the launch stream."""
+BURN_IN = 40        # untimed launches in front of the warm-up of an MFMA-bound leg (disclosed in the JSON line)
+
+
+def timed(fn, steps, warmup, burn_in=0):
+    """Returns (wall ms/step, device ms/step): K launches between two syncs, HIP events on the launch stream.
+    `burn_in` extra untimed launches come first: the shader clock needs some tens of milliseconds of MFMA load
+    to leave its idle state, which a short warm-up does not give an MFMA-bound kernel."""
     import torch
-    for _ in range(warmup):
+    for _ in range(burn_in + warmup):
         fn()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
@@ -61,12 +66,15 @@ def timed(fn, steps, warmup):
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
 
-def bench_decode(cfg, args, with_cpu):
+CPU_SAMPLE_SEQS = 128      # sequences of a decode configuration that the CPU oracle is run (and timed) on
+
+
+def bench_decode(cfg, args, with_cpu=False):
     import torch
     import mi355_attn
     from mi355_attn import workloads
 
-    case = workloads.decode_config(cfg, seed=args.seed)
+    case = workloads.decode_config(cfg, seed=args.seed, keep_bf16_seqs=CPU_SAMPLE_SEQS if with_cpu else 0)
     B, Hq, D = case.q.shape
     ws = mi355_attn.paged_decode_workspace(B, Hq, D, case.max_context, case.q.device)
     out = torch.empty_like(case.q)
@@ -91,9 +99,7 @@ def bench_decode(cfg, args, with_cpu):
             "traffic": _traffic(f"decode_cfg{cfg}"),
         },
     }
-    if with_cpu:
-        res["cpu_baseline"], res["parity"] = cpu_decode(case, out, cfg)
-    return res
+    return res, (case, out)
 
 
 def bench_prefill_backward(cfg, args):
@@ -114,7 +120,7 @@ def bench_prefill_backward(cfg, args):
     dout = torch.randn(out.shape, device=out.device, generator=g).to(torch.bfloat16)
     scale = 1.0 / (case.q.shape[-1] ** 0.5)
     wall_ms, dev_ms = timed(lambda: ops._prefill_backward(case.q, case.k, case.v, out, dout, lse, cu, cu, S, S, scale, 1),
-                            args.steps, args.warmup)
+                            args.steps, args.warmup, BURN_IN)
     flops = case.flops() * 5 // 2
     return {
         "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
@@ -297,7 +303,12 @@ def _timed_repeats(fn, min_seconds=10.0, max_reps=20):
     return out, total / reps, reps
 
 
-def cpu_decode(case, gpu_out, cfg, n_seq=128):
+# Quantisation-error bound of the fp8-KV decode against a bf16-KV fp32-math reference (e4m3 rounds with relative
+# error <= 2^-4): per element |out - ref| <= 0.15 + 2^-4 |ref|, and rms(out - ref) <= 6 % of rms(ref).
+FP8_ATOL, FP8_RTOL, FP8_RMS = 0.15, 2.0 ** -4, 0.06
+
+
+def cpu_decode(case, gpu_out, cfg, n_seq=CPU_SAMPLE_SEQS):
     """Oracle on the host cores over the first n_seq sequences; also checks the GPU result of those."""
     import torch
     from oracle import attention_oracle as orc
@@ -320,7 +331,8 @@ def cpu_decode(case, gpu_out, cfg, n_seq=128):
     ref, dt, reps = _timed_repeats(lambda: orc.paged_decode_reference(q, kc, vc, bt, ctx, k_scale=ks, v_scale=vs))
     per_token = 2 * kc.shape[1] * kc.shape[3] * kc.element_size() + (8 * kc.shape[1] / 16 if ks is not None else 0)
     sample_bytes = int(ctx.sum()) * per_token
-    err = (gpu_out[:n_seq].float().cpu() - ref).abs()
+    got = gpu_out[:n_seq].float().cpu()
+    err = (got - ref).abs()
     bound = 2e-2 + 1e-2 * ref.abs()
     base = {"value": sample_bytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
             "seconds_per_pass": dt, "passes": reps,
@@ -328,10 +340,63 @@ def cpu_decode(case, gpu_out, cfg, n_seq=128):
                       f"{reps} passes of oracle paged_decode_reference, torch CPU fp32"}
     parity = {"checked_sequences": n_seq, "max_abs_err": float(err.max()),
               "within_2e-2_abs_1e-2_rel": bool((err <= bound).all())}
-    return base, parity
+    if ks is not None:
+        parity["reference"] = "oracle on the dequantised fp8 cache (kernel parity)"
+    extra = None
+    if case.k_bf16_sample is not None and case.bf16_sample_seqs >= n_seq:
+        # the configuration's own error metric: fp8-KV result against fp32 math on the bf16 cache it was quantised from
+        n_ids = int(nblk.sum())
+        ref16 = orc.paged_decode_reference(q, case.k_bf16_sample[:n_ids].cpu(), case.v_bf16_sample[:n_ids].cpu(), bt, ctx)
+        e16 = (got - ref16).abs()
+        rms = float((got - ref16).pow(2).mean().sqrt() / ref16.pow(2).mean().sqrt())
+        extra = {"reference": "oracle (fp32 math) on the bf16 cache before quantisation", "checked_sequences": n_seq,
+                 "max_abs_err": float(e16.max()), "rms_err_over_rms_ref": rms,
+                 "bound": f"|err| <= {FP8_ATOL} + 2^-4 |ref| and rms ratio <= {FP8_RMS}",
+                 "within_bound": bool((e16 <= FP8_ATOL + FP8_RTOL * ref16.abs()).all()) and rms <= FP8_RMS}
+    return base, parity, extra
 
 
-def bench_prefill(cfg, args, with_cpu):
+def cpu_config0(args):
+    """configs[0] is the reference's own CPU-runnable case (fp32, B4, 8 = 8 heads, D64, ctx 256): the oracle is timed
+    on it (1 warm-up, best of 3) and the HIP kernel is run on the same (bf16-rounded) inputs as a parity and latency
+    figure; the working set is cache-resident on the GPU, so no roofline is claimed for it."""
+    import torch
+    import mi355_attn
+    from oracle import attention_oracle as orc
+
+    q, kc, vc, bt, cl = orc.make_paged_case(batch=4, n_q_heads=8, n_kv_heads=8, head_dim=64, block_size=16,
+                                            context_lens=[256] * 4, seed=args.seed, dtype=torch.float32)
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    orc.paged_decode_reference(q, kc, vc, bt, cl)
+    best = float("inf")
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ref = orc.paged_decode_reference(q, kc, vc, bt, cl)
+        best = min(best, time.perf_counter() - t0)
+    nbytes = int(cl.sum()) * 2 * 8 * 64 * 4
+    dev = "cuda:0"
+    qb, kb, vb = (t.to(torch.bfloat16) for t in (q, kc, vc))
+    args_gpu = [t.to(dev) for t in (qb, kb, vb, bt, cl)]
+    ws = mi355_attn.paged_decode_workspace(4, 8, 64, 256, dev)
+    out = torch.empty_like(args_gpu[0])
+    wall_ms, dev_ms = timed(lambda: mi355_attn.paged_attention_decode(*args_gpu, max_context=256, workspace=ws, out=out),
+                            args.steps, args.warmup)
+    ref16 = orc.paged_decode_reference(qb, kb, vb, bt, cl)
+    err = (out.float().cpu() - ref16).abs()
+    return {"config": {"workload": "configs[0]: paged decode, fp32 on the CPU path, batch 4, 8 q = 8 kv heads, head_dim 64, "
+                                   "block 16, ctx 256, 64-block pool permuted, seed %d" % args.seed,
+                       "algorithmic_bytes": nbytes},
+            "cpu_baseline": {"value": nbytes / best / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                             "kind": "port", "seconds_per_pass": best,
+                             "sample": "whole configuration, 1 warm-up + best of 3 passes of oracle "
+                                       "paged_decode_reference, torch CPU fp32"},
+            "gpu": {"ms_per_step": wall_ms, "device_ms": dev_ms, "dtype": "bf16", "note": "cache-resident: latency figure, "
+                    "no roofline claim"},
+            "parity": {"max_abs_err": float(err.max()), "within_2e-2_abs_1e-2_rel": bool((err <= 2e-2 + 1e-2 * ref16.abs()).all()),
+                       "max_abs_diff_bf16_inputs_vs_fp32_inputs": float((ref16 - ref).abs().max())}}
+
+
+def bench_prefill(cfg, args):
     import torch
     import mi355_attn
     from mi355_attn import workloads
@@ -347,7 +412,7 @@ def bench_prefill(cfg, args, with_cpu):
         def step():
             holder["out"] = mi355_attn.flash_attn_prefill(case.q, case.k, case.v, causal=True)
 
-    wall_ms, dev_ms = timed(step, args.steps, args.warmup)
+    wall_ms, dev_ms = timed(step, args.steps, args.warmup, BURN_IN)
     flops = case.flops()
     res = {
         "value": flops / wall_ms / 1e9,
@@ -361,9 +426,7 @@ def bench_prefill(cfg, args, with_cpu):
             "traffic": _traffic(f"prefill_cfg{cfg}"),
         },
     }
-    if with_cpu:
-        res["cpu_baseline"], res["parity"] = cpu_prefill(case, holder["out"], cfg)
-    return res
+    return res, (case, holder["out"])
 
 
 def cpu_prefill(case, gpu_out, cfg, n_heads=8):
@@ -437,9 +500,13 @@ def main():
         "metric": METRIC, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic (seeded)",
     }
-    dec = None
+    # Every GPU leg runs first, back to back (the shader clock then stays in its loaded state: a GPU that idles
+    # through a CPU leg starts the next kernel at a low clock); the CPU oracle legs follow on the kept outputs.
+    line["burn_in_launches_before_mfma_legs"] = BURN_IN
+    dec = pre = f8 = None
+    kept = {}
     if args.only in (None, "decode"):
-        dec = bench_decode(3, args, with_cpu)
+        dec, kept["decode"] = bench_decode(3, args, with_cpu)
         line.update({
             "value": dec["value"], "unit": "GB/s", "ms_per_step": dec["ms_per_step"], "dtype": "bf16",
             "config": {"workload": "configs[3]: paged decode attention, bf16 KV cache, batch 128, 32 q / 8 kv heads, "
@@ -447,22 +514,19 @@ def main():
                        "tokens": dec["tokens"], "algorithmic_bytes": dec["algorithmic_bytes"]},
             "roofline": dec["roofline"],
         })
-        if with_cpu:
-            line["cpu_baseline"] = dec["cpu_baseline"]
-            line["parity"] = dec["parity"]
     if args.only in (None, "prefill"):
-        pre = bench_prefill(2, args, with_cpu)
+        pre, kept["prefill"] = bench_prefill(2, args)
         pre["config"] = {"workload": "configs[2]: causal prefill forward, bf16, packed varlen, batch 8, 32 q / 8 kv "
                                      "heads, head_dim 128, seq 4096, seed %d" % args.seed}
         pre["dtype"] = "bf16"
         line["prefill"] = pre
-        if dec is None and args.only == "prefill":
+        if args.only == "prefill":
             line.update({"value": pre["value"], "unit": "TFLOP/s", "ms_per_step": pre["ms_per_step"], "dtype": "bf16",
                          "config": pre["config"], "roofline": pre["roofline"]})
-            if with_cpu:
-                line["cpu_baseline"] = pre["cpu_baseline"]
+    if args.only in (None, "backward"):
+        line["prefill_backward"] = bench_prefill_backward(2, args)
     if args.only in (None, "fp8"):
-        f8 = bench_decode(4, args, with_cpu)
+        f8, kept["fp8"] = bench_decode(4, args, with_cpu)
         f8["config"] = {"workload": "configs[4]: paged decode attention, fp8-e4m3 KV cache + per-(block, kv head) fp32 "
                                     "scales, batch 256, 64 q / 8 kv heads, head_dim 128, block 16, ctx log-uniform "
                                     "[128,32768], seed %d" % args.seed}
@@ -471,16 +535,27 @@ def main():
         if args.only == "fp8":
             line.update({"value": f8["value"], "unit": "GB/s", "ms_per_step": f8["ms_per_step"],
                          "dtype": f8["dtype"], "config": f8["config"], "roofline": f8["roofline"]})
-            if with_cpu:
-                line["cpu_baseline"] = f8["cpu_baseline"]
-    if args.only in (None, "backward"):
-        line["prefill_backward"] = bench_prefill_backward(2, args)
     if args.only in (None, "producers"):
         line["cache_producers"] = bench_producers(args)
     if args.only in (None, "layer"):
         line["layer_ops"] = bench_layer_ops(args)
     if args.only in (None, "loop"):
         line["decode_loop"] = bench_decode_loop(args)
+
+    if with_cpu:
+        if dec is not None:
+            dec["cpu_baseline"], dec["parity"], _ = cpu_decode(*kept.pop("decode"), 3)
+            line["cpu_baseline"], line["parity"] = dec["cpu_baseline"], dec["parity"]
+        if pre is not None:
+            pre["cpu_baseline"], pre["parity"] = cpu_prefill(*kept.pop("prefill"), 2)
+            if args.only == "prefill":
+                line["cpu_baseline"] = pre["cpu_baseline"]
+        if f8 is not None:
+            f8["cpu_baseline"], f8["parity"], f8["parity_vs_bf16_kv"] = cpu_decode(*kept.pop("fp8"), 4)
+            if args.only == "fp8":
+                line["cpu_baseline"] = f8["cpu_baseline"]
+        if args.only in (None, "decode"):
+            line["config0"] = cpu_config0(args)
     print(json.dumps(line))
 
 

@@ -120,7 +120,8 @@ int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* o
  * full forward per token at :218) calls every step.  Its result is defined by
  * reduction to model.py:308-325 on the gathered KV.
  *
- *   q, out        : (B, Hq, D) bf16, contiguous
+ *   q, out        : (B, Hq, D) bf16, contiguous; Hq a multiple of Hkv (a kv head with more than 16
+ *                   query heads is streamed once per 16 of them)
  *   k_cache/v_cache: (num_blocks, Hkv, block_size, D), bf16 (kv_dtype MI355_BF16)
  *                   or fp8-e4m3 bytes (MI355_FP8_E4M3); block_size must be 16
  *   block_tables  : int32, row b at block_tables + b*bt_row_stride; entry j is
@@ -145,6 +146,8 @@ int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cac
                            int B, int Hq, int Hkv, int D, int block_size, int64_t num_blocks, int max_ctx,
                            float softmax_scale, int kv_dtype, void* stream);
 
+/* Workspace requirement of mi355_paged_decode_fwd.  Monotonic in every argument: a workspace sized for a
+ * caller's largest batch and longest context serves every call with smaller ones. */
 size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx);
 
 /* Tokens of one sequence handled by one workgroup of the split-K pass (grows with max_ctx). */

@@ -105,23 +105,24 @@ __device__ __forceinline__ float xor32_sum(float v) {
 
 // ---- direct global -> LDS loads ---------------------------------------------
 // global_load_lds_dwordx4: every lane supplies its own 16-byte global address; the
-// wavefront's 64 x 16 bytes land at lds_base + 16*lane (lds_base is wave-uniform).
-// Issued through the builtin, the compiler treats every later LDS read of the wavefront as a
-// possible reader of the landing data and puts `s_waitcnt vmcnt(0)` in front of it, which
-// exposes the whole memory latency.  dma_to_lds_16 issues the same instruction from inline
+// wavefront's 64 x 16 bytes land at lds_base + 16*lane (lds_base is wave-uniform, passed in m0).
+// Issued through the compiler's builtin, every later LDS read of the wavefront is treated as a
+// possible reader of the landing data and gets `s_waitcnt vmcnt(0)` in front of it, which
+// exposes the whole memory latency.  dma_to_lds_16 issues the instruction from inline
 // assembly instead: the compiler then places no wait for it at all, and every consumer must
 // be preceded by wait_vmcnt<N>() (N = number of younger vector-memory instructions of this
 // wavefront allowed to stay in flight) and, across wavefronts, by a barrier.
-__device__ __forceinline__ void load_to_lds_16(const void* gptr, void* lds_base) {
-    __builtin_amdgcn_global_load_lds(gptr, (MI355_LDS void*)lds_base, 16, 0, 0);
-}
 // gbase: wave-uniform global base address; voff: this lane's byte offset from it (unsigned,
 // < 2^32); lds_addr: wave-uniform LDS byte address the wavefront's 1 KiB lands at.
+// The LDS address travels in m0 as a declared register operand: the compiler writes m0 itself and knows
+// that this statement reads it, so its own uses of m0 elsewhere in a kernel stay correct.  (The leading
+// s_nop covers the wait state the hardware wants between a write of m0 and an LDS-DMA instruction; the
+// compiler cannot see the instruction inside the statement and would not insert it.)
 __device__ __forceinline__ void dma_to_lds_16(const void* gbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
-                 : "v"(voff), "s"(gbase), "s"(lds_addr)
-                 : "memory");      // m0 is reserved by the compiler, which reloads it before each of its own uses
+                 : "v"(voff), "s"(gbase), "{m0}"(lds_addr)
+                 : "memory");
 }
 __device__ __forceinline__ uint32_t lds_address(const void* lds_ptr) {
     return (uint32_t)(uintptr_t)(const MI355_LDS void*)lds_ptr;

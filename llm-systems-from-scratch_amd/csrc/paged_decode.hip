@@ -7,7 +7,8 @@
 //   S^T (keys x queries) = K . Q^T      v_mfma_f32_16x16x32_bf16, the Hq/Hkv query
 //                                       heads that share the kv head are the N
 //                                       columns (padded to 16), so every KV byte
-//                                       is fetched once per GQA group
+//                                       is fetched once per GQA group (once per 16
+//                                       query heads when a group has more)
 //   online softmax on S^T               each lane owns ONE query column and 8 keys;
 //                                       max/sum across the 4 lanes of a column
 //   O^T (d x queries) += V^T . P^T      V^T fragments come from a wavefront-private
@@ -51,6 +52,7 @@ struct DecodeParams {
     float* ws_m;
     float* ws_l;
     int B, Hq, Hkv, max_chunks, max_ctx;
+    int n_groups;             // ceil((Hq / Hkv) / 16): a kv head with more than 16 query heads is served 16 at a time
     int tokens_per_wave;      // 256, 512 or 1024: a long stream per wavefront amortises its start-up latency
     float scale_log2;
 };
@@ -94,14 +96,16 @@ void paged_decode_split_kernel(DecodeParams p) {
     // and the first chunks of the short sequences (the smallest work items) form the tail.
     const int wg = blockIdx.x;
     const int hk = wg % p.Hkv;
-    const int b = (wg / p.Hkv) % p.B;
-    const int chunk = p.max_chunks - 1 - wg / (p.Hkv * p.B);
+    const int grp = (wg / p.Hkv) % p.n_groups;           // which 16 query heads of the kv head (0 unless Hq/Hkv > 16)
+    const int b = (wg / (p.Hkv * p.n_groups)) % p.B;
+    const int chunk = p.max_chunks - 1 - wg / (p.Hkv * p.n_groups * p.B);
     const int ctx = min(p.context_lens[b], p.max_ctx);     // a length beyond the promised bound is truncated, never chased
     const int chunk_tokens = kDecodeWaves * p.tokens_per_wave;
     const int chunk_start = chunk * chunk_tokens;
     if (chunk_start >= ctx) return;
 
-    const int G = p.Hq / p.Hkv;
+    const int h0 = hk * (p.Hq / p.Hkv) + 16 * grp;       // first query head of this work item
+    const int G = min(16, p.Hq / p.Hkv - 16 * grp);      // ... and how many it serves
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15;          // key row of K / query column of S^T / d row of V^T
@@ -119,7 +123,7 @@ void paged_decode_split_kernel(DecodeParams p) {
     //             covers d = 64t + 16kg + 8e + j, so Q uses the same d order.
     bf16x8 qf[NS];
     {
-        const __bf16* qrow = p.q + ((int64_t)b * p.Hq + (int64_t)hk * G + r) * D;
+        const __bf16* qrow = p.q + ((int64_t)b * p.Hq + h0 + r) * D;
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             const int d0 = FP8 ? (64 * (s >> 1) + 16 * kg + 8 * (s & 1)) : (32 * s + 8 * kg);
@@ -376,7 +380,7 @@ void paged_decode_split_kernel(DecodeParams p) {
             num += f * part[qi * D + d];
             den += f * part[16 * D + 16 + qi];
         }
-        const int64_t row = (int64_t)b * p.Hq + (int64_t)hk * G + qi;
+        const int64_t row = (int64_t)b * p.Hq + h0 + qi;
         if (n_chunks == 1) {
             p.out[row * D + d] = (__bf16)(num / den);
         } else {
@@ -424,7 +428,7 @@ __global__ __launch_bounds__(kCombineThreads) void paged_decode_combine_kernel(D
 
 template <int D, bool FP8>
 static int launch_decode(const DecodeParams& p, hipStream_t stream) {
-    dim3 grid((unsigned)p.max_chunks * p.Hkv * p.B);
+    dim3 grid((unsigned)p.max_chunks * p.Hkv * p.n_groups * p.B);
     hipLaunchKernelGGL((paged_decode_split_kernel<D, FP8>), grid, dim3(kDecodeWaves * 64), 0, stream, p);
     if (p.max_chunks > 1) {
         const int rows_per_wg = kCombineThreads / (D / 4);
@@ -448,12 +452,21 @@ static int tokens_per_wave_for(int max_ctx) {
 
 extern "C" int mi355_paged_decode_chunk_tokens(int max_ctx) { return kDecodeWaves * tokens_per_wave_for(max_ctx); }
 
+// Bytes of split-K partials for `chunks` chunks per (sequence, query head): O (D fp32), m, l.
+static size_t workspace_layout_bytes(size_t B, size_t Hq, size_t D, size_t chunks) {
+    const size_t rows = B * Hq * chunks;
+    return align_up(rows * D * 4, 256) + 2 * align_up(rows * 4, 256);
+}
+
+// The chunk size grows with max_ctx (1024, 2048, 4096 tokens), so the number of chunks a launch really uses,
+// ceil(max_ctx / chunk(max_ctx)), is not monotonic in max_ctx: it is at most 2 below 4096 tokens and
+// ceil(max_ctx / 4096) from there on.  The requirement reported here is the largest one over every bound up to
+// max_ctx, so a workspace sized for a caller's longest context serves every shorter one.
 extern "C" size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx) {
     if (B <= 0 || Hq <= 0 || D <= 0 || max_ctx <= 0) return 0;
-    const size_t chunk = (size_t)mi355_paged_decode_chunk_tokens(max_ctx);
-    const size_t chunks = ((size_t)max_ctx + chunk - 1) / chunk;
-    const size_t rows = (size_t)B * Hq * chunks;
-    return align_up(rows * D * 4, 256) + 2 * align_up(rows * 4, 256);
+    const size_t big = ((size_t)max_ctx + 4 * kMaxTokensPerWave - 1) / (4 * kMaxTokensPerWave);
+    const size_t small = max_ctx > 4 * 256 ? 2 : 1;
+    return workspace_layout_bytes((size_t)B, (size_t)Hq, (size_t)D, big > small ? big : small);
 }
 
 extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
@@ -466,13 +479,13 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
         return set_error(MI355_EINVAL, "paged_decode: null pointer argument");
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || max_ctx <= 0)
         return set_error(MI355_EINVAL, "paged_decode: B, Hq, Hkv and max_ctx must be positive");
-    if (Hq % Hkv != 0 || Hq / Hkv > 16)
-        return set_error(MI355_EINVAL, "paged_decode: Hq must be a multiple of Hkv with Hq/Hkv <= 16");
+    if (Hq % Hkv != 0) return set_error(MI355_EINVAL, "paged_decode: Hq must be a multiple of Hkv");
+    const int n_groups = (Hq / Hkv + 15) / 16;
     if (block_size != kBlock) return set_error(MI355_EINVAL, "paged_decode: block_size must be 16");
     if (num_blocks <= 0 || num_blocks > 0x7fffffffLL)
         return set_error(MI355_EINVAL, "paged_decode: num_blocks must be positive (and below 2^31)");
     const int chunk = mi355_paged_decode_chunk_tokens(max_ctx);
-    if ((int64_t)((max_ctx + chunk - 1) / chunk) * Hkv * B > 0x7fffffffLL)
+    if ((int64_t)((max_ctx + chunk - 1) / chunk) * Hkv * n_groups * B > 0x7fffffffLL)
         return set_error(MI355_EINVAL, "paged_decode: chunks * Hkv * B exceeds the grid limit");
     if (kv_dtype != MI355_BF16 && kv_dtype != MI355_FP8_E4M3)
         return set_error(MI355_EDTYPE, "paged_decode: kv_dtype must be MI355_BF16 or MI355_FP8_E4M3");
@@ -481,8 +494,8 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
         return set_error(MI355_EINVAL, "paged_decode: fp8 KV cache needs k_scale and v_scale");
     if (!(D == 128 || D == 64 || (D == 32 && !fp8)))
         return set_error(MI355_EINVAL, "paged_decode: head_dim must be 64 or 128 (or 32 with a bf16 cache)");
-    const size_t need = mi355_paged_decode_workspace_bytes(B, Hq, D, max_ctx);
     const int max_chunks = (max_ctx + chunk - 1) / chunk;
+    const size_t need = workspace_layout_bytes((size_t)B, (size_t)Hq, (size_t)D, (size_t)max_chunks);   // <= the reported bound
     if (max_chunks > 1 && (!workspace || workspace_bytes < need))
         return set_error(MI355_EWORKSPACE, "paged_decode: workspace smaller than mi355_paged_decode_workspace_bytes()");
 
@@ -507,6 +520,7 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
     p.Hkv = Hkv;
     p.max_chunks = max_chunks;
     p.max_ctx = max_ctx;
+    p.n_groups = n_groups;
     p.tokens_per_wave = tokens_per_wave_for(max_ctx);
     p.scale_log2 = softmax_scale * kLog2e;
 

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     const int n_wg = gridDim.x;
     int lid = blockIdx.x;
     if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
-    const int pair = lid % p.n_pairs;
+    const int pair0 = lid % p.n_pairs;
     const int h = (lid / p.n_pairs) % p.Hq;
     const int b = lid / (p.n_pairs * p.Hq);
     const int hk = h / (p.Hq / p.Hkv);
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     // Causal work grows with the query-tile index, so a workgroup takes the tiles
     // (nq-1-pair) and (pair): every workgroup of a sequence then carries the same load.
     const int nq = (sq + kBM - 1) / kBM;
-    if (2 * pair >= nq) return;          // (a sequence without keys still gets its rows written: no key kept -> NaN)
+    if (2 * pair0 >= nq) return;         // (a sequence without keys still gets its rows written: no key kept -> NaN)
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -180,6 +180,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     }
     const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
+    // The grid holds n_pairs workgroups per (batch, head), sized from the caller's Sq_max.  A packed sequence that is
+    // longer than that promise is still computed in full: its workgroups walk on through the remaining tile pairs
+    // (with a correct Sq_max this loop runs once).
+    for (int pair = pair0; 2 * pair < nq; pair += p.n_pairs)
     for (int half = 0; half < 2; ++half) {
         const int qtile = half == 0 ? nq - 1 - pair : pair;
         if (half == 1 && qtile == nq - 1 - pair) break;         // odd tile count: the middle tile has no partner

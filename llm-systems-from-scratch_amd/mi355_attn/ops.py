@@ -45,6 +45,31 @@ def _require_gpu_bf16(name, t):
         raise TypeError(f"{name} must be bfloat16 (got {t.dtype})")
 
 
+def _autocast_on() -> bool:
+    try:
+        return torch.is_autocast_enabled("cuda")
+    except TypeError:                      # older signature without a device type
+        return torch.is_autocast_enabled()
+
+
+def _to_bf16(q, k, v):
+    """The kernels compute on bf16 operands.  Inputs may be bfloat16 or float32 in any mix -- at
+    llm-core/llm_core/model.py:382 the reference passes float32 Q and K (RoPE multiplies the bf16 projections by its
+    float32 table, model.py:93-104) with a bfloat16 V under `--amp` (train.py:215), and three float32 tensors
+    without it.  float32 inputs are rounded to bf16 (what autocast does to them in front of PyTorch's SDPA; the cast
+    is differentiable).  Returns (q, k, v, out_dtype): float32 only when all three inputs are float32 and autocast
+    is off -- the case in which the reference's next operator expects float32 -- bfloat16 otherwise."""
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        if not t.is_cuda:
+            raise ValueError(f"{n} must live on the GPU (got {t.device}); this library has no CPU path")
+        if t.dtype not in (torch.bfloat16, torch.float32):
+            raise TypeError(f"{n} must be bfloat16 or float32 (got {t.dtype})")
+    all_f32 = all(t.dtype == torch.float32 for t in (q, k, v))
+    out_dtype = torch.float32 if all_f32 and not _autocast_on() else torch.bfloat16
+    q, k, v = (t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16) for t in (q, k, v))
+    return q, k, v, out_dtype
+
+
 def _rows16(name, t):
     """Return `t` with unit innermost stride and 16-byte aligned rows (copy only if needed)."""
     ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
@@ -184,17 +209,22 @@ def _needs_grad(*tensors):
 
 
 def flash_attn_prefill(q, k, v, *, causal=True, softmax_scale=None):
-    """Prefill forward.  q (B,Hq,Sq,D); k, v (B,Hkv,Sk,D) bf16 -> (B,Hq,Sq,D) bf16.
+    """Prefill forward.  q (B,Hq,Sq,D); k, v (B,Hkv,Sk,D) -> (B,Hq,Sq,D).
 
     Fills the slot of torch.nn.functional.scaled_dot_product_attention(Q, K, V,
     is_causal=True) at llm-core/llm_core/model.py:382.  With Sk > Sq the causal
     diagonal is bottom-right aligned (the queries are the last Sq positions).
+    Inputs are bfloat16 or float32 in any mix (see _to_bf16: bf16 math either way; the result is
+    float32 only for three float32 inputs outside autocast, bfloat16 otherwise).
     Differentiable: when an input requires grad, dq/dk/dv come from the HIP backward kernels
     (what autograd computes behind model.py:382 during train.py's loss.backward()).
     """
+    q, k, v, out_dtype = _to_bf16(q, k, v)
     if _needs_grad(q, k, v):
-        return _DensePrefillFn.apply(q, k, v, bool(causal), softmax_scale)
-    return _dense(q, k, v, None, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, softmax_scale)
+        out = _DensePrefillFn.apply(q, k, v, bool(causal), softmax_scale)
+    else:
+        out = _dense(q, k, v, None, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, softmax_scale)
+    return out if out.dtype == out_dtype else out.to(out_dtype)
 
 
 def sdpa_slot(Q, K, V, is_causal=True):
@@ -209,7 +239,10 @@ def scaled_dot_product_attention(Q, K, V, mask=None):
     boolean keep-mask (True = attend) broadcastable to (..., queries, keys); the
     scale is 1/sqrt(d_k).  A query row whose keys are all masked yields NaN, as
     the reference softmax (llm-core/llm_core/nn_functional.py:8-11) does.
-    Restriction of the HIP path: bf16 tensors, d_v == d_k in {32, 64, 128}.
+    Restrictions of the HIP path: d_v == d_k in {32, 64, 128}; bfloat16 or float32 tensors (bf16 math, see
+    _to_bf16).  Differentiable for mask=None (dq/dk/dv from the HIP backward kernels); the backward kernels have
+    no explicit-mask mode, so a call with a mask whose inputs require grad raises instead of returning a
+    result that autograd cannot see (use flash_attn_prefill(causal=True) for the causal mask in training).
     """
     if Q.dim() < 2 or K.dim() != Q.dim() or V.dim() != Q.dim():
         raise ValueError("Q, K and V need the same number of dimensions (>= 2)")
@@ -228,16 +261,24 @@ def scaled_dot_product_attention(Q, K, V, mask=None):
             return t.reshape((1,) * (4 - t.dim()) + tuple(t.shape))
         return t.reshape(-1, *t.shape[-3:])
 
+    Q, K, V, out_dtype = _to_bf16(Q, K, V)
     q4, k4, v4 = as4(Q, nq), as4(K, nk), as4(V, nk)
     m4 = None
     mode = _lib.MASK_NONE
+    if _needs_grad(Q, K, V):
+        if mask is not None:
+            raise NotImplementedError(
+                "scaled_dot_product_attention with an explicit mask is forward-only on the HIP path (the backward "
+                "kernels know no-mask and causal); for causal training use flash_attn_prefill / sdpa_slot")
+        out = _DensePrefillFn.apply(q4, k4, v4, False, None)
+        return out.reshape(*lead, nq, d).to(out_dtype)
     if mask is not None:
         m4 = as4(mask.expand(*mask.shape[:-2], nq, nk), nq).view(torch.uint8)
         if m4.stride(-1) != 1:
             m4 = m4.contiguous()
         mode = _lib.MASK_BOOL
     out = _dense(q4, k4, v4, m4, mode, None)
-    return out.reshape(*lead, nq, d)
+    return out.reshape(*lead, nq, d).to(out_dtype)
 
 
 def _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale, want_lse=False):
@@ -256,6 +297,12 @@ def _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, cau
         raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
     q, k, v = _rows16("q", q), _rows16("k", k), _rows16("v", v)
     B = cu_seqlens_q.numel() - 1
+    # max_seqlen_* are the caller's promise about the longest sequence (they are on the host, the lengths are not).
+    # What can be checked without reading device memory is checked here; a sequence longer than the promise is
+    # still computed in full by the kernel (its workgroups walk on through the remaining query tiles).
+    max_seqlen_q, max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+    if (Tq and max_seqlen_q < 1) or (Tk and max_seqlen_k < 1):
+        raise ValueError("max_seqlen_q and max_seqlen_k must be at least 1 when there are tokens")
     scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
     out = torch.empty(Tq, Hq, D, dtype=q.dtype, device=q.device)
     lse = torch.empty(Hq, Tq, dtype=torch.float32, device=q.device) if want_lse else None
@@ -271,14 +318,18 @@ def flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
 
     Sequence b owns rows [cu[b], cu[b+1]).  Returns (Tq,Hq,D) bf16.  Differentiable like flash_attn_prefill.
     """
+    q, k, v, out_dtype = _to_bf16(q, k, v)
     if _needs_grad(q, k, v):
-        return _VarlenPrefillFn.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, bool(causal),
-                                      softmax_scale)
-    return _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale)
+        out = _VarlenPrefillFn.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, bool(causal),
+                                     softmax_scale)
+    else:
+        out = _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale)
+    return out if out.dtype == out_dtype else out.to(out_dtype)
 
 
 def paged_decode_workspace(batch, n_q_heads, head_dim, max_context, device):
-    """Scratch tensor for paged_attention_decode (reusable across calls of the same or smaller shape)."""
+    """Scratch tensor for paged_attention_decode.  The requirement is monotonic in every argument, so a tensor
+    sized for the largest batch and longest context serves every smaller call."""
     n = _lib.load().mi355_paged_decode_workspace_bytes(batch, n_q_heads, head_dim, max_context)
     return torch.empty(max(int(n), 16), dtype=torch.uint8, device=device)
 

@@ -29,6 +29,11 @@ class DecodeCase:
     v_scale: torch.Tensor | None
     max_context: int
     context_lens_host: torch.Tensor
+    # fp8 cases only: the bf16 blocks (before quantisation) of the first `bf16_sample_seqs` sequences, in table
+    # order, so that the quantisation error can be measured against a bf16-KV reference
+    k_bf16_sample: torch.Tensor | None = None
+    v_bf16_sample: torch.Tensor | None = None
+    bf16_sample_seqs: int = 0
 
     @property
     def tokens(self) -> int:
@@ -79,7 +84,7 @@ def quantize_kv_fp8_(cache_bf16: torch.Tensor):
 
 
 def make_decode_case(*, batch, n_q_heads, n_kv_heads, head_dim, ctx_kind, ctx_lo, ctx_hi, pool_factor, seed,
-                     fp8=False, device="cuda:0") -> DecodeCase:
+                     fp8=False, keep_bf16_seqs=0, device="cuda:0") -> DecodeCase:
     ctx = draw_context_lens(ctx_kind, batch, ctx_lo, ctx_hi, seed)
     nblk = (ctx + BLOCK - 1) // BLOCK
     total = int(nblk.sum())
@@ -103,14 +108,19 @@ def make_decode_case(*, batch, n_q_heads, n_kv_heads, head_dim, ctx_kind, ctx_lo
         e = min(pool, s + step)
         kc[s:e] = torch.randn((e - s,) + shape[1:], generator=gd, device=device).to(torch.bfloat16)
         vc[s:e] = torch.randn((e - s,) + shape[1:], generator=gd, device=device).to(torch.bfloat16)
-    ks = vs = None
+    ks = vs = k_keep = v_keep = None
     if fp8:
+        keep_bf16_seqs = min(keep_bf16_seqs, batch)
+        if keep_bf16_seqs:
+            ids = torch.cat([bt[b, :int(nblk[b])] for b in range(keep_bf16_seqs)]).long().to(device)
+            k_keep, v_keep = kc[ids], vc[ids]
         kc, ks = quantize_kv_fp8_(kc)
         vc, vs = quantize_kv_fp8_(vc)
-    return DecodeCase(q, kc, vc, bt.to(device), ctx.to(device), ks, vs, max_blk * BLOCK, ctx)
+    return DecodeCase(q, kc, vc, bt.to(device), ctx.to(device), ks, vs, max_blk * BLOCK, ctx, k_keep, v_keep,
+                      keep_bf16_seqs if fp8 else 0)
 
 
-def decode_config(cfg: int, seed: int = 0, device="cuda:0") -> DecodeCase:
+def decode_config(cfg: int, seed: int = 0, device="cuda:0", keep_bf16_seqs: int = 0) -> DecodeCase:
     if cfg == 0:
         return make_decode_case(batch=4, n_q_heads=8, n_kv_heads=8, head_dim=64, ctx_kind="fixed", ctx_lo=256,
                                 ctx_hi=256, pool_factor=1.0, seed=seed, device=device)
@@ -119,7 +129,8 @@ def decode_config(cfg: int, seed: int = 0, device="cuda:0") -> DecodeCase:
                                 ctx_hi=16384, pool_factor=1.1, seed=seed, device=device)
     if cfg == 4:
         return make_decode_case(batch=256, n_q_heads=64, n_kv_heads=8, head_dim=128, ctx_kind="loguniform",
-                                ctx_lo=128, ctx_hi=32768, pool_factor=1.1, seed=seed, fp8=True, device=device)
+                                ctx_lo=128, ctx_hi=32768, pool_factor=1.1, seed=seed, fp8=True,
+                                keep_bf16_seqs=keep_bf16_seqs, device=device)
     raise ValueError(f"config {cfg} is not a decode configuration")
 
 

@@ -69,23 +69,30 @@ def _ffn_weights(params, prefix):
     return merged[:d_ff], merged[d_ff:], params[prefix + "ffn.w_down.weight"]
 
 
-def attention_block_reference(x, wq, wk, wv, wo, num_heads, freq_cache, positions=None):
-    """model.py:352-390 for x (batch, seq, d_model): project, split heads, RoPE on Q and K,
-    causal attention (model.py:384-385), merge heads, output projection."""
-    B, S, d_model = x.shape
+def attention_core_reference(q_proj, k_proj, v_proj, num_heads, freq_cache, positions=None):
+    """model.py:366-388 from the three projection outputs (batch, seq, heads*d_head) on: split heads, RoPE on Q
+    and K, causal attention (model.py:384-385), merge heads -> (batch, seq, heads*d_head)."""
+    B, S, d_model = q_proj.shape
     d_head = d_model // num_heads
 
     def split(t):                                             # (B,S,H*d) -> (B,H,S,d), model.py:366-370
         return t.view(B, S, num_heads, d_head).transpose(1, 2)
 
-    Q, K, V = split(x @ wq.T), split(x @ wk.T), split(x @ wv.T)
+    Q, K, V = split(q_proj), split(k_proj), split(v_proj)
     if positions is None:
         positions = torch.arange(S).expand(B, S)              # model.py:373-374
     pos = positions[:, None, :].expand(B, num_heads, S)
     Q = att.rope_reference(Q, pos, freq_cache)
     K = att.rope_reference(K, pos, freq_cache)
     out = att.scaled_dot_product_attention(Q, K, V, att.causal_keep_mask(S))
-    return out.transpose(1, 2).reshape(B, S, d_model) @ wo.T  # model.py:388-390
+    return out.transpose(1, 2).reshape(B, S, d_model)         # model.py:388
+
+
+def attention_block_reference(x, wq, wk, wv, wo, num_heads, freq_cache, positions=None):
+    """model.py:352-390 for x (batch, seq, d_model): project (model.py:362-364), attention_core_reference,
+    output projection (model.py:390)."""
+    merged = attention_core_reference(x @ wq.T, x @ wk.T, x @ wv.T, num_heads, freq_cache, positions)
+    return merged @ wo.T
 
 
 def transformer_lm_reference(params: dict, config: dict, token_ids: torch.Tensor) -> torch.Tensor:

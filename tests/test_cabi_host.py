@@ -46,6 +46,22 @@ def test_version_and_workspace_queries(lib):
     assert lib.mi355_paged_decode_workspace_bytes(0, 8, 64, 256) == 0
 
 
+def test_workspace_requirement_is_monotonic_in_max_ctx(lib):
+    """A workspace sized for the longest context must serve every shorter one, although the chunk size (and with it
+    the number of chunks a launch uses) changes at 2048 and 4096 tokens."""
+    for B, Hq, D in ((64, 16, 128), (3, 8, 64)):
+        prev = 0
+        for m in list(range(1, 9000, 7)) + [16384, 16385, 32768, 100000]:
+            cur = lib.mi355_paged_decode_workspace_bytes(B, Hq, D, m)
+            assert cur >= prev, (B, Hq, D, m)
+            chunk = lib.mi355_paged_decode_chunk_tokens(m)
+            rows = B * Hq * ((m + chunk - 1) // chunk)          # what a launch with this bound really lays out
+            assert cur >= rows * D * 4 + 2 * rows * 4, (B, Hq, D, m)
+            prev = cur
+        # and in the batch and head counts
+        assert lib.mi355_paged_decode_workspace_bytes(B - 1, Hq, D, 5000) <= lib.mi355_paged_decode_workspace_bytes(B, Hq, D, 5000)
+
+
 def test_prefill_rejects_bad_arguments_without_a_gpu(lib):
     s3 = _lib.strides3((8, 8, 8))
     buf = C.create_string_buffer(64)
@@ -77,7 +93,6 @@ def test_decode_rejects_bad_arguments_without_a_gpu(lib):
 
     assert call(bs=32) == -1 and b"block_size" in lib.mi355_last_error()
     assert call(Hq=7) == -1
-    assert call(Hq=64, Hkv=2) == -1            # more than 16 query heads per kv head
     assert call(D=96) == -1
     assert call(kv=5) == -3
     assert call(kv=_lib.MI355_FP8_E4M3, ks=None) == -1 and b"scale" in lib.mi355_last_error()

@@ -83,3 +83,50 @@ def test_continuous_batching_matches_dense_causal_attention():
         ref = orc.prefill_reference(q_rot[None], k_rot[None], v.transpose(0, 1)[None], causal=True)[0].transpose(0, 1)
         err = (got[s] - ref).abs()
         assert bool((err <= 2e-2 + 1e-2 * ref.abs()).all()), (s, float(err.max()))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("ctx_len", [2048, 4096])
+def test_decode_with_full_batch_at_long_context_lengths(ctx_len):
+    """The engine sizes its split-K workspace once, for (max_batch, context_length).  The kernel's chunk size
+    changes with the longest context of a step (2048 and 4096 tokens are the thresholds), so steps at shorter
+    lengths use MORE chunks per sequence than the sizing call: every such step must still fit the workspace."""
+    import mi355_attn
+    print(f"case: engine full batch at context_length {ctx_len}", flush=True)
+    Hq, Hkv, D, B = 8, 2, 64, 6
+    eng = mi355_attn.PagedAttentionEngine(num_blocks=B * ctx_len // 16, n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D,
+                                          context_length=ctx_len, max_batch=B)
+    fc = orc.build_rope_cache(ctx_len, D)
+    lens = [ctx_len - 1 - 16 * i for i in range(B)]
+    lens[-1] = 1500                                      # and one sequence between the thresholds' chunk sizes
+    qs = [rnd(n + 1, Hq, D, seed=70 + i) for i, n in enumerate(lens)]
+    ks = [rnd(n + 1, Hkv, D, seed=80 + i) for i, n in enumerate(lens)]
+    vs = [rnd(n + 1, Hkv, D, seed=90 + i) for i, n in enumerate(lens)]
+    sids = list(range(B))
+    for s in sids:
+        eng.add_sequence(s)
+    eng.prefill(sids, lens, torch.cat([q[:-1] for q in qs]).cuda(), torch.cat([k[:-1] for k in ks]).cuda(),
+                torch.cat([v[:-1] for v in vs]).cuda())
+    out = eng.decode_step(sids, torch.stack([q[-1] for q in qs]).cuda(), torch.stack([k[-1] for k in ks]).cuda(),
+                          torch.stack([v[-1] for v in vs]).cuda()).float().cpu()
+    # a second step at a much shorter longest context (other chunk regime) reuses the same workspace
+    for s in sids[:-1]:
+        eng.remove_sequence(s)
+    q2, k2, v2 = rnd(1, Hq, D, seed=101), rnd(1, Hkv, D, seed=102), rnd(1, Hkv, D, seed=103)
+    out2 = eng.decode_step([sids[-1]], q2.cuda(), k2.cuda(), v2.cuda()).float().cpu()
+    torch.cuda.synchronize()
+    for i, n in enumerate(lens):
+        p = torch.arange(n + 1)
+        q_rot = orc.rope_reference(qs[i][-1:].float().transpose(0, 1), p[-1:], fc).to(torch.bfloat16)
+        k_rot = orc.rope_reference(ks[i].float().transpose(0, 1), p, fc).to(torch.bfloat16)
+        ref = orc.prefill_reference(q_rot[None], k_rot[None], vs[i].transpose(0, 1)[None], causal=True)[0, :, 0]
+        err = (out[i] - ref).abs()
+        assert bool((err <= 2e-2 + 1e-2 * ref.abs()).all()), (i, float(err.max()))
+    i, n = B - 1, lens[-1] + 2
+    p = torch.arange(n)
+    k_all, v_all = torch.cat([ks[i], k2]), torch.cat([vs[i], v2])
+    q_rot = orc.rope_reference(q2.float().transpose(0, 1), p[-1:], fc).to(torch.bfloat16)
+    k_rot = orc.rope_reference(k_all.float().transpose(0, 1), p, fc).to(torch.bfloat16)
+    ref = orc.prefill_reference(q_rot[None], k_rot[None], v_all.transpose(0, 1)[None], causal=True)[0, :, 0]
+    err = (out2[0] - ref).abs()
+    assert bool((err <= 2e-2 + 1e-2 * ref.abs()).all()), float(err.max())

@@ -275,6 +275,125 @@ def test_prefill_varlen_ragged(ops, lens):
     check(got, ref, what="varlen")
 
 
+def _reference_module_tensors(x_proj, freq, num_heads, amp):
+    """Q, K, V exactly as CausalMultiHeadSelfAttention.forward hands them to the attention call
+    (llm-core/llm_core/model.py:362-378) from the three projection outputs (B, S, H*d): `rearrange` views, then
+    RotaryEmbedding.forward (model.py:93-104) on Q and K with the float32 (2, ctx, d/2) table.  Under `--amp` the
+    projections are bf16, so Q and K come out float32 and contiguous and V stays a strided bf16 view."""
+    from einops import rearrange
+    qp, kp, vp = x_proj
+    Q, K, V = (rearrange(t, "... seq (heads d) -> ... heads seq d", heads=num_heads) for t in (qp, kp, vp))
+    S = qp.shape[1]
+    pos = torch.arange(S, device=qp.device).view(1, S)
+    pos = rearrange(pos, "... seq -> ... 1 seq")
+
+    def rope(x):
+        x1, x2 = x[..., 0::2], x[..., 1::2]
+        cos, sin = freq[:, pos, :]
+        return rearrange([cos * x1 - sin * x2, sin * x1 + cos * x2], "xy ... half_d -> ... (half_d xy)", xy=2).contiguous()
+
+    Q, K = rope(Q), rope(K)
+    if amp:
+        assert Q.dtype == torch.float32 and K.dtype == torch.float32 and V.dtype == torch.bfloat16
+    assert Q.is_contiguous() and not V.is_contiguous()
+    return Q, K, V
+
+
+@pytest.mark.parametrize("amp", [True, False])
+def test_sdpa_slot_takes_the_reference_modules_tensors(ops, amp):
+    """The swap at model.py:382 with the tensors the reference really passes there: float32 Q/K + strided bf16 V
+    under autocast (train.py:215), three float32 tensors without it; the reference's sample shape (d_head 32,
+    16 heads, configures/sample.yaml).  Checked through the head merge of model.py:388 against the oracle's
+    attention block run on the same projection outputs.  float32 inputs are rounded to bf16 by the slot (bf16
+    math, as autocast SDPA does), hence the bf16 tolerance for the float32 case too."""
+    from einops import rearrange
+    from oracle import model_oracle as morc
+    print(f"case: sdpa_slot reference dtype flow amp={amp}", flush=True)
+    B, S, H, d = 3, 256, 16, 32
+    g = torch.Generator().manual_seed(31)
+    proj = [torch.randn(B, S, H * d, generator=g) * 0.7 for _ in range(3)]
+    if amp:
+        proj = [t.to(torch.bfloat16) for t in proj]                   # what a Linear gives under autocast
+    freq = orc.build_rope_cache(S, d)
+    ref = morc.attention_core_reference(*(t.float() for t in proj), H, freq)
+
+    Q, K, V = _reference_module_tensors([t.cuda() for t in proj], freq.cuda(), H, amp)
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=amp):
+        out = ops.sdpa_slot(Q, K, V, is_causal=True)
+    assert out.shape == (B, H, S, d)
+    assert out.dtype == (torch.bfloat16 if amp else torch.float32)    # what F.scaled_dot_product_attention returns there
+    merged = rearrange(out, "... heads seq d_head -> ... seq (heads d_head)").contiguous()
+    torch.cuda.synchronize()
+    check(merged, ref, what=f"model.py:382 slot, amp={amp}")
+
+
+def test_sdpa_slot_trains_through_the_reference_dtype_flow(ops):
+    """Gradients reach the float32 Q/K and the bf16 V of the autocast flow (the casts in front of the kernel are
+    differentiable) and match the oracle's hand-derived backward."""
+    print("case: sdpa_slot backward through mixed dtypes", flush=True)
+    B, H, S, d = 2, 4, 96, 32
+    q32, k32 = rnd(B, H, S, d, seed=41, scale=0.5).float(), rnd(B, H, S, d, seed=42, scale=0.5).float()
+    v16, dout = rnd(B, H, S, d, seed=43, scale=0.5), rnd(B, H, S, d, seed=44, scale=0.5)
+    Q, K, V = q32.cuda().requires_grad_(), k32.cuda().requires_grad_(), v16.cuda().requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = ops.sdpa_slot(Q, K, V, is_causal=True)
+    assert out.dtype == torch.bfloat16 and out.requires_grad
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    assert Q.grad.dtype == torch.float32 and V.grad.dtype == torch.bfloat16
+    dq, dk, dv, _ = orc.prefill_backward_reference(q32.bfloat16(), k32.bfloat16(), v16, dout, causal=True)
+    for name, got, ref in (("dq", Q.grad, dq), ("dk", K.grad, dk), ("dv", V.grad, dv)):
+        check(got, ref, atol=2e-2 * float(ref.abs().max()), rtol=2e-2, what=name)
+
+
+def test_sdpa_reference_signature_autograd(ops):
+    """scaled_dot_product_attention (the model.py:384-385 branch, used in training without --flash-attn): with
+    mask=None the result carries a grad_fn and the gradients match the oracle; with a mask it raises instead of
+    silently returning a detached result."""
+    print("case: sdpa signature autograd", flush=True)
+    B, H, S, D = 1, 2, 80, 64
+    q, k, v, dout = (rnd(B, H, S, D, seed=s, scale=0.5) for s in (51, 52, 53, 54))
+    Q, K, V = (t.cuda().requires_grad_() for t in (q, k, v))
+    out = ops.scaled_dot_product_attention(Q, K, V)
+    assert out.requires_grad and out.grad_fn is not None
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    dq, dk, dv, _ = orc.prefill_backward_reference(q, k, v, dout, causal=False)
+    for name, got, ref in (("dq", Q.grad, dq), ("dk", K.grad, dk), ("dv", V.grad, dv)):
+        check(got, ref, atol=2e-2 * float(ref.abs().max()), rtol=2e-2, what=name)
+    tril = torch.tril(torch.ones(S, S, dtype=torch.bool, device="cuda"))
+    with pytest.raises(NotImplementedError, match="forward-only"):
+        ops.scaled_dot_product_attention(Q, K, V, tril)
+    with torch.no_grad():                                              # forward-only use is unaffected
+        assert not ops.scaled_dot_product_attention(Q, K, V, tril).requires_grad
+
+
+def test_prefill_varlen_sequence_longer_than_promised(ops):
+    """max_seqlen_q smaller than the longest sequence: every row is still computed (the workgroups of a sequence
+    walk on through its remaining query tiles), none is left unwritten."""
+    print("case: prefill varlen with too small a max_seqlen", flush=True)
+    lens = [40, 1500, 700]
+    Hq, Hkv, D = 4, 2, 64
+    T = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q, k, v = rnd(T, Hq, D, seed=61, scale=0.5), rnd(T, Hkv, D, seed=62, scale=0.5), rnd(T, Hkv, D, seed=63, scale=0.5)
+    ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True)
+    got = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), 300, 300, causal=True)
+    check(got, ref, what="varlen, promise too small")
+    with pytest.raises(ValueError, match="max_seqlen"):
+        ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), 0, 0, causal=True)
+
+
+def test_decode_more_than_16_query_heads_per_kv_head(ops):
+    """Hq/Hkv = 32 and 20 (multi-query style): the kv head is streamed once per 16 query heads."""
+    for Hq, Hkv, D in ((32, 1, 128), (40, 2, 64)):
+        print(f"case: decode Hq/Hkv > 16: {Hq}/{Hkv}", flush=True)
+        ctx = [1, 17, 300, 5000]
+        q, kc, vc, bt, cl = orc.make_paged_case(batch=len(ctx), n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                                context_lens=ctx, pool_factor=1.2, seed=Hq, dtype=torch.bfloat16)
+        check(run_decode(ops, q, kc, vc, bt, cl), orc.paged_decode_reference(q, kc, vc, bt, cl), what=f"{Hq}/{Hkv}")
+
+
 def test_sdpa_with_reference_signature(ops):
     """scaled_dot_product_attention(Q, K, V, mask): None, the reference's tril mask, and an arbitrary keep-mask."""
     print("case: sdpa signature", flush=True)
@@ -311,7 +430,9 @@ def test_sdpa_fully_masked_row_is_nan_like_reference(ops):
 def test_errors_are_python_exceptions(ops):
     q = torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(TypeError):
-        ops.flash_attn_prefill(q.float(), q.float(), q.float())
+        ops.flash_attn_prefill(q.half(), q.half(), q.half())          # bfloat16 and float32 only
+    with pytest.raises(TypeError):
+        ops.sdpa_slot(q.double(), q.double(), q.double())
     with pytest.raises(ValueError):
         ops.flash_attn_prefill(q, q[:, :, :, :32], q)
     with pytest.raises(ValueError):
