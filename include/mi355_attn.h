@@ -150,6 +150,29 @@ int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cac
  * caller's largest batch and longest context serves every call with smaller ones. */
 size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx);
 
+/*
+ * mi355_paged_decode_fwd without a workspace argument and without any allocation: the split-K partials go to a
+ * device array that is part of the library's own code object (MI355_STATIC_SCRATCH_BYTES per GPU, held from the
+ * first load until the process ends).  It has no counterpart in the reference; it exists for callers that cannot
+ * allocate or size a workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same arguments, kernels and results (bit for bit) as mi355_paged_decode_fwd otherwise.
+ *   - a call whose partials need more than the array (mi355_paged_decode_workspace_bytes of the layout actually
+ *     used, i.e. B * Hq * ceil(max_ctx / mi355_paged_decode_chunk_tokens(max_ctx)) * (D + 2) * 4 bytes plus padding)
+ *     is rejected with MI355_EWORKSPACE; max_ctx up to one chunk needs no scratch at all;
+ *   - all calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
+ *     threads) race on it and must be serialised by the caller; the array's old contents never matter (every
+ *     partial that the combine pass reads is written by the split pass of the same call);
+ *   - the array's address is looked up on the first call on each device (not a stream operation); make that
+ *     first call outside a graph capture, like the first launch of any kernel.
+ */
+#define MI355_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
+int mi355_paged_decode_fwd_static(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                  const int32_t* block_tables, int64_t bt_row_stride,
+                                  const int32_t* context_lens,
+                                  const float* k_scale, const float* v_scale,
+                                  int B, int Hq, int Hkv, int D, int block_size, int64_t num_blocks, int max_ctx,
+                                  float softmax_scale, int kv_dtype, void* stream);
+
 /* Tokens of one sequence handled by one workgroup of the split-K pass (grows with max_ctx). */
 int mi355_paged_decode_chunk_tokens(int max_ctx);
 

@@ -25,6 +25,7 @@
 // chunk is normalised and written straight to `out`, otherwise the chunk's
 // partial goes to the workspace and the combine kernel finishes it:
 //   o = sum_c 2^(m_c - m) o_c / sum_c 2^(m_c - m) l_c      (m = max_c m_c).
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -469,12 +470,15 @@ extern "C" size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int m
     return workspace_layout_bytes((size_t)B, (size_t)Hq, (size_t)D, big > small ? big : small);
 }
 
-extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                      const int32_t* block_tables, int64_t bt_row_stride,
-                                      const int32_t* context_lens, const float* k_scale,
-                                      const float* v_scale, void* workspace, size_t workspace_bytes, int B,
-                                      int Hq, int Hkv, int D, int block_size, int64_t num_blocks, int max_ctx,
-                                      float softmax_scale, int kv_dtype, void* stream) {
+// Argument checks and launches shared by the two entry points.  `static_scratch`: the workspace is the library's
+// own device array (its capacity is `workspace_bytes`), fetched only once the arguments have passed the checks.
+static int scratch_for_current_device(void** ptr);
+
+static int decode_common(const void* q, const void* k_cache, const void* v_cache, void* out,
+                         const int32_t* block_tables, int64_t bt_row_stride, const int32_t* context_lens,
+                         const float* k_scale, const float* v_scale, void* workspace, size_t workspace_bytes,
+                         bool static_scratch, int B, int Hq, int Hkv, int D, int block_size, int64_t num_blocks,
+                         int max_ctx, float softmax_scale, int kv_dtype, void* stream) {
     if (!q || !k_cache || !v_cache || !out || !block_tables || !context_lens)
         return set_error(MI355_EINVAL, "paged_decode: null pointer argument");
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || max_ctx <= 0)
@@ -496,8 +500,19 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
         return set_error(MI355_EINVAL, "paged_decode: head_dim must be 64 or 128 (or 32 with a bf16 cache)");
     const int max_chunks = (max_ctx + chunk - 1) / chunk;
     const size_t need = workspace_layout_bytes((size_t)B, (size_t)Hq, (size_t)D, (size_t)max_chunks);   // <= the reported bound
-    if (max_chunks > 1 && (!workspace || workspace_bytes < need))
+    if (static_scratch) {
+        if (max_chunks > 1 && need > workspace_bytes)
+            return set_error(MI355_EWORKSPACE,
+                             "paged_decode_static: B * Hq * chunks(max_ctx) * (D + 2) * 4 bytes of split-K partials exceed the "
+                             "library's static scratch (MI355_STATIC_SCRATCH_BYTES); use "
+                             "mi355_paged_decode_fwd with a caller-provided workspace");
+        if (max_chunks > 1) {
+            const int rc = scratch_for_current_device(&workspace);
+            if (rc != 0) return rc;
+        }
+    } else if (max_chunks > 1 && (!workspace || workspace_bytes < need)) {
         return set_error(MI355_EWORKSPACE, "paged_decode: workspace smaller than mi355_paged_decode_workspace_bytes()");
+    }
 
     DecodeParams p;
     p.q = (const __bf16*)q;
@@ -534,4 +549,57 @@ extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const 
     }
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;
+}
+
+extern "C" int mi355_paged_decode_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                      const int32_t* block_tables, int64_t bt_row_stride,
+                                      const int32_t* context_lens, const float* k_scale,
+                                      const float* v_scale, void* workspace, size_t workspace_bytes, int B,
+                                      int Hq, int Hkv, int D, int block_size, int64_t num_blocks, int max_ctx,
+                                      float softmax_scale, int kv_dtype, void* stream) {
+    return decode_common(q, k_cache, v_cache, out, block_tables, bt_row_stride, context_lens, k_scale, v_scale, workspace,
+                         workspace_bytes, false, B, Hq, Hkv, D, block_size, num_blocks, max_ctx, softmax_scale, kv_dtype,
+                         stream);
+}
+
+// ---- the variant that allocates nothing -------------------------------------------------------------------
+// Split-K partials live in a file-scope device array instead of a caller-provided workspace.  Every GPU that
+// loads the library holds its own copy of the array (at its own address) until the process ends.  In host code
+// the array's name is only a stand-in for the symbol, not a device address: the address on a device is asked for
+// once per device, with that device current, and kept; kernels only ever see that pointer.
+constexpr size_t kStaticScratchBytes = MI355_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];            // device address of `scratch`, per device (null: not asked yet)
+static std::mutex g_scratch_mutex;
+
+static int scratch_for_current_device(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_error((int)e, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return set_error(MI355_EINVAL, "paged_decode_static: device index out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            return set_error(e != hipSuccess ? (int)e : MI355_EINVAL,
+                             e != hipSuccess ? hipGetErrorString(e) : "paged_decode_static: no address for the static scratch");
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return MI355_OK;
+}
+
+extern "C" int mi355_paged_decode_fwd_static(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                             const int32_t* block_tables, int64_t bt_row_stride,
+                                             const int32_t* context_lens, const float* k_scale,
+                                             const float* v_scale, int B, int Hq, int Hkv, int D, int block_size,
+                                             int64_t num_blocks, int max_ctx, float softmax_scale, int kv_dtype,
+                                             void* stream) {
+    return decode_common(q, k_cache, v_cache, out, block_tables, bt_row_stride, context_lens, k_scale, v_scale, nullptr,
+                         kStaticScratchBytes, true, B, Hq, Hkv, D, block_size, num_blocks, max_ctx, softmax_scale,
+                         kv_dtype, stream);
 }

@@ -11,6 +11,7 @@ MI355_BF16 = 0
 MI355_FP8_E4M3 = 1
 MI355_FP32 = 2
 MASK_NONE, MASK_CAUSAL, MASK_BOOL = 0, 1, 2
+STATIC_SCRATCH_BYTES = 16 << 20          # MI355_STATIC_SCRATCH_BYTES
 
 _i64x3 = C.c_int64 * 3
 _i64x2 = C.c_int64 * 2
@@ -21,6 +22,7 @@ EXPORTS = (
     "mi355_prefill_fwd_lse",
     "mi355_prefill_bwd",
     "mi355_paged_decode_fwd",
+    "mi355_paged_decode_fwd_static",
     "mi355_paged_decode_workspace_bytes",
     "mi355_paged_decode_chunk_tokens",
     "mi355_rope_and_cache",
@@ -61,6 +63,9 @@ def load():
     lib.mi355_paged_decode_fwd.restype = i32
     lib.mi355_paged_decode_fwd.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, sz,
                                            i32, i32, i32, i32, i32, i64, i32, f32, i32, vp]
+    lib.mi355_paged_decode_fwd_static.restype = i32
+    lib.mi355_paged_decode_fwd_static.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, vp,
+                                                  i32, i32, i32, i32, i32, i64, i32, f32, i32, vp]
     lib.mi355_paged_decode_workspace_bytes.restype = sz
     lib.mi355_paged_decode_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.mi355_paged_decode_chunk_tokens.restype = i32

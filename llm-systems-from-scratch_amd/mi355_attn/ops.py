@@ -335,7 +335,8 @@ def paged_decode_workspace(batch, n_q_heads, head_dim, max_context, device):
 
 
 def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, softmax_scale=None,
-                           k_scale=None, v_scale=None, max_context=None, workspace=None, out=None):
+                           k_scale=None, v_scale=None, max_context=None, workspace=None, out=None,
+                           static_scratch=False):
     """Paged-KV decode attention, one query token per sequence.
 
     q (B,Hq,D) bf16; k_cache, v_cache (num_blocks,Hkv,16,D) bf16, or fp8-e4m3
@@ -343,6 +344,9 @@ def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, s
     (num_blocks,Hkv) fp32 are given; block_tables (B,max_blocks) int32;
     context_lens (B,) int32 >= 1.  `max_context` bounds context_lens (default:
     block_tables.shape[1]*16) so no device->host sync is needed.  Returns (B,Hq,D) bf16.
+    static_scratch=True (needs `out`) goes through mi355_paged_decode_fwd_static: nothing is allocated, the
+    split-K partials live in the library's own device array (16 MiB per GPU; larger problems are rejected; calls
+    that overlap in time on one GPU must be serialised by the caller).
     """
     _require_gpu_bf16("q", q)
     if q.dim() != 3:
@@ -383,10 +387,24 @@ def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, s
         raise ValueError("max_context exceeds what block_tables can address")
     scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
     if out is None:
+        if static_scratch:
+            raise ValueError("static_scratch=True allocates nothing: pass `out`")
         out = torch.empty_like(q)
     if B == 0:
         return out
     lib = _lib.load()
+    if static_scratch:
+        if workspace is not None:
+            raise ValueError("static_scratch and workspace exclude each other")
+        with _on(q, k_cache, v_cache, out, block_tables, context_lens, k_scale, v_scale) as stream:
+            rc = lib.mi355_paged_decode_fwd_static(
+                q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+                block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
+                k_scale.data_ptr() if fp8 else None, v_scale.data_ptr() if fp8 else None,
+                B, Hq, Hkv, D, bs, k_cache.shape[0], int(max_context), float(scale),
+                _lib.MI355_FP8_E4M3 if fp8 else _lib.MI355_BF16, stream)
+        _lib.check(rc, "mi355_paged_decode_fwd_static")
+        return out
     if workspace is None:
         workspace = paged_decode_workspace(B, Hq, D, max_context, q.device)
     with _on(q, k_cache, v_cache, out, block_tables, context_lens, k_scale, v_scale, workspace) as stream:
