@@ -14,7 +14,11 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "mi355_attn")
 LIB_NAME = "libmi355attn.so"
-SOURCES = ["api.hip", "paged_decode.hip", "prefill_fwd.hip", "prefill_bwd.hip", "kv_cache_ops.hip", "layer_ops.hip"]
+SOURCES = ["api.hip", "paged_decode.hip", "prefill_fwd.hip", "prefill_fwd_w64.hip", "prefill_bwd.hip", "kv_cache_ops.hip",
+           "layer_ops.hip"]
+# prefill_fwd_w64.hip keeps its output accumulators in AGPRs that only its assembly statements touch: its builtin MFMAs
+# must therefore be selected in VGPR form, so that the compiler allocates no AGPR for them.
+EXTRA_FLAGS = {"prefill_fwd_w64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -38,13 +42,15 @@ def library_path() -> str:
 
 
 def build_library(verbose: bool = True) -> str:
+    # the hand-scheduled assembly of prefill_fwd_w64.hip is generated text: regenerate it so that it cannot go stale
+    _run([sys.executable, os.path.join(CSRC, "gen_prefill_w64_loop.py")])
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
 
     def compile_one(src):
         obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        log = _run([HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        log = _run([HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj])
         return obj, log
 
     with ThreadPoolExecutor(max_workers=4) as ex:

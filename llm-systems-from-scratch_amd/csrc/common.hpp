@@ -41,6 +41,16 @@ __device__ __forceinline__ i16x4 lds_read_tr16(const void* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((MI355_LDS i16x4*)p);
 }
 
+// Reads through an absolute LDS byte address (what lds_address() returns), for code that shares precomputed
+// addresses with hand-written assembly.
+template <class T>
+__device__ __forceinline__ T lds_load_at(uint32_t addr) {
+    return *reinterpret_cast<const MI355_LDS T*>((size_t)addr);
+}
+__device__ __forceinline__ i16x4 lds_read_tr16_at(uint32_t addr) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<MI355_LDS i16x4*>((size_t)addr));
+}
+
 __device__ __forceinline__ bf16x8 join_bf16x8(i16x4 lo, i16x4 hi) {
     struct { i16x4 a, b; } t{lo, hi};
     return __builtin_bit_cast(bf16x8, t);

@@ -1,0 +1,466 @@
+// Prefill forward for head_dim 128 (no mask or causal), one wavefront per SIMD, 64 queries per wavefront.
+//
+// One workgroup = 4 wavefronts = one tile of 256 queries of one (batch, head); a wavefront owns 64 query rows as two
+// column blocks A and B of 32.  It runs alone on its SIMD with the whole register file: the output accumulators
+// (2 x 4 x 16 registers) live in AGPRs, everything the vector unit touches in VGPRs.  K/V tiles of 64 keys are
+// double-buffered in LDS (direct-to-LDS loads, XOR-swizzled rows) and shared by the four wavefronts; every K
+// fragment and every V^T fragment read from LDS feeds two MFMAs (one per column block).
+//
+// The mathematics is that of prefill_fwd.hip (transposed problem: S^T = K . Q^T, O^T += V^T . P^T, one query per
+// lane, weights 2^(s * scale * log2(e) + nb) with one fma and one exp2 per score), with two changes that take vector
+// work out of the loop: row sums come from a 16x16x32 MFMA against a 0/1 operand instead of adds, and the exponent
+// reference is looked at only through the weights themselves.  A query tile starts with the reference preset to 0
+// (nb = -32: the weight of a score x is 2^(x - 32)) and the loop watches for a weight that reaches 2 (the top exponent
+// bit of its bf16 pattern): only then ordinary code moves the reference of that row up to its maximum, rescales and
+// resumes.  For scores between -60 and +33 binary orders -- anything a trained model produces -- no row maximum is
+// ever computed.  A row whose scores are all so negative that its sum stays below 2^-92 may have lost terms to
+// underflow; the workgroup then computes the whole query tile again with references taken from the data.
+// (Folding the scale into the Q fragments would save the fma too, but rounds Q once more: the error of a score then
+// grows with the score, and outlier keys came out 3x less accurate.  Not done.)
+//
+// What differs most from prefill_fwd.hip is who schedules the instructions.  The loop over the K/V tiles of a query
+// tile is hand-scheduled assembly (prefill_w64_asm.inc, written by gen_prefill_w64_loop.py: vector and LDS
+// instructions sit at fixed places in the shadow of the MFMAs, which one wavefront per SIMD cannot leave to chance);
+// it covers unmasked tiles, the tiles on the causal diagonal and the tiles above it.  Ragged ends, reference moves and
+// the recomputation go through step_cxx below, ordinary HIP code on the same state.
+//
+// Hand-over protocol between the two (and between tiles): when a tile step starts, its tile has landed in LDS, the
+// workgroup has met at a barrier after that, and the next tile's loads are in flight.  A step ends by waiting for its
+// own share of the next tile, meeting the others at the barrier and requesting the tile after next.
+#include <type_traits>
+
+#include "common.hpp"
+#include "launch.hpp"
+#include "prefill_params.hpp"
+#include "prefill_tile.hpp"
+#include "prefill_w64_asm.inc"
+
+namespace mi355 {
+
+// ---- the accumulators in the AGPRs, as ordinary code sees them ------------------------------------------------
+// O^T (2 column blocks x 4 d-tiles x 16 registers) and the row sums (2 x 4 registers) stay in a[0:135] for a whole
+// query tile.  This file is compiled with its builtin MFMAs in VGPR form (see build.py), so the compiler allocates no
+// AGPR of its own, and every statement below names the registers it touches as clobbered.
+template <int C, int DT>
+__device__ __forceinline__ void acc_pv(bf16x8 vt, bf16x8 pt) {      // O^T(C, DT) += vt . pt
+    if constexpr (C == 0 && DT == 0) asm volatile(W64_PV_0_0 : : "v"(vt), "v"(pt) : W64_CLOBBER_ACC);
+    if constexpr (C == 0 && DT == 1) asm volatile(W64_PV_0_1 : : "v"(vt), "v"(pt) : W64_CLOBBER_ACC);
+    if constexpr (C == 0 && DT == 2) asm volatile(W64_PV_0_2 : : "v"(vt), "v"(pt) : W64_CLOBBER_ACC);
+    if constexpr (C == 0 && DT == 3) asm volatile(W64_PV_0_3 : : "v"(vt), "v"(pt) : W64_CLOBBER_ACC);
+    if constexpr (C == 1 && DT == 0) asm volatile(W64_PV_1_0 : : "v"(vt), "v"(pt) : W64_CLOBBER_ACC);
+    if constexpr (C == 1 && DT == 1) asm volatile(W64_PV_1_1 : : "v"(vt), "v"(pt) : W64_CLOBBER_ACC);
+    if constexpr (C == 1 && DT == 2) asm volatile(W64_PV_1_2 : : "v"(vt), "v"(pt) : W64_CLOBBER_ACC);
+    if constexpr (C == 1 && DT == 3) asm volatile(W64_PV_1_3 : : "v"(vt), "v"(pt) : W64_CLOBBER_ACC);
+}
+template <int C>
+__device__ __forceinline__ void acc_sum(bf16x8 sum_a, bf16x8 pt) {  // row sums of block C += sum_a . pt
+    if constexpr (C == 0) asm volatile(W64_SUM_0 : : "v"(sum_a), "v"(pt) : W64_CLOBBER_ACC);
+    else asm volatile(W64_SUM_1 : : "v"(sum_a), "v"(pt) : W64_CLOBBER_ACC);
+}
+template <int C>
+__device__ __forceinline__ void acc_scale(float alpha, float a_lo, float a_hi) {   // O^T(C, .) *= alpha, row sums likewise
+    float scratch;
+    if constexpr (C == 0) asm volatile(W64_SCALE_0 : "=&v"(scratch) : "v"(alpha), "v"(a_lo), "v"(a_hi) : W64_CLOBBER_ACC);
+    else asm volatile(W64_SCALE_1 : "=&v"(scratch) : "v"(alpha), "v"(a_lo), "v"(a_hi) : W64_CLOBBER_ACC);
+}
+#define W64_OUT16(x) "=v"(x[0]), "=v"(x[1]), "=v"(x[2]), "=v"(x[3]), "=v"(x[4]), "=v"(x[5]), "=v"(x[6]), "=v"(x[7]), \
+                     "=v"(x[8]), "=v"(x[9]), "=v"(x[10]), "=v"(x[11]), "=v"(x[12]), "=v"(x[13]), "=v"(x[14]), "=v"(x[15])
+template <int C, int DT>
+__device__ __forceinline__ void acc_read(float (&x)[16]) {
+    if constexpr (C == 0 && DT == 0) asm volatile(W64_READ_0_0 : W64_OUT16(x) : : W64_CLOBBER_ACC);
+    if constexpr (C == 0 && DT == 1) asm volatile(W64_READ_0_1 : W64_OUT16(x) : : W64_CLOBBER_ACC);
+    if constexpr (C == 0 && DT == 2) asm volatile(W64_READ_0_2 : W64_OUT16(x) : : W64_CLOBBER_ACC);
+    if constexpr (C == 0 && DT == 3) asm volatile(W64_READ_0_3 : W64_OUT16(x) : : W64_CLOBBER_ACC);
+    if constexpr (C == 1 && DT == 0) asm volatile(W64_READ_1_0 : W64_OUT16(x) : : W64_CLOBBER_ACC);
+    if constexpr (C == 1 && DT == 1) asm volatile(W64_READ_1_1 : W64_OUT16(x) : : W64_CLOBBER_ACC);
+    if constexpr (C == 1 && DT == 2) asm volatile(W64_READ_1_2 : W64_OUT16(x) : : W64_CLOBBER_ACC);
+    if constexpr (C == 1 && DT == 3) asm volatile(W64_READ_1_3 : W64_OUT16(x) : : W64_CLOBBER_ACC);
+}
+template <int C>
+__device__ __forceinline__ void acc_read_sums(float& lo, float& hi) {
+    if constexpr (C == 0) asm volatile(W64_READL_0 : "=v"(lo), "=v"(hi) : : W64_CLOBBER_ACC);
+    else asm volatile(W64_READL_1 : "=v"(lo), "=v"(hi) : : W64_CLOBBER_ACC);
+}
+
+constexpr int kWWaves = 4;
+constexpr int kWBM = 256;            // queries per workgroup
+constexpr int kWBN = 64;             // keys per LDS tile
+constexpr int kWD = 128;
+constexpr int kWRow = kWD * 2;       // bytes per LDS row
+constexpr int kWTile = kWBN * kWRow; // bytes per K (or V) tile
+constexpr int kWORow = kWD * 2 + 16; // bytes per row of the query/output staging slab
+
+// Direct-to-LDS load of 16 bytes per lane (see dma_to_lds_16 in common.hpp).  This variant writes m0 inside the
+// statement: the assembly loop of this kernel writes m0 too, behind the compiler's back, so nothing here may rely on
+// the compiler's idea of what m0 holds.
+__device__ __forceinline__ void dma_to_lds_16_m0(const void* gbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voff), "s"(gbase), "s"(lds_addr)
+                 : "memory");
+}
+
+template <bool CAUSAL>
+__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p) {
+    constexpr int D = kWD, NS = D / 16, NDT = D / 32, CPR = D / 8;
+    constexpr float kBias = 32.0f;             // the largest weight sits at 2^-kBias when a reference is set
+    constexpr float kUnderflow = 0x1p-92f;     // a row sum below this may have lost terms (see the file header)
+
+    // K buffers 0,1 then V buffers 0,1 (the assembly loop addresses all four relative to one base)
+    __shared__ __attribute__((aligned(1024))) unsigned char kv_lds[4 * kWTile];
+    __shared__ __attribute__((aligned(16))) unsigned char o_lds[kWWaves * 64 * kWORow];
+    unsigned char* const k_lds = kv_lds;
+    unsigned char* const v_lds = kv_lds + 2 * kWTile;
+
+    const int n_wg = gridDim.x;
+    int lid = blockIdx.x;
+    if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;      // contiguous logical range per XCD
+    const int pair0 = lid % p.n_pairs;
+    const int h = (lid / p.n_pairs) % p.Hq;
+    const int b = lid / (p.n_pairs * p.Hq);
+    const int hk = h / (p.Hq / p.Hkv);
+
+    int sq, sk;
+    const __bf16 *qb, *kb, *vb;
+    __bf16* ob;
+    if (p.cu_q) {
+        const int q_start = p.cu_q[b], k_start = p.cu_k[b];
+        sq = p.cu_q[b + 1] - q_start;
+        sk = p.cu_k[b + 1] - k_start;
+        qb = p.q + (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
+        kb = p.k + (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
+        vb = p.v + (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
+        ob = p.out + (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
+    } else {
+        sq = p.Sq;
+        sk = p.Sk;
+        qb = p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
+        kb = p.k + (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
+        vb = p.v + (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
+        ob = p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[1];
+    }
+    const int nq = (sq + kWBM - 1) / kWBM;
+    if (2 * pair0 >= nq) return;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31;          // query column inside a block / key row of K / d row of V^T
+    const int kg = lane >> 5;
+    const int coff = sk - sq;         // bottom-right aligned causal diagonal
+
+    // ---- tile loader: wavefront w, instruction j covers LDS chunks (4w + j)*64 .. +63, i.e. rows 16w + 4j + lane/16;
+    // the lane fetches global chunk (lane%16) ^ swz(row) of its row, and swz(row) = ((lane/16) << 2) | j here ----
+    const int ld_q = lane >> 4;
+    const int ld_c0 = (lane & 15) ^ (ld_q << 2);
+    // byte offset of the lane's 16 bytes from the wavefront's first row of step j: row part + ((ld_c0 ^ j) << 4)
+    const uint32_t dma_row_k = (uint32_t)(ld_q * (int)p.ks[2] * 2), dma_row_v = (uint32_t)(ld_q * (int)p.vs[2] * 2);
+    const uint32_t lds_dst = __builtin_amdgcn_readfirstlane(lds_address(kv_lds + wave * 4096));
+    const uint32_t k_step = (uint32_t)(4 * p.ks[2] * 2), v_step = (uint32_t)(4 * p.vs[2] * 2);   // 4 rows, in bytes
+    auto issue_tile = [&](int tile, int buf) {
+        const unsigned char* kbase = reinterpret_cast<const unsigned char*>(kb + ((int64_t)tile * kWBN + 16 * wave) * p.ks[2]);
+        const unsigned char* vbase = reinterpret_cast<const unsigned char*>(vb + ((int64_t)tile * kWBN + 16 * wave) * p.vs[2]);
+        if (tile * kWBN + kWBN <= sk) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                dma_to_lds_16_m0(kbase + (size_t)j * k_step, dma_row_k + ((ld_c0 ^ j) << 4), lds_dst + buf * kWTile + j * 1024);
+                dma_to_lds_16_m0(vbase + (size_t)j * v_step, dma_row_v + ((ld_c0 ^ j) << 4), lds_dst + (2 + buf) * kWTile + j * 1024);
+            }
+        } else {
+            // last, partial tile: rows past the end re-read the last row (finite; their scores are masked)
+            const int last = sk - 1 - tile * kWBN;
+            const unsigned char* kt0 = reinterpret_cast<const unsigned char*>(kb + (int64_t)tile * kWBN * p.ks[2]);
+            const unsigned char* vt0 = reinterpret_cast<const unsigned char*>(vb + (int64_t)tile * kWBN * p.vs[2]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int row = min(16 * wave + 4 * j + ld_q, last);                 // row inside the tile
+                const int col = (ld_c0 ^ j) << 4;
+                dma_to_lds_16_m0(kt0, (uint32_t)(row * (int)p.ks[2] * 2 + col), lds_dst + buf * kWTile + j * 1024);
+                dma_to_lds_16_m0(vt0, (uint32_t)(row * (int)p.vs[2] * 2 + col), lds_dst + (2 + buf) * kWTile + j * 1024);
+            }
+        }
+    };
+
+    // ---- per-lane LDS read addresses for buffer 0 (absolute: the assembly loop uses them as they are) ----
+    // K fragment of step s, key row 32t + n: chunk (2s + kg) ^ swz(n);  V^T fragment of d-tile dt: source lane s16 of
+    // group g16 addresses key row 4(g16>>1) + (s16>>2) (+8 for the upper half), d = 32dt + 16(g16&1) + 4(s16&3)..+3
+    uint32_t rd_addr[16];             // [0..7] K per step, [8..11] V^T lower half per d-tile, [12..15] upper half
+    {
+        const uint32_t kbase = lds_address(k_lds), vbase = lds_address(v_lds);
+#pragma unroll
+        for (int s = 0; s < NS; ++s) rd_addr[s] = kbase + n * kWRow + (((2 * s + kg) ^ swz<D>(n)) << 4);
+        const int g16 = lane >> 4, s16 = lane & 15;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int row = 4 * (g16 >> 1) + (s16 >> 2) + 8 * e;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const int d = 32 * dt + 16 * (g16 & 1) + 4 * (s16 & 3);
+                rd_addr[8 + 4 * e + dt] = vbase + row * kWRow + ((((d >> 3)) ^ swz<D>(row)) << 4) + (d & 7) * 2;
+            }
+        }
+    }
+
+    // A operand of the row-sum MFMA (see prefill_fwd.hip): row 0 sums k = 0..7, 16..23 (query c), row 1 the rest (c + 16)
+    uint32_t sum_word;
+    {
+        const int r16 = lane & 15, g = (lane >> 4) & 1;
+        sum_word = ((r16 == 0 && g == 0) || (r16 == 1 && g == 1)) ? 0x3f803f80u : 0u;     // bf16 1.0 twice
+    }
+    const bf16x8 sum_a = as_bf16x8(u32x4{sum_word, sum_word, sum_word, sum_word});
+
+    for (int pair = pair0; 2 * pair < nq; pair += p.n_pairs)
+    for (int half = 0; half < 2; ++half) {
+        const int qtile = half == 0 ? nq - 1 - pair : pair;
+        if (half == 1 && qtile == nq - 1 - pair) break;
+        const int q0 = qtile * kWBM;
+        const int qw0 = q0 + 64 * wave;                    // first query of this wavefront
+
+        int kv_end = sk;
+        if (CAUSAL) kv_end = max(0, min(sk, min(sq, q0 + kWBM) + coff));
+        const int n_tiles = (kv_end + kWBN - 1) / kWBN;
+        // tile kinds of this wavefront: [0, n_plain) every key visible to each of its queries, [n_plain, n_mask) some,
+        // [n_mask, n_tiles) none (the wavefront then only takes part in the hand-over)
+        int n_plain = sk / kWBN, n_mask = n_tiles;
+        if (CAUSAL) {
+            n_plain = min(n_plain, max(0, qw0 + coff + 1) / kWBN);
+            n_mask = min(n_tiles, max(0, qw0 + 63 + coff + kWBN) / kWBN);      // first tile whose first key is past query qw0+63
+        }
+        n_plain = min(n_plain, n_tiles);
+        // the assembly loop requests tile+2 with whole-tile loads: it may run tile t only if tile t+2 is a whole tile
+        // (or does not exist), so it stops three tiles before a partial last tile
+        const int n_asm = n_tiles > sk / kWBN ? max(0, n_tiles - 3) : n_tiles;
+
+        // ---- Q rows -> staging slab (the fragments stay there for the whole query tile: the assembly loop loads them
+        // into its registers when it starts, ordinary code reads them as it needs them; the slab is reused for the
+        // output rows at the end).  Rows past the end of the sequence are zero. ----
+        unsigned char* const slab = o_lds + wave * (64 * kWORow);
+        __syncthreads();                     // the previous query tile's readers are done with the LDS buffers
+        if (n_tiles > 0) issue_tile(0, 0);
+        if (n_tiles > 1) issue_tile(1, 1);
+        {
+            constexpr int kRowsPerPass = 64 / CPR;           // 4 rows per pass, 16 passes
+            const int c16 = lane % CPR, r0 = lane / CPR;
+            u32x4 rows[64 / kRowsPerPass];
+#pragma unroll
+            for (int i = 0; i < 64 / kRowsPerPass; ++i) {
+                const int r = i * kRowsPerPass + r0;
+                rows[i] = u32x4{0u, 0u, 0u, 0u};
+                if (qw0 + r < sq) rows[i] = *reinterpret_cast<const u32x4*>(qb + (int64_t)(qw0 + r) * p.qs[2] + c16 * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 64 / kRowsPerPass; ++i)
+                *reinterpret_cast<u32x4*>(slab + (i * kRowsPerPass + r0) * kWORow + c16 * 16) = rows[i];
+        }
+        const uint32_t q_addr = lds_address(slab + n * kWORow + 8 * kg * 2);
+        auto qfrag = [&](int c, int s) { return as_bf16x8(lds_load_at<u32x4>(q_addr + c * 32 * kWORow + 32 * s)); };
+
+        // Two attempts at most: the first with the references preset to 0, the second -- only if some row's sum came
+        // out suspiciously small -- entirely in ordinary code with references taken from the data.
+        for (int attempt = 0; attempt < 2; ++attempt) {
+        const bool preset = attempt == 0;
+        if (!preset) {                        // start over: the buffers are free (everybody passed the vote below)
+            if (n_tiles > 0) issue_tile(0, 0);
+            if (n_tiles > 1) issue_tile(1, 1);
+        }
+        asm volatile(W64_ZERO : : : W64_CLOBBER_ACC);               // O^T and the row sums
+        // per column block: r_ref exponent reference in the log2 domain (-inf: none yet), nb = -r_ref - kBias
+        float r_ref[2], nb[2];
+        r_ref[0] = r_ref[1] = preset ? 0.f : -INFINITY;
+        nb[0] = nb[1] = preset ? -kBias : 0.f;
+
+        // wait for tile 0 (this wavefront's 8 loads of tile 1 may stay in flight), meet the others
+        if (n_tiles > 1) wait_vmcnt<8>(); else wait_vmcnt<0>();
+        __syncthreads();
+
+        // One 32-key half of a tile for one column block, in ordinary code: scores, mask, reference move, weights,
+        // accumulation.  (Rare: ragged end, a row maximum that outgrew its reference, the second attempt.)
+        auto sub_block = [&](auto c_c, int tile, int t, bool masked) {
+            constexpr int c = decltype(c_c)::value;
+            const int buf = tile & 1;
+            const int k0 = tile * kWBN + 32 * t;
+            f32x16 s_acc;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) s_acc[j] = 0.f;
+            // (all fragment reads first, then the MFMAs: one LDS latency instead of eight)
+            u32x4 kf[NS];
+            bf16x8 qf[NS];
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                kf[s] = lds_load_at<u32x4>(rd_addr[s] + buf * kWTile + t * 32 * kWRow);
+                qf[s] = qfrag(c, s);
+            }
+#pragma unroll
+            for (int s = 0; s < NS; ++s) s_acc = mfma32(as_bf16x8(kf[s]), qf[s], s_acc);
+            const int qi = qw0 + 32 * c + n;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float x = fmaf(s_acc[i], p.scale_log2, nb[c]);
+                if (masked) {
+                    const int key = k0 + 8 * (i >> 2) + 4 * kg + (i & 3);
+                    bool keep = key < sk;
+                    if (CAUSAL) keep = keep & (key <= qi + coff);
+                    x = keep ? x : -INFINITY;
+                }
+                s_acc[i] = x;
+                mx = fmaxf(mx, x);
+            }
+            mx = xor32_max(mx);
+            const float r_new = fmaxf(r_ref[c], mx - nb[c]);
+            const float alpha = r_ref[c] == -INFINITY ? 1.0f : fast_exp2(r_ref[c] - r_new);
+            const float nb_new = r_new == -INFINITY ? 0.f : -r_new - kBias;
+            const float delta = nb_new - nb[c];
+            r_ref[c] = r_new;
+            nb[c] = nb_new;
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0)      // (lanes 0..15 hold the sums of queries c and c + 16)
+                acc_scale<c>(alpha, __shfl(alpha, lane & 15, 64), __shfl(alpha, (lane & 15) + 16, 64));
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const int u = 2 * t + hf;
+                u32x4 pw;
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    pw[w] = pack_bf16(fast_exp2(s_acc[8 * hf + 2 * w] + delta), fast_exp2(s_acc[8 * hf + 2 * w + 1] + delta));
+                const bf16x8 pf = as_bf16x8(pw);
+                bf16x8 vf[NDT];
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+                    vf[dt] = join_bf16x8(lds_read_tr16_at(rd_addr[8 + dt] + buf * kWTile + 16 * u * kWRow),
+                                         lds_read_tr16_at(rd_addr[12 + dt] + buf * kWTile + 16 * u * kWRow));
+                acc_sum<c>(sum_a, pf);
+                acc_pv<c, 0>(vf[0], pf);
+                acc_pv<c, 1>(vf[1], pf);
+                acc_pv<c, 2>(vf[2], pf);
+                acc_pv<c, 3>(vf[3], pf);
+            }
+        };
+        // the end of every tile step: own share of the next tile landed, everybody done with this one, tile+2 requested
+        auto hand_over = [&](int tile) {
+            if (tile + 1 < n_tiles) {
+                wait_vmcnt<0>();
+                __syncthreads();
+                if (tile + 2 < n_tiles) issue_tile(tile + 2, tile & 1);
+            }
+        };
+        auto step_cxx = [&](int tile, int t_first) {
+            if (tile < n_mask) {                      // (a tile past n_mask has nothing for this wavefront)
+                const bool masked = tile >= n_plain;
+                for (int t = t_first; t < 2; ++t) {
+                    sub_block(std::integral_constant<int, 0>{}, tile, t, masked);
+                    sub_block(std::integral_constant<int, 1>{}, tile, t, masked);
+                }
+            }
+            hand_over(tile);
+        };
+
+        int tile = 0;
+        const int n_loop = preset ? n_asm : 0;
+        while (tile < n_tiles) {
+            if (tile >= n_loop) {
+                step_cxx(tile, 0);
+                ++tile;
+                continue;
+            }
+            // ---- the hand-scheduled loop over tiles [tile, n_loop); leaves early when a weight reaches 2 ----
+            const uint64_t kptr = (uint64_t)(uintptr_t)(kb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.ks[2]);
+            const uint64_t vptr = (uint64_t)(uintptr_t)(vb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.vs[2]);
+            // mask thresholds for the first masked tile the loop will meet: a key at index j of that tile is kept by
+            // query i of the wavefront iff j <= i + (qw0 + coff - k0) and j < sk - k0 (the lane part 4*kg of a key's
+            // index is folded in)
+            const int k0m = max(tile, n_plain) * kWBN;
+            const int diag = CAUSAL ? qw0 + coff - k0m : (1 << 20);
+            // vector operands: read once when the block starts, scratch registers of the block afterwards
+            float v_nb0 = nb[0], v_nb1 = nb[1];
+            int v_thr0 = min(n + diag, sk - 1 - k0m) - 4 * kg, v_thr1 = min(n + 32 + diag, sk - 1 - k0m) - 4 * kg;
+            uint32_t v_sum = sum_word, v_k0 = rd_addr[0], v_vlo = rd_addr[8], v_vhi = rd_addr[12];
+            uint32_t v_rowk = dma_row_k, v_rowv = dma_row_v, v_c0s = (uint32_t)(ld_c0 << 4), v_q = q_addr;
+            int status;
+            int tile_s = __builtin_amdgcn_readfirstlane(tile);
+            asm volatile(W64_LOOP
+                : [tile] "+&s"(tile_s), [t2] "=&s"(status),
+                  [nb0] "+v"(v_nb0), [nb1] "+v"(v_nb1), [suma] "+v"(v_sum), [k0] "+v"(v_k0), [vlo0] "+v"(v_vlo),
+                  [vhi0] "+v"(v_vhi), [rowk] "+v"(v_rowk), [rowv] "+v"(v_rowv), [c0s] "+v"(v_c0s), [qaddr] "+v"(v_q),
+                  [thr0] "+v"(v_thr0), [thr1] "+v"(v_thr1)
+                : [n_tiles] "s"(__builtin_amdgcn_readfirstlane(n_tiles)), [n_end] "s"(__builtin_amdgcn_readfirstlane(n_loop)),
+                  [n_plain] "s"(__builtin_amdgcn_readfirstlane(n_plain)), [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)),
+                  [kstep] "s"(__builtin_amdgcn_readfirstlane(k_step)), [vstep] "s"(__builtin_amdgcn_readfirstlane(v_step)),
+                  [ldsdst] "s"(lds_dst), [scale] "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, p.scale_log2))),
+                  [klo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)kptr)), [khi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kptr >> 32))),
+                  [vlo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)vptr)), [vhi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(vptr >> 32)))
+                : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
+            tile = tile_s;
+            // status 0: tiles up to n_loop done.  1: a weight of tile `tile` reached 2, nothing of that tile is
+            // accumulated.  2: likewise for its keys 32..63; keys 0..31 are accumulated.
+            if (status != 0) {
+                step_cxx(tile, status == 2 ? 1 : 0);
+                ++tile;
+            }
+        }
+
+        // ---- row sums; on the first attempt the workgroup votes on doing the query tile again ----
+        float l_row[2];
+        const auto read_sums = [&](auto c_c) {
+            constexpr int c = decltype(c_c)::value;
+            float s_lo, s_hi;
+            acc_read_sums<c>(s_lo, s_hi);
+            const float l_lo = __shfl(s_lo, lane & 15, 64), l_hi = __shfl(s_hi, lane & 15, 64);
+            l_row[c] = (n & 16) ? l_hi : l_lo;
+        };
+        read_sums(std::integral_constant<int, 0>{});
+        read_sums(std::integral_constant<int, 1>{});
+        if (preset) {
+            // (rows past the end of the sequence count too: their sums are sk * 2^-32, far above the limit)
+            const bool small = !(l_row[0] >= kUnderflow) || !(l_row[1] >= kUnderflow);
+            if (__syncthreads_or(small ? 1 : 0)) continue;
+        }
+
+        // ---- normalise and store: lane owns query qw0 + 32c + n, d = 32dt + 8(i/4) + 4kg + i%4 ----
+        const auto store_block = [&](auto c_c) {
+            constexpr int c = decltype(c_c)::value;
+            const float inv = 1.0f / l_row[c];     // l == 0 (no key kept) -> NaN row, like the reference softmax
+            unsigned char* mine = slab + (32 * c + n) * kWORow + 8 * kg;
+            const auto store_dt = [&](auto dt_c) {
+                constexpr int dt = decltype(dt_c)::value;
+                float x[16];
+                acc_read<c, dt>(x);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    u32x2 w;
+                    w[0] = pack_bf16(x[4 * g + 0] * inv, x[4 * g + 1] * inv);
+                    w[1] = pack_bf16(x[4 * g + 2] * inv, x[4 * g + 3] * inv);
+                    *reinterpret_cast<u32x2*>(mine + (32 * dt + 8 * g) * 2) = w;
+                }
+            };
+            store_dt(std::integral_constant<int, 0>{});
+            store_dt(std::integral_constant<int, 1>{});
+            store_dt(std::integral_constant<int, 2>{});
+            store_dt(std::integral_constant<int, 3>{});
+        };
+        store_block(std::integral_constant<int, 0>{});
+        store_block(std::integral_constant<int, 1>{});
+        break;
+        }   // attempts
+        {
+            constexpr int kRowsPerPass = 64 / CPR;
+            const int c16 = lane % CPR, r0 = lane / CPR;
+#pragma unroll
+            for (int i = 0; i < 64 / kRowsPerPass; ++i) {
+                const int r = i * kRowsPerPass + r0;
+                const u32x4 w = *reinterpret_cast<const u32x4*>(slab + r * kWORow + c16 * 16);
+                if (qw0 + r < sq) *reinterpret_cast<u32x4*>(ob + (int64_t)(qw0 + r) * p.os[2] + c16 * 8) = w;
+            }
+        }
+    }
+}
+
+int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
+    dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B)), block(kWWaves * 64);
+    if (p.mask_mode == MI355_MASK_CAUSAL)
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), grid, block, 0, stream, p);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mi355

@@ -275,6 +275,45 @@ def test_prefill_varlen_ragged(ops, lens):
     check(got, ref, what="varlen")
 
 
+@pytest.mark.parametrize("Sq,Sk", [(256, 4096), (700, 1500), (64, 191), (513, 64), (300, 8192 + 37)])
+def test_prefill_unmasked_head_dim_128_long_and_ragged(ops, Sq, Sk):
+    """head_dim 128 without a mask runs on the kernel with 64 queries per wavefront, whose loop over whole K/V tiles
+    is hand-scheduled assembly: many tiles, ragged query and key ends (the assembly stops three tiles before a
+    partial last tile), GQA, fewer rows than a wavefront owns."""
+    print(f"case: prefill unmasked D128 Sq={Sq} Sk={Sk}", flush=True)
+    B, Hq, Hkv, D = 2, 4, 2, 128
+    q, k, v = rnd(B, Hq, Sq, D, seed=81, scale=0.5), rnd(B, Hkv, Sk, D, seed=82, scale=0.5), rnd(B, Hkv, Sk, D, seed=83, scale=0.5)
+    ref = orc.prefill_reference(q, k, v, causal=False)
+    got = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=False)
+    torch.cuda.synchronize()
+    check(got, ref, what=f"unmasked D128 {Sq}x{Sk}")
+    # the reference's own signature (no GQA there: first kv head only) lands on the same kernel
+    got2 = ops.scaled_dot_product_attention(q[:, :2].cuda(), k[:, :1].cuda(), v[:, :1].cuda())
+    assert torch.equal(got[:, :2], got2)
+
+
+def test_prefill_unmasked_scores_that_outgrow_the_reference(ops):
+    """Keys far along the sequence whose scores exceed everything before them by hundreds of binary orders: the
+    assembly loop sees a weight reach 2, leaves (once with nothing of the tile accumulated, once with half of it),
+    ordinary code moves the reference and the loop resumes.  Also a block of keys with hugely negative scores."""
+    print("case: prefill unmasked D128, reference moves", flush=True)
+    B, H, Sq, Sk, D = 1, 2, 128, 2048, 128
+    q, k, v = rnd(B, H, Sq, D, seed=84, scale=1.0), rnd(B, H, Sk, D, seed=85, scale=1.0), rnd(B, H, Sk, D, seed=86, scale=1.0)
+    k = k.float()
+    k[:, :, 700] *= 9.0            # keys 0..31 of tile 10: first check of that tile
+    k[:, :, 1000] *= 30.0          # key 40 of tile 15: second check (keys 32..63)
+    k[:, :, 1300:1364] *= -25.0    # a whole tile of extreme scores of both signs
+    k[:, :, 1999] *= 60.0
+    k = k.to(torch.bfloat16)
+    ref = orc.prefill_reference(q, k, v, causal=False)
+    got = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=False)
+    torch.cuda.synchronize()
+    check(got, ref, what="reference moves")
+    # the same through the 8-wavefront kernel (an all-true explicit mask takes that path): both must agree with the oracle
+    keep = torch.ones(Sq, Sk, dtype=torch.bool, device="cuda")
+    check(ops.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), keep), ref, what="reference moves, masked path")
+
+
 def _reference_module_tensors(x_proj, freq, num_heads, amp):
     """Q, K, V exactly as CausalMultiHeadSelfAttention.forward hands them to the attention call
     (llm-core/llm_core/model.py:362-378) from the three projection outputs (B, S, H*d): `rearrange` views, then
