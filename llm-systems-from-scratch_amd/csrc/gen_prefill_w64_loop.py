@@ -22,7 +22,9 @@ One tile (64 keys) of one wavefront (64 queries = column blocks A and B, head_di
   phase 4b  O += V[48:64]^T . P(.,1)             8 + 2 MFMA: covers the latency of those reads
 Tiles come in three kinds, by index: [0, n_plain) every key visible to every query; [n_plain, n_mask) masked (causal
 diagonal: key <= threshold of the lane's query; the threshold moves down by 64 per tile); [n_mask, n_end) nothing
-visible for this wavefront -- it only takes part in the hand-over.
+visible for this wavefront -- it only takes part in the hand-over.  When the diagonal is aligned with the tiles
+(operand `aligned`: query i of the wavefront sees key j of the one masked tile iff j <= i) that tile takes a cheaper
+body: only the two triangular 32x32 sub-blocks get mask code, and the invisible one is neither scored nor accumulated.
 
 Register map (physical, fixed; the block loads them itself from its operands, see entry()):
   v[0:31] Q^T fragments of block A (step s = v[4s:4s+3]), v[32:63] block B
@@ -135,19 +137,20 @@ def v_read(e, buf, u, dt, base):
     e.lds_read(f"ds_read_b64_tr_b16 v{rng(base + 2, 2)}, v{VOFF + 4 + dt} offset:{off}", base + 2)
 
 
-def exp_ops(t, dst, masked):
-    """Vector work that turns S(.,t) into packed bf16 weights in dst[block] (+ slice * 4).  The result of a
-    transcendental may not feed the next vector instruction, so the packing of a pair trails its exponentials.
-    Accumulator register i of a lane holds key 32t + 8(i/4) + 4(lane/32) + i%4 of the tile; a masked tile keeps the
-    score only if that index is <= the lane's threshold (the lane part of the index is folded into the threshold)."""
+def exp_ops(t, dst, mask, blocks="AB"):
+    """Vector work that turns S(c,t), c in `blocks`, into packed bf16 weights in dst[c] (+ slice * 4).  The result of
+    a transcendental may not feed the next vector instruction, so the packing of a pair trails its exponentials.
+    Accumulator register i of a lane holds key 32t + 8(i/4) + 4(lane/32) + i%4 of the tile; where mask[c] is set the
+    score is kept only if that index is <= the lane's threshold (the lane part of the index is folded into the
+    threshold)."""
     ops, pend = [], []
     i = 0
-    for c in "AB":
+    for c in blocks:
         for w in range(8):                      # packed word w of the block: accumulator registers 2w, 2w+1
             t0, t1 = ETMP[2 * (i % 4)], ETMP[2 * (i % 4) + 1]
             for tmp, r in ((t0, 2 * w), (t1, 2 * w + 1)):
                 ops.append(f"v_fma_f32 {tmp}, v{S[(c, t)] + r}, %[scale], v{NB[c]}")
-                if masked:
+                if mask[c]:
                     ops.append(f"v_cmp_le_i32_e64 vcc, {32 * t + 8 * (r // 4) + r % 4}, v{THR[c]}")
                     ops.append(f"v_cndmask_b32 {tmp}, v{NEGINF}, {tmp}, vcc")
             ops.append(f"v_exp_f32 {t0}, {t0}")
@@ -224,10 +227,23 @@ def hand_over(e, buf, tag):
     e.raw(f"7{tag}:")
 
 
-def tile_body(e, buf, masked):
-    tag = f"{buf}{1 if masked else 0}"
+KINDS = {"plain": 0, "masked": 1, "diag": 3}
+
+
+def tile_body(e, buf, kind):
+    """kind: "plain" no mask; "masked" every score against its threshold; "diag" the tile on an ALIGNED causal
+    diagonal (query i of the wavefront sees key j of the tile iff j <= i): S(A,0) and S(B,1) are triangular, S(B,0)
+    is fully visible, and S(A,1) is not computed at all -- block A neither scores nor accumulates keys 32..63."""
+    tag = f"{buf}{KINDS[kind]}"
+    diag = kind == "diag"
+    t1_blocks = "B" if diag else "AB"
+    mask0 = {"A": kind != "plain", "B": kind == "masked"}
+    mask1 = {"A": kind == "masked", "B": kind != "plain"}
+    qreg = {"A": QA, "B": QB}
+    oreg = {"A": OA, "B": OB}
+    lreg = {"A": LA, "B": LB}
     # ---- phase 1: scores of keys 0..31.  K fragments 0..3 of this tile are in flight (or in registers) ----
-    e.raw(f"; ---- {'masked' if masked else 'plain'} tile in buffer {buf}: phase 1")
+    e.raw(f"; ---- {kind} tile in buffer {buf}: phase 1")
     m = []
     for s in range(8):
         slot = s % 4
@@ -252,9 +268,10 @@ def tile_body(e, buf, masked):
             else:
                 dt = s - 4
                 v_read(e, buf, 0, dt, VF0 + 4 * dt)
-        m.append((mfma32_v(S[("A", 1)], KF + 4 * slot, QA + 4 * s, None if s == 0 else S[("A", 1)]), (KF + 4 * slot,), None))
-        m.append((mfma32_v(S[("B", 1)], KF + 4 * slot, QB + 4 * s, None if s == 0 else S[("B", 1)]), None, refill))
-    spread(e, m, exp_ops(0, PW0, masked), hold=3)
+        for ci, c in enumerate(t1_blocks):
+            m.append((mfma32_v(S[(c, 1)], KF + 4 * slot, qreg[c] + 4 * s, None if s == 0 else S[(c, 1)]),
+                      (KF + 4 * slot,) if ci == 0 else None, refill if ci == len(t1_blocks) - 1 else None))
+    spread(e, m, exp_ops(0, PW0, mask0), hold=1 if diag else 3)
     check(e, "91f")
     # ---- phase 3: values of keys 0..31 | weights of keys 32..63 ----
     e.raw("; phase 3")
@@ -270,25 +287,25 @@ def tile_body(e, buf, masked):
                 v_read(e, buf, u + 2, dt, vf + 4 * dt)
             m.append((mfma32_a(OA + 16 * dt, vf + 4 * dt, PW0["A"] + 4 * u), (vf + 4 * dt, vf + 4 * dt + 2), None))
             m.append((mfma32_a(OB + 16 * dt, vf + 4 * dt, PW0["B"] + 4 * u), None, refill))
-    spread(e, m, exp_ops(1, PW1, masked), hold=3)
+    spread(e, m, exp_ops(1, PW1, mask1, t1_blocks), hold=3)
     check(e, "92f")
     # ---- phase 4a: values of keys 32..47 (fragments are in registers or about to arrive) ----
     e.raw("; phase 4a")
-    m = [(mfma16_a(LA, SUMA, PW1["A"]), None, None), (mfma16_a(LB, SUMA, PW1["B"]), None, None)]
+    m = [(mfma16_a(lreg[c], SUMA, PW1[c]), None, None) for c in t1_blocks]
     for dt in range(4):
-        m.append((mfma32_a(OA + 16 * dt, VF0 + 4 * dt, PW1["A"]), (VF0 + 4 * dt, VF0 + 4 * dt + 2), None))
-        m.append((mfma32_a(OB + 16 * dt, VF0 + 4 * dt, PW1["B"]), None, None))
+        for ci, c in enumerate(t1_blocks):
+            m.append((mfma32_a(oreg[c] + 16 * dt, VF0 + 4 * dt, PW1[c]), (VF0 + 4 * dt, VF0 + 4 * dt + 2) if ci == 0 else None, None))
     spread(e, m, [])
-    if masked:                                   # the next tile's keys are 64 further along: thresholds move down
+    if kind != "plain":                          # the next tile's keys are 64 further along: thresholds move down
         e.raw(f"v_subrev_u32 v{THR['A']}, 64, v{THR['A']}")
         e.raw(f"v_subrev_u32 v{THR['B']}, 64, v{THR['B']}")
     hand_over(e, buf, tag)
     # ---- phase 4b: values of keys 48..63 ----
     e.raw("; phase 4b")
-    m = [(mfma16_a(LA, SUMA, PW1["A"] + 4), None, None), (mfma16_a(LB, SUMA, PW1["B"] + 4), None, None)]
+    m = [(mfma16_a(lreg[c], SUMA, PW1[c] + 4), None, None) for c in t1_blocks]
     for dt in range(4):
-        m.append((mfma32_a(OA + 16 * dt, VF1 + 4 * dt, PW1["A"] + 4), None, None))
-        m.append((mfma32_a(OB + 16 * dt, VF1 + 4 * dt, PW1["B"] + 4), None, None))
+        for c in t1_blocks:
+            m.append((mfma32_a(oreg[c] + 16 * dt, VF1 + 4 * dt, PW1[c] + 4), None, None))
     spread(e, m, [])
     e.raw("s_branch 20b")
 
@@ -350,14 +367,16 @@ def generate():
             e.raw(f"{lab}:")
         e.raw("s_cmp_lt_u32 %[tile], %[n_plain]")
         e.raw(f"s_cbranch_scc1 3{buf}0f")
-        e.raw("s_cmp_lt_u32 %[tile], %[n_mask]")
-        e.raw(f"s_cbranch_scc1 3{buf}1f")
-        e.raw(f"s_branch 3{buf}2f")
+        e.raw("s_cmp_ge_u32 %[tile], %[n_mask]")
+        e.raw(f"s_cbranch_scc1 3{buf}2f")
+        e.raw("s_cmp_lg_u32 %[aligned], 0")              # masked: on an aligned diagonal the cheaper body
+        e.raw(f"s_cbranch_scc1 3{buf}3f")
+        e.raw(f"s_branch 3{buf}1f")
     for buf in (0, 1):
-        for masked in (False, True):
+        for kind in ("plain", "masked", "diag"):
             e.pending = list(start)
-            e.raw(f"3{buf}{1 if masked else 0}:")
-            tile_body(e, buf, masked)
+            e.raw(f"3{buf}{KINDS[kind]}:")
+            tile_body(e, buf, kind)
             assert e.pending == start, (e.pending, start)
         # nothing visible in this tile: the wavefront only takes part in the hand-over
         e.pending = list(start)

@@ -101,7 +101,7 @@ __device__ __forceinline__ void dma_to_lds_16_m0(const void* gbase, uint32_t vof
 }
 
 template <bool CAUSAL>
-__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p) {
+__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int n_logical) {
     constexpr int D = kWD, NS = D / 16, NDT = D / 32, CPR = D / 8;
     constexpr float kBias = 32.0f;             // the largest weight sits at 2^-kBias when a reference is set
     constexpr float kUnderflow = 0x1p-92f;     // a row sum below this may have lost terms (see the file header)
@@ -112,42 +112,69 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     unsigned char* const k_lds = kv_lds;
     unsigned char* const v_lds = kv_lds + 2 * kWTile;
 
-    const int n_wg = gridDim.x;
-    int lid = blockIdx.x;
-    if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;      // contiguous logical range per XCD
-    const int pair0 = lid % p.n_pairs;
-    const int h = (lid / p.n_pairs) % p.Hq;
-    const int b = lid / (p.n_pairs * p.Hq);
-    const int hk = h / (p.Hq / p.Hkv);
-
-    int sq, sk;
-    const __bf16 *qb, *kb, *vb;
-    __bf16* ob;
-    if (p.cu_q) {
-        const int q_start = p.cu_q[b], k_start = p.cu_k[b];
-        sq = p.cu_q[b + 1] - q_start;
-        sk = p.cu_k[b + 1] - k_start;
-        qb = p.q + (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
-        kb = p.k + (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
-        vb = p.v + (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
-        ob = p.out + (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
-    } else {
-        sq = p.Sq;
-        sk = p.Sk;
-        qb = p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
-        kb = p.k + (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
-        vb = p.v + (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
-        ob = p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[1];
-    }
-    const int nq = (sq + kWBM - 1) / kWBM;
-    if (2 * pair0 >= nq) return;
-
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31;          // query column inside a block / key row of K / d row of V^T
     const int kg = lane >> 5;
-    const int coff = sk - sq;         // bottom-right aligned causal diagonal
+
+    // ---- jobs: a workgroup works through query tiles, one "job" each.  Logical id = (batch, head, tile pair); a
+    // pair is the query tiles (nq-1-i, i) of a sequence, so that causal work is the same for every id.  The ids are
+    // dealt so that the workgroups resident on one XCD (workgroup ids are dealt round-robin to the 8 XCDs) walk
+    // through one contiguous range of ids together and stream the same K/V through that XCD's L2. ----
+    struct Job {
+        const __bf16 *qb, *kb, *vb;
+        __bf16* ob;
+        int sq, sk, q0;
+    };
+    const int G = gridDim.x, bid = blockIdx.x;
+    const bool by_xcd = (n_logical % 8 == 0) && (G % 8 == 0);
+    int job_k = -1, job_nq = 0, job_pair = 0, job_half = 1;      // position: "after the last query tile of id number job_k"
+    Job job_seq{};                                               // sequence-level fields of the current id
+    auto next_job = [&](Job& j) -> bool {
+        if (job_half == 0 && job_pair != job_nq - 1 - job_pair) {           // second query tile of the pair
+            job_half = 1;
+            j = job_seq;
+            j.q0 = job_pair * kWBM;
+            return true;
+        }
+        job_pair += p.n_pairs;                // a further pair of the same sequence: only if it is longer than Sq_max promised
+        while (!(job_k >= 0 && 2 * job_pair < job_nq)) {
+            ++job_k;
+            int lid;
+            if (by_xcd) {
+                const int per = n_logical / 8, slot = bid / 8 + job_k * (G / 8);
+                if (slot >= per) return false;
+                lid = (bid % 8) * per + slot;
+            } else {
+                lid = bid + job_k * G;
+                if (lid >= n_logical) return false;
+            }
+            const int h = (lid / p.n_pairs) % p.Hq, b = lid / (p.n_pairs * p.Hq), hk = h / (p.Hq / p.Hkv);
+            if (p.cu_q) {
+                const int q_start = p.cu_q[b], k_start = p.cu_k[b];
+                job_seq.sq = p.cu_q[b + 1] - q_start;
+                job_seq.sk = p.cu_k[b + 1] - k_start;
+                job_seq.qb = p.q + (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
+                job_seq.kb = p.k + (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
+                job_seq.vb = p.v + (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
+                job_seq.ob = p.out + (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
+            } else {
+                job_seq.sq = p.Sq;
+                job_seq.sk = p.Sk;
+                job_seq.qb = p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
+                job_seq.kb = p.k + (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
+                job_seq.vb = p.v + (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
+                job_seq.ob = p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[1];
+            }
+            job_nq = (job_seq.sq + kWBM - 1) / kWBM;
+            job_pair = lid % p.n_pairs;
+        }
+        job_half = 0;
+        j = job_seq;
+        j.q0 = (job_nq - 1 - job_pair) * kWBM;
+        return true;
+    };
 
     // ---- tile loader: wavefront w, instruction j covers LDS chunks (4w + j)*64 .. +63, i.e. rows 16w + 4j + lane/16;
     // the lane fetches global chunk (lane%16) ^ swz(row) of its row, and swz(row) = ((lane/16) << 2) | j here ----
@@ -157,10 +184,10 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const uint32_t dma_row_k = (uint32_t)(ld_q * (int)p.ks[2] * 2), dma_row_v = (uint32_t)(ld_q * (int)p.vs[2] * 2);
     const uint32_t lds_dst = __builtin_amdgcn_readfirstlane(lds_address(kv_lds + wave * 4096));
     const uint32_t k_step = (uint32_t)(4 * p.ks[2] * 2), v_step = (uint32_t)(4 * p.vs[2] * 2);   // 4 rows, in bytes
-    auto issue_tile = [&](int tile, int buf) {
-        const unsigned char* kbase = reinterpret_cast<const unsigned char*>(kb + ((int64_t)tile * kWBN + 16 * wave) * p.ks[2]);
-        const unsigned char* vbase = reinterpret_cast<const unsigned char*>(vb + ((int64_t)tile * kWBN + 16 * wave) * p.vs[2]);
-        if (tile * kWBN + kWBN <= sk) {
+    auto issue_tile = [&](const Job& jb, int tile, int buf) {
+        const unsigned char* kbase = reinterpret_cast<const unsigned char*>(jb.kb + ((int64_t)tile * kWBN + 16 * wave) * p.ks[2]);
+        const unsigned char* vbase = reinterpret_cast<const unsigned char*>(jb.vb + ((int64_t)tile * kWBN + 16 * wave) * p.vs[2]);
+        if (tile * kWBN + kWBN <= jb.sk) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 dma_to_lds_16_m0(kbase + (size_t)j * k_step, dma_row_k + ((ld_c0 ^ j) << 4), lds_dst + buf * kWTile + j * 1024);
@@ -168,9 +195,9 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             }
         } else {
             // last, partial tile: rows past the end re-read the last row (finite; their scores are masked)
-            const int last = sk - 1 - tile * kWBN;
-            const unsigned char* kt0 = reinterpret_cast<const unsigned char*>(kb + (int64_t)tile * kWBN * p.ks[2]);
-            const unsigned char* vt0 = reinterpret_cast<const unsigned char*>(vb + (int64_t)tile * kWBN * p.vs[2]);
+            const int last = jb.sk - 1 - tile * kWBN;
+            const unsigned char* kt0 = reinterpret_cast<const unsigned char*>(jb.kb + (int64_t)tile * kWBN * p.ks[2]);
+            const unsigned char* vt0 = reinterpret_cast<const unsigned char*>(jb.vb + (int64_t)tile * kWBN * p.vs[2]);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int row = min(16 * wave + 4 * j + ld_q, last);                 // row inside the tile
@@ -179,6 +206,12 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 dma_to_lds_16_m0(vt0, (uint32_t)(row * (int)p.vs[2] * 2 + col), lds_dst + (2 + buf) * kWTile + j * 1024);
             }
         }
+    };
+    // number of K/V tiles of a job (the same for the four wavefronts)
+    auto tiles_of = [&](const Job& jb) {
+        int kv_end = jb.sk;
+        if (CAUSAL) kv_end = max(0, min(jb.sk, min(jb.sq, jb.q0 + kWBM) + (jb.sk - jb.sq)));
+        return (kv_end + kWBN - 1) / kWBN;
     };
 
     // ---- per-lane LDS read addresses for buffer 0 (absolute: the assembly loop uses them as they are) ----
@@ -209,16 +242,39 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     }
     const bf16x8 sum_a = as_bf16x8(u32x4{sum_word, sum_word, sum_word, sum_word});
 
-    for (int pair = pair0; 2 * pair < nq; pair += p.n_pairs)
-    for (int half = 0; half < 2; ++half) {
-        const int qtile = half == 0 ? nq - 1 - pair : pair;
-        if (half == 1 && qtile == nq - 1 - pair) break;
-        const int q0 = qtile * kWBM;
-        const int qw0 = q0 + 64 * wave;                    // first query of this wavefront
+    // The staging slab of the wavefront: its 64 query rows during a job (the assembly loop loads its fragments from
+    // here whenever it starts, ordinary code reads them as it needs them), the output rows at the end of the job.
+    unsigned char* const slab = o_lds + wave * (64 * kWORow);
+    const uint32_t q_addr = lds_address(slab + n * kWORow + 8 * kg * 2);
+    auto qfrag = [&](int c, int s) { return as_bf16x8(lds_load_at<u32x4>(q_addr + c * 32 * kWORow + 32 * s)); };
+    constexpr int kRowsPerPass = 64 / CPR;           // the slab is filled and emptied 4 whole rows at a time, 16 passes
+    const int c16 = lane % CPR, r0 = lane / CPR;
 
-        int kv_end = sk;
-        if (CAUSAL) kv_end = max(0, min(sk, min(sq, q0 + kWBM) + coff));
-        const int n_tiles = (kv_end + kWBN - 1) / kWBN;
+    // What a job needs before it can start is requested as early as possible -- for the first job right here, for
+    // every other one while the job before it normalises and stores its output: K/V tiles 0 and 1 (direct-to-LDS)
+    // and the wavefront's query rows (into registers; rows past the end of the sequence are zero).
+    u32x4 q_rows[64 / kRowsPerPass];
+    auto prefetch = [&](const Job& jb) {
+        const int nt = tiles_of(jb);
+        if (nt > 0) issue_tile(jb, 0, 0);
+        if (nt > 1) issue_tile(jb, 1, 1);
+        const int qw0 = jb.q0 + 64 * wave;
+#pragma unroll
+        for (int i = 0; i < 64 / kRowsPerPass; ++i) {
+            const int r = i * kRowsPerPass + r0;
+            q_rows[i] = u32x4{0u, 0u, 0u, 0u};
+            if (qw0 + r < jb.sq) q_rows[i] = *reinterpret_cast<const u32x4*>(jb.qb + (int64_t)(qw0 + r) * p.qs[2] + c16 * 8);
+        }
+    };
+
+    Job cur{}, nxt{};
+    bool have = next_job(cur);
+    if (have) prefetch(cur);
+    while (have) {
+        const int sq = cur.sq, sk = cur.sk, q0 = cur.q0;
+        const int coff = sk - sq;                          // bottom-right aligned causal diagonal
+        const int qw0 = q0 + 64 * wave;                    // first query of this wavefront
+        const int n_tiles = tiles_of(cur);
         // tile kinds of this wavefront: [0, n_plain) every key visible to each of its queries, [n_plain, n_mask) some,
         // [n_mask, n_tiles) none (the wavefront then only takes part in the hand-over)
         int n_plain = sk / kWBN, n_mask = n_tiles;
@@ -227,41 +283,26 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             n_mask = min(n_tiles, max(0, qw0 + 63 + coff + kWBN) / kWBN);      // first tile whose first key is past query qw0+63
         }
         n_plain = min(n_plain, n_tiles);
+        // diagonal aligned with the tiles: query i of the wavefront sees key j of its one masked tile iff j <= i
+        const int aligned = CAUSAL && n_mask == n_plain + 1 && qw0 + coff == n_plain * kWBN && (n_plain + 1) * kWBN <= sk;
         // the assembly loop requests tile+2 with whole-tile loads: it may run tile t only if tile t+2 is a whole tile
         // (or does not exist), so it stops three tiles before a partial last tile
         const int n_asm = n_tiles > sk / kWBN ? max(0, n_tiles - 3) : n_tiles;
 
-        // ---- Q rows -> staging slab (the fragments stay there for the whole query tile: the assembly loop loads them
-        // into its registers when it starts, ordinary code reads them as it needs them; the slab is reused for the
-        // output rows at the end).  Rows past the end of the sequence are zero. ----
-        unsigned char* const slab = o_lds + wave * (64 * kWORow);
-        __syncthreads();                     // the previous query tile's readers are done with the LDS buffers
-        if (n_tiles > 0) issue_tile(0, 0);
-        if (n_tiles > 1) issue_tile(1, 1);
-        {
-            constexpr int kRowsPerPass = 64 / CPR;           // 4 rows per pass, 16 passes
-            const int c16 = lane % CPR, r0 = lane / CPR;
-            u32x4 rows[64 / kRowsPerPass];
+        // query rows: registers -> slab (the previous job has read its output rows back from the slab by now: LDS
+        // operations of a wavefront execute in order)
 #pragma unroll
-            for (int i = 0; i < 64 / kRowsPerPass; ++i) {
-                const int r = i * kRowsPerPass + r0;
-                rows[i] = u32x4{0u, 0u, 0u, 0u};
-                if (qw0 + r < sq) rows[i] = *reinterpret_cast<const u32x4*>(qb + (int64_t)(qw0 + r) * p.qs[2] + c16 * 8);
-            }
-#pragma unroll
-            for (int i = 0; i < 64 / kRowsPerPass; ++i)
-                *reinterpret_cast<u32x4*>(slab + (i * kRowsPerPass + r0) * kWORow + c16 * 16) = rows[i];
-        }
-        const uint32_t q_addr = lds_address(slab + n * kWORow + 8 * kg * 2);
-        auto qfrag = [&](int c, int s) { return as_bf16x8(lds_load_at<u32x4>(q_addr + c * 32 * kWORow + 32 * s)); };
+        for (int i = 0; i < 64 / kRowsPerPass; ++i)
+            *reinterpret_cast<u32x4*>(slab + (i * kRowsPerPass + r0) * kWORow + c16 * 16) = q_rows[i];
 
         // Two attempts at most: the first with the references preset to 0, the second -- only if some row's sum came
         // out suspiciously small -- entirely in ordinary code with references taken from the data.
+        bool have_next = false;
         for (int attempt = 0; attempt < 2; ++attempt) {
         const bool preset = attempt == 0;
         if (!preset) {                        // start over: the buffers are free (everybody passed the vote below)
-            if (n_tiles > 0) issue_tile(0, 0);
-            if (n_tiles > 1) issue_tile(1, 1);
+            if (n_tiles > 0) issue_tile(cur, 0, 0);
+            if (n_tiles > 1) issue_tile(cur, 1, 1);
         }
         asm volatile(W64_ZERO : : : W64_CLOBBER_ACC);               // O^T and the row sums
         // per column block: r_ref exponent reference in the log2 domain (-inf: none yet), nb = -r_ref - kBias
@@ -269,8 +310,10 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         r_ref[0] = r_ref[1] = preset ? 0.f : -INFINITY;
         nb[0] = nb[1] = preset ? -kBias : 0.f;
 
-        // wait for tile 0 (this wavefront's 8 loads of tile 1 may stay in flight), meet the others
-        if (n_tiles > 1) wait_vmcnt<8>(); else wait_vmcnt<0>();
+        // Wait for tile 0 and meet the others.  First attempt: the tiles were requested before the query rows, which
+        // have arrived (they are in the slab), and only the previous job's 16 output stores may be younger.  Second
+        // attempt: this wavefront's 8 loads of tile 1 may stay in flight.
+        if (preset) wait_vmcnt<16>(); else if (n_tiles > 1) wait_vmcnt<8>(); else wait_vmcnt<0>();
         __syncthreads();
 
         // One 32-key half of a tile for one column block, in ordinary code: scores, mask, reference move, weights,
@@ -340,7 +383,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             if (tile + 1 < n_tiles) {
                 wait_vmcnt<0>();
                 __syncthreads();
-                if (tile + 2 < n_tiles) issue_tile(tile + 2, tile & 1);
+                if (tile + 2 < n_tiles) issue_tile(cur, tile + 2, tile & 1);
             }
         };
         auto step_cxx = [&](int tile, int t_first) {
@@ -363,8 +406,8 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 continue;
             }
             // ---- the hand-scheduled loop over tiles [tile, n_loop); leaves early when a weight reaches 2 ----
-            const uint64_t kptr = (uint64_t)(uintptr_t)(kb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.ks[2]);
-            const uint64_t vptr = (uint64_t)(uintptr_t)(vb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.vs[2]);
+            const uint64_t kptr = (uint64_t)(uintptr_t)(cur.kb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.ks[2]);
+            const uint64_t vptr = (uint64_t)(uintptr_t)(cur.vb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.vs[2]);
             // mask thresholds for the first masked tile the loop will meet: a key at index j of that tile is kept by
             // query i of the wavefront iff j <= i + (qw0 + coff - k0) and j < sk - k0 (the lane part 4*kg of a key's
             // index is folded in)
@@ -384,6 +427,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                   [thr0] "+v"(v_thr0), [thr1] "+v"(v_thr1)
                 : [n_tiles] "s"(__builtin_amdgcn_readfirstlane(n_tiles)), [n_end] "s"(__builtin_amdgcn_readfirstlane(n_loop)),
                   [n_plain] "s"(__builtin_amdgcn_readfirstlane(n_plain)), [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)),
+                  [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)),
                   [kstep] "s"(__builtin_amdgcn_readfirstlane(k_step)), [vstep] "s"(__builtin_amdgcn_readfirstlane(v_step)),
                   [ldsdst] "s"(lds_dst), [scale] "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, p.scale_log2))),
                   [klo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)kptr)), [khi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kptr >> 32))),
@@ -398,7 +442,8 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             }
         }
 
-        // ---- row sums; on the first attempt the workgroup votes on doing the query tile again ----
+        // ---- row sums; the workgroup meets (everybody is done with the K/V buffers) and, on the first attempt,
+        // votes on doing the query tile again ----
         float l_row[2];
         const auto read_sums = [&](auto c_c) {
             constexpr int c = decltype(c_c)::value;
@@ -413,9 +458,15 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             // (rows past the end of the sequence count too: their sums are sk * 2^-32, far above the limit)
             const bool small = !(l_row[0] >= kUnderflow) || !(l_row[1] >= kUnderflow);
             if (__syncthreads_or(small ? 1 : 0)) continue;
+        } else {
+            __syncthreads();
         }
 
-        // ---- normalise and store: lane owns query qw0 + 32c + n, d = 32dt + 8(i/4) + 4kg + i%4 ----
+        // the next job's first tiles and query rows are on their way while this one finishes
+        have_next = next_job(nxt);
+        if (have_next) prefetch(nxt);
+
+        // ---- normalise: lane owns query qw0 + 32c + n, d = 32dt + 8(i/4) + 4kg + i%4 ----
         const auto store_block = [&](auto c_c) {
             constexpr int c = decltype(c_c)::value;
             const float inv = 1.0f / l_row[c];     // l == 0 (no key kept) -> NaN row, like the reference softmax
@@ -441,25 +492,33 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         store_block(std::integral_constant<int, 1>{});
         break;
         }   // attempts
-        {
-            constexpr int kRowsPerPass = 64 / CPR;
-            const int c16 = lane % CPR, r0 = lane / CPR;
+        // ---- output rows leave whole, through the slab ----
 #pragma unroll
-            for (int i = 0; i < 64 / kRowsPerPass; ++i) {
-                const int r = i * kRowsPerPass + r0;
-                const u32x4 w = *reinterpret_cast<const u32x4*>(slab + r * kWORow + c16 * 16);
-                if (qw0 + r < sq) *reinterpret_cast<u32x4*>(ob + (int64_t)(qw0 + r) * p.os[2] + c16 * 8) = w;
-            }
+        for (int i = 0; i < 64 / kRowsPerPass; ++i) {
+            const int r = i * kRowsPerPass + r0;
+            const u32x4 w = *reinterpret_cast<const u32x4*>(slab + r * kWORow + c16 * 16);
+            if (qw0 + r < sq) *reinterpret_cast<u32x4*>(cur.ob + (int64_t)(qw0 + r) * p.os[2] + c16 * 8) = w;
         }
+        cur = nxt;
+        have = have_next;
     }
 }
 
 int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
-    dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B)), block(kWWaves * 64);
+    // One resident workgroup per compute unit, each working through its share of the (batch, head, tile pair) ids.
+    int dev = 0, n_cu = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return (int)e;
+    const int n_logical = p.n_pairs * p.Hq * p.B;
+    if (n_logical <= 0) return 0;
+    int grid = n_logical < n_cu ? n_logical : n_cu;
+    if (n_logical % 8 == 0 && grid >= 8) grid -= grid % 8;          // whole number of workgroups per XCD
+    dim3 block(kWWaves * 64);
     if (p.mask_mode == MI355_MASK_CAUSAL)
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), dim3((unsigned)grid), block, 0, stream, p, n_logical);
     else
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), dim3((unsigned)grid), block, 0, stream, p, n_logical);
     return (int)hipGetLastError();
 }
 
