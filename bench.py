@@ -420,7 +420,7 @@ def bench_prefill(cfg, args):
         "ms_per_step": wall_ms,
         "algorithmic_flops": flops,
         "roofline": {
-            "bound": "mfma", "kernel": "prefill_fwd_kernel",
+            "bound": "mfma", "kernel": "prefill_fwd_w64_kernel<causal>" if case.q.shape[-1] == 128 else "prefill_fwd_kernel",
             "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms,
             "traffic": _traffic(f"prefill_cfg{cfg}"),
