@@ -64,42 +64,64 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeCacheParams p) 
     }
 }
 
-// The same work with 16-byte accesses: one thread per (token, head slot, group of 4 pairs).
+// The same work with 16-byte accesses.  A thread owns one group of 4 pairs (8 elements, index c) of a token
+// in kRopeHeads head slots, so the angles of (position, c) are fetched once for all of them: reading
+// the table per head slot would put twice the payload's bytes through the vector memory pipeline and
+// bound the kernel there instead of at HBM.  Consecutive threads own consecutive (head slot, c), so one
+// wavefront instruction still covers 1 KiB of adjacent memory; the thread's head slots are
+// hu, hu + n_hu, hu + 2 n_hu, ... with n_hu = ceil(head slots / kRopeHeads).
 // Requires D % 8 == 0, token strides that are multiples of 8 elements and 16-byte aligned bases.
-__global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParams p) {
+// The grid covers the work once (workgroups in dispatch order walk through memory as one window).
+constexpr int kRopeHeads = 4;
+__global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParams p, int n_hu) {
     const int groups = p.D / 8;
     const int half = p.D / 2;
     const int slots_per_tok = p.Hq + 2 * p.Hkv;
-    const int64_t total = (int64_t)p.T * slots_per_tok * groups;
+    const int64_t total = (int64_t)p.T * n_hu * groups;
     for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
          idx += (int64_t)gridDim.x * blockDim.x) {
         const int c = (int)(idx % groups);
-        const int hs = (int)((idx / groups) % slots_per_tok);
-        const int t = (int)(idx / ((int64_t)groups * slots_per_tok));
+        const int hu = (int)((idx / groups) % n_hu);
+        const int t = (int)(idx / ((int64_t)groups * n_hu));
         int64_t slot = p.slots ? p.slots[t] : -1;
         if (slot >= p.n_slots) slot = -1;
-        const bool is_q = hs < p.Hq;
-        if (!is_q && slot < 0) continue;
-        const bool is_v = hs >= p.Hq + p.Hkv;
-        const int hk = is_v ? hs - p.Hq - p.Hkv : hs - p.Hq;
-        const __bf16* src = is_q ? p.q_in + t * p.q_tok + (int64_t)hs * p.D
-                                 : (is_v ? p.v_in + t * p.v_tok : p.k_in + t * p.k_tok) + (int64_t)hk * p.D;
-        u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 8 * c));
-        if (!is_v) {
-            const int pos = min(max(p.positions[t], 0), p.ctx_len - 1);
-            const f32x4 cs = *reinterpret_cast<const f32x4*>(p.freq + (int64_t)pos * half + 4 * c);
-            const f32x4 sn = *reinterpret_cast<const f32x4*>(p.freq + ((int64_t)p.ctx_len + pos) * half + 4 * c);
+        const int pos = min(max(p.positions[t], 0), p.ctx_len - 1);     // a position outside the table is clamped into it
+        u32x4 raw[kRopeHeads];
+        __bf16* dst[kRopeHeads];
+        bool rotate[kRopeHeads];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t w = raw[j];           // scalar copy first: a bit_cast of a vector element misreads it
-                const bf16x2 x = __builtin_bit_cast(bf16x2, w);
-                const float x1 = (float)x[0], x2 = (float)x[1];
-                raw[j] = pack_bf16(cs[j] * x1 - sn[j] * x2, sn[j] * x1 + cs[j] * x2);
-            }
+        for (int j = 0; j < kRopeHeads; ++j) {
+            const int hs = hu + j * n_hu;
+            const bool is_q = hs < p.Hq;
+            dst[j] = nullptr;
+            rotate[j] = false;
+            if (hs >= slots_per_tok || (!is_q && slot < 0)) continue;
+            const bool is_v = hs >= p.Hq + p.Hkv;
+            const int hk = is_v ? hs - p.Hq - p.Hkv : hs - p.Hq;
+            const __bf16* src = is_q ? p.q_in + t * p.q_tok + (int64_t)hs * p.D
+                                     : (is_v ? p.v_in + t * p.v_tok : p.k_in + t * p.k_tok) + (int64_t)hk * p.D;
+            raw[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 8 * c));
+            rotate[j] = !is_v;
+            dst[j] = (is_q ? p.q_out + t * p.qo_tok + (int64_t)hs * p.D
+                           : (is_v ? p.v_cache : p.k_cache) + (((slot >> 4) * p.Hkv + hk) * 16 + (slot & 15)) * p.D) + 8 * c;
         }
-        __bf16* dst = is_q ? p.q_out + t * p.qo_tok + (int64_t)hs * p.D
-                           : (is_v ? p.v_cache : p.k_cache) + (((slot >> 4) * p.Hkv + hk) * 16 + (slot & 15)) * p.D;
-        *reinterpret_cast<u32x4*>(dst + 8 * c) = raw;
+        const f32x4 cs = *reinterpret_cast<const f32x4*>(p.freq + (int64_t)pos * half + 4 * c);
+        const f32x4 sn = *reinterpret_cast<const f32x4*>(p.freq + ((int64_t)p.ctx_len + pos) * half + 4 * c);
+#pragma unroll
+        for (int j = 0; j < kRopeHeads; ++j) {
+            if (!dst[j]) continue;
+            u32x4 w4 = raw[j];
+            if (rotate[j]) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t w = raw[j][e];           // scalar copy first: a bit_cast of a vector element misreads it
+                    const bf16x2 x = __builtin_bit_cast(bf16x2, w);
+                    const float x1 = (float)x[0], x2 = (float)x[1];
+                    w4[e] = pack_bf16(cs[e] * x1 - sn[e] * x2, sn[e] * x1 + cs[e] * x2);
+                }
+            }
+            __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(dst[j]));
+        }
     }
 }
 
@@ -142,7 +164,7 @@ __global__ __launch_bounds__(256) void quantize_kv_fp8_kernel(const __bf16* __re
             u32x2 out;
             out[0] = (uint32_t)w0;
             out[1] = (uint32_t)w1;
-            *reinterpret_cast<u32x2*>(d + 512 * j) = out;
+            __builtin_nontemporal_store(out, reinterpret_cast<u32x2*>(d + 512 * j));
         }
     }
 }
@@ -343,11 +365,12 @@ extern "C" int mi355_rope_and_cache(const void* q_in, const void* k_in, const vo
     const bool vec8 = D % 8 == 0 && ((q_token_stride | k_token_stride | v_token_stride | q_out_token_stride) & 7) == 0 &&
                       aligned16(q_in) && aligned16(k_in) && aligned16(v_in) && aligned16(q_out) && aligned16(k_cache) &&
                       aligned16(v_cache) && aligned16(freq_cache);
-    const int64_t total = (int64_t)T * (Hq + 2 * Hkv) * (vec8 ? D / 8 : D / 2);
+    const int n_hu = (Hq + 2 * Hkv + kRopeHeads - 1) / kRopeHeads;
+    const int64_t total = vec8 ? (int64_t)T * n_hu * (D / 8) : (int64_t)T * (Hq + 2 * Hkv) * (D / 2);
     const int64_t blocks = (total + 255) / 256;
-    const unsigned grid = (unsigned)(blocks < 256 * 64 ? blocks : 256 * 64);
+    const unsigned grid = (unsigned)(blocks < 0x7fffffffLL ? blocks : 0x7fffffffLL);
     if (vec8)
-        hipLaunchKernelGGL(rope_and_cache_vec8_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(rope_and_cache_vec8_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, p, n_hu);
     else
         hipLaunchKernelGGL(rope_and_cache_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, p);
     const int rc = (int)hipGetLastError();
@@ -364,7 +387,7 @@ extern "C" int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, fl
     const int64_t n_slabs = num_blocks * Hkv;
     if (n_slabs == 0) return MI355_OK;
     const int64_t wgs = (n_slabs + 3) / 4;                  // four wavefronts (slabs) per workgroup
-    const unsigned grid = (unsigned)(wgs < 256 * 64 ? wgs : 256 * 64);
+    const unsigned grid = (unsigned)(wgs < 0x7fffffffLL ? wgs : 0x7fffffffLL);
     hipStream_t s = (hipStream_t)stream;
     if (D == 128)
         hipLaunchKernelGGL(quantize_kv_fp8_kernel<128>, dim3(grid), dim3(256), 0, s, (const __bf16*)cache_bf16,
@@ -421,10 +444,11 @@ extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, cons
     pq.ctx_len = context_length;
     pq.n_slots = 0;
     {
-        const int64_t total = (int64_t)T * Hq * (D / 8);
+        const int n_hu = (Hq + kRopeHeads - 1) / kRopeHeads;
+        const int64_t total = (int64_t)T * n_hu * (D / 8);
         const int64_t blocks = (total + 255) / 256;
-        const unsigned grid = (unsigned)(blocks < 256 * 64 ? blocks : 256 * 64);
-        hipLaunchKernelGGL(rope_and_cache_vec8_kernel, dim3(grid), dim3(256), 0, s, pq);
+        const unsigned grid = (unsigned)(blocks < 0x7fffffffLL ? blocks : 0x7fffffffLL);
+        hipLaunchKernelGGL(rope_and_cache_vec8_kernel, dim3(grid), dim3(256), 0, s, pq, n_hu);
     }
     RopeCacheFp8Params p;
     p.k_in = (const __bf16*)k_in;

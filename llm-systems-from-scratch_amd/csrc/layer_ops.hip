@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
                 for (int e = 0; e < 4; ++e)
                     s[e] = pack_bf16((float)a[2 * e] + (float)b[2 * e], (float)a[2 * e + 1] + (float)b[2 * e + 1]);
                 raw[c] = s;
-                if (p.sum_out) *reinterpret_cast<u32x4*>(p.sum_out + row * p.ss + col) = s;
+                if (p.sum_out) __builtin_nontemporal_store(s, reinterpret_cast<u32x4*>(p.sum_out + row * p.ss + col));
             }
             const bf16x8 v = as_bf16x8(raw[c]);
 #pragma unroll
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 o[e] = pack_bf16(w[2 * e] * ((float)v[2 * e] * rstd), w[2 * e + 1] * ((float)v[2 * e + 1] * rstd));
-            *reinterpret_cast<u32x4*>(yr + col) = o;
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(yr + col));
         }
     }
 }
@@ -144,6 +144,10 @@ __device__ __forceinline__ float silu_mul_one(float g, float u) {
 }
 
 // One thread per 8 adjacent elements of a row.  Requires n_cols % 8 == 0 and 16-byte aligned rows.
+// The grid covers the tensor once (the loop only runs again beyond 2^31 workgroups): workgroups are
+// dispatched in order, so the accesses in flight at any time form one window that moves through the
+// tensor, which DRAM serves faster than the scattered windows of a small persistent grid (measured:
+// 6.4 against 4.9 TB/s for a two-reads-one-write stream of this size).
 __global__ __launch_bounds__(256) void silu_mul_vec8_kernel(SiluMulParams p) {
     const int groups = p.n_cols / 8;
     const int64_t total = p.n_rows * groups;
@@ -158,7 +162,7 @@ __global__ __launch_bounds__(256) void silu_mul_vec8_kernel(SiluMulParams p) {
         for (int e = 0; e < 4; ++e)
             o[e] = pack_bf16(silu_mul_one((float)g[2 * e], (float)u[2 * e]),
                              silu_mul_one((float)g[2 * e + 1], (float)u[2 * e + 1]));
-        *reinterpret_cast<u32x4*>(p.out + row * p.os + col) = o;
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(p.out + row * p.os + col));
     }
 }
 
@@ -241,7 +245,7 @@ extern "C" int mi355_silu_mul_fwd(const void* gate, const void* up, void* out, i
                      ((gate_row_stride | up_row_stride | out_row_stride) & 7) == 0;
     const int64_t total = vec ? n_rows * (n_cols / 8) : n_rows * (int64_t)n_cols;
     const int64_t blocks = (total + 255) / 256;
-    const unsigned grid = (unsigned)(blocks < 256 * 64 ? blocks : 256 * 64);
+    const unsigned grid = (unsigned)(blocks < 0x7fffffffLL ? blocks : 0x7fffffffLL);
     hipStream_t s = (hipStream_t)stream;
     if (vec) hipLaunchKernelGGL(silu_mul_vec8_kernel, dim3(grid), dim3(256), 0, s, p);
     else hipLaunchKernelGGL(silu_mul_generic_kernel, dim3(grid), dim3(256), 0, s, p);
