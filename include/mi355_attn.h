@@ -92,6 +92,27 @@ int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out
                           float softmax_scale, int mask_mode, int dtype, void* stream);
 
 /*
+ * Causal prefill of a CHUNK of new tokens on top of context that is already in a paged bf16 cache
+ * (chunked prefill / prefix reuse).  The keys and values of all context_lens[b] tokens of sequence b
+ * -- the chunk's own included: write them first with mi355_rope_and_cache -- are read through
+ * block_tables (the layout of mi355_paged_decode_fwd: int32 (B, table_stride), entry j = physical
+ * block of tokens [16j, 16j+16); k_cache/v_cache (num_blocks,Hkv,16,D) bf16).  The chunk's queries
+ * are packed: q/out (T,Hq,D) with contiguous heads, sequence b owning rows
+ * [cu_seqlens_q[b], cu_seqlens_q[b+1]); its query i keeps key j iff
+ * j <= i + (context_lens[b] - chunk length), the bottom-right aligned mask of MI355_MASK_CAUSAL.
+ * Only table entries of blocks that hold a valid key are read.  Sq_max = longest chunk.
+ * Same mathematics as mi355_prefill_fwd (model.py:308-325 / :382) -- the reference has no cache,
+ * so it has no counterpart of the table walk; what it replaces is re-running the whole prefix at
+ * model.py:218 when a prompt arrives in pieces.
+ */
+int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
+                            int64_t q_token_stride, int64_t out_token_stride,
+                            const int32_t* cu_seqlens_q, const int32_t* block_tables, int64_t table_stride,
+                            const int32_t* context_lens, int B, int Hq, int Hkv, int Sq_max, int D,
+                            int block_size, int64_t num_blocks, float softmax_scale, int kv_dtype,
+                            void* stream);
+
+/*
  * Prefill backward: dq, dk, dv of out = softmax(q k^T * softmax_scale [causal]) v given dout,
  * i.e. the gradient that autograd derives for the attention call at model.py:380-385
  * (model.py:308-325 is its definition) during loss.backward() (train.py:224).
@@ -188,14 +209,17 @@ int mi355_paged_decode_chunk_tokens(int max_ctx);
  * The scatter has no counterpart in the reference (it has no KV cache).
  *   q_in/q_out (T,Hq,D), k_in/v_in (T,Hkv,D) bf16, heads contiguous, token strides in elements;
  *   positions int32 (T), each < context_length (a position outside the table is clamped into it);
- *   k_cache/v_cache (num_blocks,Hkv,16,D) bf16; a slot outside [0, num_blocks*16) is not written.
+ *   k_cache/v_cache (num_blocks,Hkv,16,D) bf16; a slot outside [0, num_blocks*16) is not written;
+ *   k_out (optional, else NULL): the rotated keys once more, packed (T,Hkv,D) bf16 with token stride
+ *   k_out_token_stride -- the K operand of a prefill over the same tokens (mi355_prefill_fwd), so that
+ *   one launch serves the cache and the prefill; may alias k_in.
  */
 int mi355_rope_and_cache(const void* q_in, const void* k_in, const void* v_in, void* q_out,
                          void* k_cache, void* v_cache, const float* freq_cache,
                          const int32_t* positions, const int64_t* slot_mapping, int64_t num_blocks,
                          int T, int Hq, int Hkv, int D, int context_length,
                          int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
-                         int64_t q_out_token_stride, void* stream);
+                         int64_t q_out_token_stride, void* k_out, int64_t k_out_token_stride, void* stream);
 
 /*
  * Per-(block, kv head) absmax quantisation of a bf16 cache (num_blocks,Hkv,16,D) to OCP
@@ -217,8 +241,10 @@ int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, float* scale,
  * Tokens that share a block must be adjacent in the packed order with consecutive slots (a run),
  * and a block may receive one run per call (one sequence = one run per block, as a prefill or a
  * decode step produces them).  Slots outside [0, 16*num_blocks) are skipped.  Needs 16-byte
- * aligned tensors, token strides that are multiples of 8, D in {32, 64, 128}.  No reference
- * counterpart (the reference has no KV cache).
+ * aligned tensors, token strides that are multiples of 8, D in {32, 64, 128}.  k_out (optional)
+ * receives the rotated keys in bf16, packed (T,Hkv,D), as in mi355_rope_and_cache: a prefill over
+ * the tokens of this call then attends to unquantised keys.  No reference counterpart (the reference
+ * has no KV cache).
  */
 int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, const void* v_in, void* q_out,
                              void* k_cache_fp8, void* v_cache_fp8, float* k_scale, float* v_scale,
@@ -226,7 +252,8 @@ int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, const void* v_i
                              const int64_t* slot_mapping, int64_t num_blocks,
                              int T, int Hq, int Hkv, int D, int context_length,
                              int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
-                             int64_t q_out_token_stride, void* stream);
+                             int64_t q_out_token_stride, void* k_out, int64_t k_out_token_stride,
+                             void* stream);
 
 /*
  * RMSNorm forward over the rows of a (n_rows, n_cols) bf16 matrix:

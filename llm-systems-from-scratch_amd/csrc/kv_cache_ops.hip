@@ -16,8 +16,10 @@ struct RopeCacheParams {
     const float* freq;            // (2, context_length, D/2): cos plane then sin plane
     const int32_t* positions;     // (T)
     const int64_t* slots;         // (T): block * 16 + offset, negative = do not write the cache
-    int64_t q_tok, k_tok, v_tok, qo_tok;   // token strides (elements); heads are contiguous (stride D)
+    __bf16* k_out;                // optional: rotated keys, packed (T, Hkv, D), for a prefill over the same tokens
+    int64_t q_tok, k_tok, v_tok, qo_tok, ko_tok;   // token strides (elements); heads are contiguous (stride D)
     int T, Hq, Hkv, D, ctx_len;
+    int head_slots;                // head slots served per token: Hq query heads, then Hkv key heads, then Hkv value heads
     int64_t n_slots;               // num_blocks * 16: slots outside [0, n_slots) are not written
 };
 
@@ -26,7 +28,7 @@ struct RopeCacheParams {
 // of (position, i), in fp32, rounded once to bf16.
 __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeCacheParams p) {
     const int half = p.D / 2;
-    const int slots_per_tok = p.Hq + 2 * p.Hkv;
+    const int slots_per_tok = p.head_slots;
     const int64_t total = (int64_t)p.T * slots_per_tok * half;
     for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
          idx += (int64_t)gridDim.x * blockDim.x) {
@@ -45,15 +47,17 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeCacheParams p) 
             *reinterpret_cast<uint32_t*>(p.q_out + t * p.qo_tok + (int64_t)hs * p.D + 2 * i) =
                 pack_bf16(c * x1 - s * x2, s * x1 + c * x2);
         } else if (hs < p.Hq + p.Hkv) {
-            if (slot < 0) continue;
+            if (slot < 0 && !p.k_out) continue;
             const int hk = hs - p.Hq;
             const uint32_t raw = *reinterpret_cast<const uint32_t*>(p.k_in + t * p.k_tok + (int64_t)hk * p.D + 2 * i);
             const bf16x2 x = __builtin_bit_cast(bf16x2, raw);
             const float c = p.freq[(int64_t)pos * half + i];
             const float s = p.freq[((int64_t)p.ctx_len + pos) * half + i];
             const float x1 = (float)x[0], x2 = (float)x[1];
-            const int64_t dst = (((slot >> 4) * p.Hkv + hk) * 16 + (slot & 15)) * p.D + 2 * i;
-            *reinterpret_cast<uint32_t*>(p.k_cache + dst) = pack_bf16(c * x1 - s * x2, s * x1 + c * x2);
+            const uint32_t rot = pack_bf16(c * x1 - s * x2, s * x1 + c * x2);
+            if (slot >= 0)
+                *reinterpret_cast<uint32_t*>(p.k_cache + (((slot >> 4) * p.Hkv + hk) * 16 + (slot & 15)) * p.D + 2 * i) = rot;
+            if (p.k_out) *reinterpret_cast<uint32_t*>(p.k_out + t * p.ko_tok + (int64_t)hk * p.D + 2 * i) = rot;
         } else {
             if (slot < 0) continue;
             const int hk = hs - p.Hq - p.Hkv;
@@ -76,7 +80,7 @@ constexpr int kRopeHeads = 4;
 __global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParams p, int n_hu) {
     const int groups = p.D / 8;
     const int half = p.D / 2;
-    const int slots_per_tok = p.Hq + 2 * p.Hkv;
+    const int slots_per_tok = p.head_slots;
     const int64_t total = (int64_t)p.T * n_hu * groups;
     for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
          idx += (int64_t)gridDim.x * blockDim.x) {
@@ -87,29 +91,30 @@ __global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParam
         if (slot >= p.n_slots) slot = -1;
         const int pos = min(max(p.positions[t], 0), p.ctx_len - 1);     // a position outside the table is clamped into it
         u32x4 raw[kRopeHeads];
-        __bf16* dst[kRopeHeads];
+        __bf16 *dst[kRopeHeads], *dst2[kRopeHeads];        // dst2: a key's second home, the packed k_out
         bool rotate[kRopeHeads];
 #pragma unroll
         for (int j = 0; j < kRopeHeads; ++j) {
             const int hs = hu + j * n_hu;
             const bool is_q = hs < p.Hq;
-            dst[j] = nullptr;
+            dst[j] = dst2[j] = nullptr;
             rotate[j] = false;
-            if (hs >= slots_per_tok || (!is_q && slot < 0)) continue;
             const bool is_v = hs >= p.Hq + p.Hkv;
+            if (hs >= slots_per_tok || (!is_q && slot < 0 && (is_v || !p.k_out))) continue;
             const int hk = is_v ? hs - p.Hq - p.Hkv : hs - p.Hq;
             const __bf16* src = is_q ? p.q_in + t * p.q_tok + (int64_t)hs * p.D
                                      : (is_v ? p.v_in + t * p.v_tok : p.k_in + t * p.k_tok) + (int64_t)hk * p.D;
             raw[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 8 * c));
             rotate[j] = !is_v;
-            dst[j] = (is_q ? p.q_out + t * p.qo_tok + (int64_t)hs * p.D
-                           : (is_v ? p.v_cache : p.k_cache) + (((slot >> 4) * p.Hkv + hk) * 16 + (slot & 15)) * p.D) + 8 * c;
+            if (is_q) dst[j] = p.q_out + t * p.qo_tok + (int64_t)hs * p.D + 8 * c;
+            else if (slot >= 0) dst[j] = (is_v ? p.v_cache : p.k_cache) + (((slot >> 4) * p.Hkv + hk) * 16 + (slot & 15)) * p.D + 8 * c;
+            if (!is_q && !is_v && p.k_out) dst2[j] = p.k_out + t * p.ko_tok + (int64_t)hk * p.D + 8 * c;
         }
         const f32x4 cs = *reinterpret_cast<const f32x4*>(p.freq + (int64_t)pos * half + 4 * c);
         const f32x4 sn = *reinterpret_cast<const f32x4*>(p.freq + ((int64_t)p.ctx_len + pos) * half + 4 * c);
 #pragma unroll
         for (int j = 0; j < kRopeHeads; ++j) {
-            if (!dst[j]) continue;
+            if (!dst[j] && !dst2[j]) continue;
             u32x4 w4 = raw[j];
             if (rotate[j]) {
 #pragma unroll
@@ -120,7 +125,8 @@ __global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParam
                     w4[e] = pack_bf16(cs[e] * x1 - sn[e] * x2, sn[e] * x1 + cs[e] * x2);
                 }
             }
-            __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(dst[j]));
+            if (dst[j]) __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(dst[j]));
+            if (dst2[j]) __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(dst2[j]));
         }
     }
 }
@@ -329,9 +335,11 @@ extern "C" int mi355_rope_and_cache(const void* q_in, const void* k_in, const vo
                                     const int64_t* slot_mapping, int64_t num_blocks, int T, int Hq, int Hkv, int D,
                                     int context_length,
                                     int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
-                                    int64_t q_out_token_stride, void* stream) {
+                                    int64_t q_out_token_stride, void* k_out, int64_t k_out_token_stride, void* stream) {
     if (!q_in || !k_in || !v_in || !q_out || !freq_cache || !positions)
         return set_error(MI355_EINVAL, "rope_and_cache: null pointer argument");
+    if (k_out && (k_out_token_stride & 1))
+        return set_error(MI355_EINVAL, "rope_and_cache: token strides must be even (4-byte aligned pairs)");
     if (slot_mapping && (!k_cache || !v_cache))
         return set_error(MI355_EINVAL, "rope_and_cache: slot_mapping given without k_cache/v_cache");
     if (slot_mapping && num_blocks <= 0) return set_error(MI355_EINVAL, "rope_and_cache: num_blocks must be positive");
@@ -355,18 +363,21 @@ extern "C" int mi355_rope_and_cache(const void* q_in, const void* k_in, const vo
     p.k_tok = k_token_stride;
     p.v_tok = v_token_stride;
     p.qo_tok = q_out_token_stride;
+    p.k_out = (__bf16*)k_out;
+    p.ko_tok = k_out ? k_out_token_stride : 0;
     p.T = T;
     p.Hq = Hq;
     p.Hkv = Hkv;
     p.D = D;
     p.ctx_len = context_length;
+    p.head_slots = slot_mapping ? Hq + 2 * Hkv : (k_out ? Hq + Hkv : Hq);     // nothing to do for values without a cache
     p.n_slots = slot_mapping ? num_blocks * 16 : 0;
     const auto aligned16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
     const bool vec8 = D % 8 == 0 && ((q_token_stride | k_token_stride | v_token_stride | q_out_token_stride) & 7) == 0 &&
                       aligned16(q_in) && aligned16(k_in) && aligned16(v_in) && aligned16(q_out) && aligned16(k_cache) &&
-                      aligned16(v_cache) && aligned16(freq_cache);
-    const int n_hu = (Hq + 2 * Hkv + kRopeHeads - 1) / kRopeHeads;
-    const int64_t total = vec8 ? (int64_t)T * n_hu * (D / 8) : (int64_t)T * (Hq + 2 * Hkv) * (D / 2);
+                      aligned16(v_cache) && aligned16(freq_cache) && aligned16(k_out) && (p.ko_tok & 7) == 0;
+    const int n_hu = (p.head_slots + kRopeHeads - 1) / kRopeHeads;
+    const int64_t total = vec8 ? (int64_t)T * n_hu * (D / 8) : (int64_t)T * p.head_slots * (D / 2);
     const int64_t blocks = (total + 255) / 256;
     const unsigned grid = (unsigned)(blocks < 0x7fffffffLL ? blocks : 0x7fffffffLL);
     if (vec8)
@@ -409,7 +420,8 @@ extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, cons
                                         const float* freq_cache, const int32_t* positions, const int64_t* slot_mapping,
                                         int64_t num_blocks, int T, int Hq, int Hkv, int D, int context_length,
                                         int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
-                                        int64_t q_out_token_stride, void* stream) {
+                                        int64_t q_out_token_stride, void* k_out, int64_t k_out_token_stride,
+                                        void* stream) {
     if (!q_in || !k_in || !v_in || !q_out || !freq_cache || !positions || !slot_mapping || !k_cache_fp8 || !v_cache_fp8 ||
         !k_scale || !v_scale)
         return set_error(MI355_EINVAL, "rope_and_cache_fp8: null pointer argument");
@@ -420,11 +432,11 @@ extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, cons
     const auto aligned16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
     if (((q_token_stride | k_token_stride | v_token_stride | q_out_token_stride) & 7) != 0 || !aligned16(q_in) ||
         !aligned16(k_in) || !aligned16(v_in) || !aligned16(q_out) || !aligned16(k_cache_fp8) || !aligned16(v_cache_fp8) ||
-        !aligned16(freq_cache))
+        !aligned16(freq_cache) || !aligned16(k_out) || (k_out && (k_out_token_stride & 7) != 0))
         return set_error(MI355_EINVAL, "rope_and_cache_fp8: tensors must be 16-byte aligned with token strides that are multiples of 8");
     if (T == 0) return MI355_OK;
     hipStream_t s = (hipStream_t)stream;
-    // queries: the bf16 kernel with no key/value heads rotates q_in into q_out and touches nothing else
+    // queries (and, when asked for, the packed rotated keys): the bf16 kernel without a cache
     RopeCacheParams pq{};
     pq.q_in = (const __bf16*)q_in;
     pq.k_in = (const __bf16*)k_in;
@@ -437,14 +449,17 @@ extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, cons
     pq.k_tok = k_token_stride;
     pq.v_tok = v_token_stride;
     pq.qo_tok = q_out_token_stride;
+    pq.k_out = (__bf16*)k_out;
+    pq.ko_tok = k_out ? k_out_token_stride : 0;
     pq.T = T;
     pq.Hq = Hq;
-    pq.Hkv = 0;
+    pq.Hkv = Hkv;
     pq.D = D;
     pq.ctx_len = context_length;
+    pq.head_slots = k_out ? Hq + Hkv : Hq;
     pq.n_slots = 0;
     {
-        const int n_hu = (Hq + kRopeHeads - 1) / kRopeHeads;
+        const int n_hu = (pq.head_slots + kRopeHeads - 1) / kRopeHeads;
         const int64_t total = (int64_t)T * n_hu * (D / 8);
         const int64_t blocks = (total + 255) / 256;
         const unsigned grid = (unsigned)(blocks < 0x7fffffffLL ? blocks : 0x7fffffffLL);

@@ -36,7 +36,10 @@ constexpr int kBM = 256;   // queries per workgroup
 constexpr int kBN = 64;    // keys per LDS tile
 
 
-template <int D, int MODE>
+// PAGED: keys and values are read from a paged cache through a block table (16 rows per block, so
+// every direct-to-LDS instruction -- 4, 8 or 16 whole rows -- stays inside one block and needs one
+// table entry, a scalar load); queries and outputs are packed.
+template <int D, int MODE, bool PAGED = false>
 __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillParams p) {
     constexpr int NS = D / 16;                    // MFMA k-steps of K.Q^T
     constexpr int NDT = D / 32;                   // 32-row tiles of O^T
@@ -71,7 +74,15 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     const __bf16 *qb, *kb, *vb;
     __bf16* ob;
     float* lb;
-    if (p.cu_q) {
+    if constexpr (PAGED) {
+        const int q_start = p.cu_q[b];
+        sq = p.cu_q[b + 1] - q_start;
+        sk = p.ctx_lens[b];
+        qb = p.q + (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
+        kb = vb = nullptr;
+        ob = p.out + (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
+        lb = nullptr;
+    } else if (p.cu_q) {
         const int q_start = p.cu_q[b], k_start = p.cu_k[b];
         sq = p.cu_q[b + 1] - q_start;
         sk = p.cu_k[b + 1] - k_start;
@@ -120,6 +131,32 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     const bool ld_active = wave * NI < NT;
     auto issue_tile = [&](int tile, int buf) {
         if (!ld_active) return;
+        if constexpr (PAGED) {
+            const uint32_t kdst = __builtin_amdgcn_readfirstlane(lds_address(k_lds + buf * kTile + wave * NI * 1024));
+            const uint32_t vdst = __builtin_amdgcn_readfirstlane(lds_address(v_lds + buf * kTile + wave * NI * 1024));
+            const int last = sk - 1, last_b = last >> 4;            // last valid key and its logical block
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                // the instruction's rows (64 / CPR of them, aligned) lie in logical block bidx of the sequence;
+                // rows past the last key re-read the last key's row (finite; their scores are masked), and a
+                // block past the last one is never looked up (its table entry need not exist)
+                int bidx = tile * (kBN / 16) + (((wave * NI + j) * (64 / CPR)) >> 4);
+                int rin = ld_row[j] & 15;
+                if (bidx > last_b) {
+                    bidx = last_b;
+                    rin = last & 15;
+                } else if (bidx == last_b) {
+                    rin = min(rin, last & 15);
+                }
+                int phys = p.block_table[(int64_t)b * p.table_stride + bidx];
+                phys = min(max(phys, 0), p.num_blocks - 1);           // a corrupt table cannot leave the pool
+                const int64_t base = ((int64_t)phys * p.Hkv + hk) * (16 * D);
+                const uint32_t voff = (uint32_t)(rin * kRow + ld_col[j]);
+                dma_to_lds_16(reinterpret_cast<const unsigned char*>(p.k + base), voff, kdst + j * 1024);
+                dma_to_lds_16(reinterpret_cast<const unsigned char*>(p.v + base), voff, vdst + j * 1024);
+            }
+            return;
+        }
         const unsigned char* kbase = reinterpret_cast<const unsigned char*>(kb + (int64_t)tile * kBN * p.ks[2]);
         const unsigned char* vbase = reinterpret_cast<const unsigned char*>(vb + (int64_t)tile * kBN * p.vs[2]);
         const uint32_t kdst = __builtin_amdgcn_readfirstlane(lds_address(k_lds + buf * kTile + wave * NI * 1024));
@@ -396,6 +433,13 @@ static int launch_prefill(const PrefillParams& p, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+template <int D>
+static int launch_prefill_paged(const PrefillParams& p, hipStream_t stream) {
+    dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B));
+    hipLaunchKernelGGL((prefill_fwd_kernel<D, MI355_MASK_CAUSAL, true>), grid, dim3(kPfWaves * 64), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -455,12 +499,16 @@ static int prefill_common(const void* q, const void* k, const void* v, void* out
     p.mask_mode = mask_mode;
     p.n_qtiles = (Sq_max + kBM - 1) / kBM;
     p.n_pairs = (p.n_qtiles + 1) / 2;
+    p.block_table = nullptr;
+    p.ctx_lens = nullptr;
+    p.table_stride = 0;
+    p.num_blocks = 0;
     if ((int64_t)p.n_pairs * Hq * B > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill: too many workgroups");
 
     hipStream_t s = (hipStream_t)stream;
     int rc;
-    // head_dim 128 without any mask and without lse: the kernel with 64 queries per wavefront and a hand-scheduled
-    // tile loop (measured faster there; with a causal mask its per-query-tile overheads outweigh its faster loop)
+    // head_dim 128 without an explicit mask and without lse: the kernel with 64 queries per wavefront and a
+    // hand-scheduled tile loop
     if (D == 128 && mask_mode != MI355_MASK_BOOL && !lse) rc = launch_prefill_w64(p, s);
     else rc = D == 128 ? launch_prefill<128>(p, s) : (D == 64 ? launch_prefill<64>(p, s) : launch_prefill<32>(p, s));
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
@@ -491,4 +539,54 @@ extern "C" int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v
     return prefill_common(q, k, v, out, q_strides, k_strides, v_strides, o_strides, cu_seqlens_q, cu_seqlens_k, nullptr,
                           nullptr, B, Hq, Hkv, Sq_max, Sk_max, D, softmax_scale, mask_mode, dtype, lse, lse_strides,
                           stream);
+}
+
+extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       int64_t q_token_stride, int64_t out_token_stride, const int32_t* cu_seqlens_q,
+                                       const int32_t* block_tables, int64_t table_stride, const int32_t* context_lens,
+                                       int B, int Hq, int Hkv, int Sq_max, int D, int block_size, int64_t num_blocks,
+                                       float softmax_scale, int kv_dtype, void* stream) {
+    if (!q || !k_cache || !v_cache || !out || !cu_seqlens_q || !block_tables || !context_lens)
+        return set_error(MI355_EINVAL, "prefill_paged: null pointer argument");
+    if (kv_dtype != MI355_BF16) return set_error(MI355_EDTYPE, "prefill_paged: the cache must be MI355_BF16");
+    if (block_size != 16) return set_error(MI355_EINVAL, "prefill_paged: block_size must be 16");
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Sq_max <= 0) return set_error(MI355_EINVAL, "prefill_paged: B, Hq, Hkv and Sq_max must be positive");
+    if (Hq % Hkv != 0) return set_error(MI355_EINVAL, "prefill_paged: Hq must be a multiple of Hkv");
+    if (!(D == 128 || D == 64 || D == 32)) return set_error(MI355_EINVAL, "prefill_paged: head_dim must be 32, 64 or 128");
+    if (num_blocks <= 0 || num_blocks > 0x7fffffffLL || table_stride <= 0)
+        return set_error(MI355_EINVAL, "prefill_paged: num_blocks and table_stride must be positive");
+    if ((q_token_stride | out_token_stride) & 7)
+        return set_error(MI355_EINVAL, "prefill_paged: token strides must be multiples of 8 elements (16-byte rows)");
+    if (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15)
+        return set_error(MI355_EINVAL, "prefill_paged: q, caches and out must be 16-byte aligned");
+    PrefillParams p{};
+    p.q = (const __bf16*)q;
+    p.k = (const __bf16*)k_cache;
+    p.v = (const __bf16*)v_cache;
+    p.out = (__bf16*)out;
+    p.qs[1] = D;
+    p.qs[2] = q_token_stride;
+    p.os[1] = D;
+    p.os[2] = out_token_stride;
+    p.ks[1] = p.vs[1] = 16 * D;
+    p.ks[2] = p.vs[2] = D;
+    p.cu_q = cu_seqlens_q;
+    p.B = B;
+    p.Hq = Hq;
+    p.Hkv = Hkv;
+    p.Sq = Sq_max;
+    p.Sk = 0;
+    p.scale_log2 = softmax_scale * kLog2e;
+    p.mask_mode = MI355_MASK_CAUSAL;
+    p.n_qtiles = (Sq_max + kBM - 1) / kBM;
+    p.n_pairs = (p.n_qtiles + 1) / 2;
+    p.block_table = block_tables;
+    p.ctx_lens = context_lens;
+    p.table_stride = table_stride;
+    p.num_blocks = (int)num_blocks;
+    if ((int64_t)p.n_pairs * Hq * B > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill_paged: too many workgroups");
+    hipStream_t s = (hipStream_t)stream;
+    const int rc = D == 128 ? launch_prefill_paged<128>(p, s) : (D == 64 ? launch_prefill_paged<64>(p, s) : launch_prefill_paged<32>(p, s));
+    if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
+    return MI355_OK;
 }

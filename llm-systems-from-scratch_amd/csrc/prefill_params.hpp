@@ -22,6 +22,12 @@ struct PrefillParams {
     int mask_mode;
     int n_qtiles;
     int n_pairs;
+    // paged keys and values (prefill of a chunk on top of cached context): k, v are cache pools
+    // (num_blocks, Hkv, 16, D); sequence b owns blocks block_table[b * table_stride + j] and ctx_lens[b] keys
+    const int32_t* block_table;
+    const int32_t* ctx_lens;
+    int64_t table_stride;
+    int num_blocks;
 };
 
 // The 64-queries-per-wavefront kernel (head_dim 128, no mask or causal, no lse): prefill_fwd_w64.hip.

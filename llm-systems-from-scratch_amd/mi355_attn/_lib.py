@@ -25,6 +25,7 @@ EXPORTS = (
     "mi355_paged_decode_fwd_static",
     "mi355_paged_decode_workspace_bytes",
     "mi355_paged_decode_chunk_tokens",
+    "mi355_prefill_paged_fwd",
     "mi355_rope_and_cache",
     "mi355_rope_and_cache_fp8",
     "mi355_quantize_kv_fp8",
@@ -60,6 +61,9 @@ def load():
     lib.mi355_prefill_bwd.restype = i32
     lib.mi355_prefill_bwd.argtypes = [vp] * 10 + [_i64x3] * 8 + [_i64x2, vp, vp,
                                                                  i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
+    lib.mi355_prefill_paged_fwd.restype = i32
+    lib.mi355_prefill_paged_fwd.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, i64, vp,
+                                            i32, i32, i32, i32, i32, i32, i64, f32, i32, vp]
     lib.mi355_paged_decode_fwd.restype = i32
     lib.mi355_paged_decode_fwd.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, sz,
                                            i32, i32, i32, i32, i32, i64, i32, f32, i32, vp]
@@ -72,9 +76,9 @@ def load():
     lib.mi355_paged_decode_chunk_tokens.argtypes = [i32]
     lib.mi355_rope_and_cache.restype = i32
     lib.mi355_rope_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32,
-                                         i64, i64, i64, i64, vp]
+                                         i64, i64, i64, i64, vp, i64, vp]
     lib.mi355_rope_and_cache_fp8.restype = i32
-    lib.mi355_rope_and_cache_fp8.argtypes = [vp] * 11 + [i64, i32, i32, i32, i32, i32, i64, i64, i64, i64, vp]
+    lib.mi355_rope_and_cache_fp8.argtypes = [vp] * 11 + [i64, i32, i32, i32, i32, i32, i64, i64, i64, i64, vp, i64, vp]
     lib.mi355_quantize_kv_fp8.restype = i32
     lib.mi355_quantize_kv_fp8.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp]
     lib.mi355_rms_norm_fwd.restype = i32

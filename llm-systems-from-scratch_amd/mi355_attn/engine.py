@@ -11,7 +11,7 @@ of a model; every layer has its own K/V pools.  A step is planned once (`plan_pr
 the caller.
 
 All tensor work runs on the HIP kernels (rope_and_cache, flash_attn_varlen_prefill,
-paged_attention_decode); the bookkeeping here is plain Python on host integers.
+flash_attn_paged_prefill, paged_attention_decode); the bookkeeping here is plain Python on host integers.
 """
 from __future__ import annotations
 
@@ -55,6 +55,10 @@ class PrefillPlan:
     cu_seqlens: torch.Tensor     # (B+1,) int32
     max_len: int
     last_rows: torch.Tensor      # (B,) int64: packed row of each sequence's last token
+    # set when some sequence already had tokens in the cache (a further chunk of its prompt): the attention
+    # then reads all keys and values through the block tables
+    tables: torch.Tensor | None = None        # (B, max_blocks) int32
+    context_lens: torch.Tensor | None = None  # (B,) int32: tokens in the cache, this chunk included
 
 
 @dataclass
@@ -171,27 +175,43 @@ class PagedAttentionEngine:
 
     # ---- planning (once per step) ---------------------------------------------
     def plan_prefill(self, seq_ids, lens) -> PrefillPlan:
-        """Reserves cache slots for the prompts of `seq_ids` (new, empty sequences) with `lens` tokens each."""
+        """Reserves cache slots for the next `lens[i]` prompt tokens of each sequence in `seq_ids`.  A sequence
+        may be new (the usual case) or already hold tokens -- a further chunk of a long prompt, or a prompt on
+        top of a cached prefix: the chunk's queries then attend to everything cached so far (bf16 cache only)."""
         if len(seq_ids) != len(lens) or not seq_ids:
             raise ValueError("seq_ids and lens must be non-empty and of equal length")
+        if len(set(seq_ids)) != len(seq_ids):
+            raise ValueError("a sequence may appear only once per prefill")
         for sid, n in zip(seq_ids, lens):
-            if n < 1 or n > self.context_length:
-                raise ValueError(f"prompt lengths must be in 1..{self.context_length}")
-            if self.lengths[sid] != 0:
-                raise ValueError(f"sequence {sid} already has tokens; chunked prefill is not supported")
-        need = sum((n + BLOCK - 1) // BLOCK for n in lens)
+            if n < 1 or self.lengths[sid] + n > self.context_length:
+                raise ValueError(f"prompt lengths must be in 1..{self.context_length} (tokens already cached included)")
+        chunked = any(self.lengths[sid] != 0 for sid in seq_ids)
+        if chunked and self.kv_dtype != "bf16":
+            raise NotImplementedError("a further chunk of a prompt needs a bf16 cache: the chunk would attend to "
+                                      "quantised keys and values of its own prefix")
+        need = sum((self.lengths[sid] + n + BLOCK - 1) // BLOCK - len(self.blocks[sid]) for sid, n in zip(seq_ids, lens))
         if need > self.allocator.num_free:
             raise OutOfBlocks(f"prefill needs {need} blocks, {self.allocator.num_free} free")
         slots, positions, cu = [], [], [0]
         for sid, n in zip(seq_ids, lens):
+            start = self.lengths[sid]
             slots += self._reserve(sid, n)
-            positions += list(range(n))
+            positions += list(range(start, start + n))
             cu.append(cu[-1] + n)
         dev = self.device
-        return PrefillPlan(torch.tensor(positions, dtype=torch.int32, device=dev),
+        plan = PrefillPlan(torch.tensor(positions, dtype=torch.int32, device=dev),
                            torch.tensor(slots, dtype=torch.int64, device=dev),
                            torch.tensor(cu, dtype=torch.int32, device=dev), max(lens),
                            torch.tensor([c - 1 for c in cu[1:]], dtype=torch.int64, device=dev))
+        if chunked:
+            max_blk = max(len(self.blocks[sid]) for sid in seq_ids)
+            rows = torch.zeros(len(seq_ids), max_blk, dtype=torch.int32)
+            for i, sid in enumerate(seq_ids):
+                b = self.blocks[sid]
+                rows[i, :len(b)] = torch.tensor(b, dtype=torch.int32)
+            plan.tables = rows.to(dev)
+            plan.context_lens = torch.tensor([self.lengths[sid] for sid in seq_ids], dtype=torch.int32, device=dev)
+        return plan
 
     def _reserve_decode(self, seq_ids):
         """Host side of a decode step: checks, reserves one slot per sequence.  Returns (positions, slots)."""
@@ -249,22 +269,28 @@ class PagedAttentionEngine:
         return static.plan
 
     # ---- attention calls (once per layer) -----------------------------------------
-    def _write_cache(self, layer: int, plan, q, k, v):
+    def _write_cache(self, layer: int, plan, q, k, v, k_out=None):
         """RoPE on q and k, rotated k and v into layer `layer`'s cache (quantised when the cache is fp8);
-        returns the rotated q."""
+        returns the rotated q -- with k_out=True the pair (rotated q, rotated k in packed form)."""
         kc, vc = self.k_caches[layer], self.v_caches[layer]
         if self.kv_dtype == "bf16":
-            return ops.rope_and_cache(q, k, v, plan.positions, self.freq_cache, kc, vc, plan.slots)
+            return ops.rope_and_cache(q, k, v, plan.positions, self.freq_cache, kc, vc, plan.slots, k_out=k_out)
         return ops.rope_and_cache_fp8(q, k, v, plan.positions, self.freq_cache, kc, vc, self.k_scales[layer],
-                                      self.v_scales[layer], plan.slots)
+                                      self.v_scales[layer], plan.slots, k_out=k_out)
 
     def attend_prefill(self, layer: int, plan: PrefillPlan, q, k, v):
         """q (T,Hq,D), k/v (T,Hkv,D) packed along dim 0 (token strides free, heads contiguous).  Writes
-        rotated K and V of layer `layer` into its cache and returns causal attention output (T,Hq,D)."""
+        rotated K and V of layer `layer` into its cache and returns causal attention output (T,Hq,D).
+        New sequences attend to the packed tensors themselves (one launch rotates q and k and fills the
+        cache); when a sequence already had cached tokens, keys and values are read back through the
+        block tables, old and new alike."""
         if q.shape[0] != plan.positions.shape[0]:
             raise ValueError("the plan and the packed tensors disagree on the number of tokens")
-        q_rot = self._write_cache(layer, plan, q, k, v)
-        k_rot = ops.rope_and_cache(k, k, v, plan.positions, self.freq_cache)   # rotated keys, packed, for the prefill kernel
+        if plan.tables is not None:
+            q_rot = self._write_cache(layer, plan, q, k, v)
+            return ops.flash_attn_paged_prefill(q_rot, self.k_caches[layer], self.v_caches[layer], plan.cu_seqlens,
+                                                plan.tables, plan.context_lens, plan.max_len)
+        q_rot, k_rot = self._write_cache(layer, plan, q, k, v, k_out=True)
         return ops.flash_attn_varlen_prefill(q_rot, k_rot, v, plan.cu_seqlens, plan.cu_seqlens, plan.max_len,
                                              plan.max_len, causal=True)
 

@@ -419,6 +419,66 @@ def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, s
     return out
 
 
+def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, context_lens, max_seqlen_q, *,
+                             softmax_scale=None, out=None):
+    """Causal prefill of a chunk of new tokens over context that already sits in a paged bf16 cache.
+
+    q (T,Hq,D) bf16, packed, contiguous heads (token stride free): sequence b owns rows
+    [cu_seqlens_q[b], cu_seqlens_q[b+1]).  k_cache, v_cache (num_blocks,Hkv,16,D) bf16 hold ALL
+    context_lens[b] tokens of sequence b -- the chunk's own too (write them first with rope_and_cache) --
+    addressed through block_tables (B,max_blocks) int32.  Query i of the chunk keeps key j iff
+    j <= i + (context_lens[b] - chunk length).  max_seqlen_q = longest chunk.  Returns (T,Hq,D) bf16.
+    The mathematics is that of llm-core/llm_core/model.py:308-325 with the mask of :384; the reference
+    itself would re-run the whole prefix (model.py:218)."""
+    _require_gpu_bf16("q", q)
+    if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
+        raise ValueError("q must be (tokens, heads, d_head) with contiguous heads")
+    T, Hq, D = q.shape
+    for n, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+        if c.dtype != torch.bfloat16:
+            raise TypeError(f"{n} must be bfloat16 (got {c.dtype}); chunked prefill reads a bf16 cache")
+        if c.dim() != 4 or c.shape[2] != _BLOCK or c.shape[3] != D or not c.is_contiguous() or not c.is_cuda:
+            raise ValueError(f"{n} must be a contiguous GPU tensor (num_blocks, kv_heads, {_BLOCK}, {D})")
+    if k_cache.shape != v_cache.shape:
+        raise ValueError("k_cache and v_cache must have the same shape")
+    Hkv = k_cache.shape[1]
+    if D not in (32, 64, 128):
+        raise ValueError("d_head must be 32, 64 or 128")
+    if Hq % Hkv != 0:
+        raise ValueError("the number of query heads must be a multiple of the number of kv heads")
+    for n, t in (("cu_seqlens_q", cu_seqlens_q), ("block_tables", block_tables), ("context_lens", context_lens)):
+        if t.dtype != torch.int32:
+            raise TypeError(f"{n} must be int32")
+    B = cu_seqlens_q.numel() - 1
+    if cu_seqlens_q.dim() != 1 or B < 0 or not cu_seqlens_q.is_contiguous():
+        raise ValueError("cu_seqlens_q must be a contiguous (batch + 1,) tensor")
+    if block_tables.dim() != 2 or block_tables.shape[0] != B or block_tables.stride(1) != 1:
+        raise ValueError("block_tables must be (batch, max_blocks) with unit column stride")
+    if context_lens.shape != (B,) or not context_lens.is_contiguous():
+        raise ValueError("context_lens must be a contiguous (batch,) tensor")
+    if int(max_seqlen_q) < 1 and T > 0:
+        raise ValueError("max_seqlen_q must be at least 1")
+    if q.stride(0) % 8 != 0 or q.data_ptr() % 16 != 0:
+        raise ValueError("q must be 16-byte aligned with a token stride that is a multiple of 8 elements")
+    if out is None:
+        out = torch.empty(T, Hq, D, dtype=q.dtype, device=q.device)
+    else:
+        _require_gpu_bf16("out", out)
+        if out.shape != q.shape or out.stride(2) != 1 or out.stride(1) != D or out.stride(0) % 8 != 0 \
+                or out.data_ptr() % 16 != 0:
+            raise ValueError("out must have q's shape with contiguous heads, 16-byte aligned")
+    if T == 0 or B == 0:
+        return out
+    scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
+    with _on(q, k_cache, v_cache, out, cu_seqlens_q, block_tables, context_lens) as stream:
+        rc = _lib.load().mi355_prefill_paged_fwd(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), q.stride(0), out.stride(0),
+            cu_seqlens_q.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
+            B, Hq, Hkv, int(max_seqlen_q), D, _BLOCK, k_cache.shape[0], float(scale), _lib.MI355_BF16, stream)
+    _lib.check(rc, "mi355_prefill_paged_fwd")
+    return out
+
+
 def build_rope_cache(context_length, d, theta=10000.0, device="cuda"):
     """cos/sin table in the reference's layout (2, context_length, d/2) fp32, as
     RotaryEmbedding._build_cache builds it (llm-core/llm_core/model.py:86-91)."""
@@ -427,14 +487,30 @@ def build_rope_cache(context_length, d, theta=10000.0, device="cuda"):
     return torch.stack((torch.cos(angles), torch.sin(angles))).to(device)
 
 
-def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, slot_mapping=None, *, out=None):
+def _packed_k_out(k_out, k):
+    """k_out argument of the cache writes: None, True (allocate) or a tensor of k's shape to fill."""
+    if k_out is None or k_out is False:
+        return None
+    if k_out is True:
+        return torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    _require_gpu_bf16("k_out", k_out)
+    if k_out.shape != k.shape or k_out.stride(2) != 1 or k_out.stride(1) != k.shape[2] or k_out.stride(0) % 8 != 0 \
+            or k_out.data_ptr() % 16 != 0:
+        raise ValueError("k_out must have k's shape with contiguous heads, 16-byte aligned, token stride a multiple of 8")
+    return k_out
+
+
+def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, slot_mapping=None, *, out=None,
+                   k_out=None):
     """RoPE on q and k (interleaved pairs, llm-core/llm_core/model.py:93-104) and scatter of the
     rotated k and of v into the paged cache.
 
     q (T,Hq,D), k, v (T,Hkv,D) bf16 with contiguous heads; positions (T,) int32; freq_cache
     (2, context_length, D/2) fp32; slot_mapping (T,) int64 = block*16 + offset (negative: skip).
     Returns the rotated q (T,Hq,D) (written into `out` when given; `out` may be q itself); the
-    caches are updated in place.
+    caches are updated in place.  With `k_out` (True, or a (T,Hkv,D) tensor to fill) the same launch
+    also writes the rotated keys in packed form -- the K operand of a prefill over the same tokens --
+    and the return value is (rotated q, rotated k).
     """
     for n, t in (("q", q), ("k", k), ("v", v)):
         _require_gpu_bf16(n, t)
@@ -463,24 +539,29 @@ def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, s
         _require_gpu_bf16("out", q_out)
         if q_out.shape != q.shape or q_out.stride(2) != 1 or q_out.stride(1) != D:
             raise ValueError("out must have q's shape with contiguous heads")
+    k_rot = _packed_k_out(k_out, k)
     if T == 0:
-        return q_out
-    with _on(q, k, v, q_out, freq_cache, positions, slot_mapping, k_cache, v_cache) as stream:
+        return q_out if k_rot is None else (q_out, k_rot)
+    with _on(q, k, v, q_out, freq_cache, positions, slot_mapping, k_cache, v_cache, k_rot) as stream:
         rc = _lib.load().mi355_rope_and_cache(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
             None if slot_mapping is None else k_cache.data_ptr(), None if slot_mapping is None else v_cache.data_ptr(),
             freq_cache.data_ptr(), positions.data_ptr(), None if slot_mapping is None else slot_mapping.data_ptr(),
-            0 if slot_mapping is None else k_cache.shape[0], T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0), stream)
+            0 if slot_mapping is None else k_cache.shape[0], T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0),
+            v.stride(0), q_out.stride(0), None if k_rot is None else k_rot.data_ptr(),
+            0 if k_rot is None else k_rot.stride(0), stream)
     _lib.check(rc, "mi355_rope_and_cache")
-    return q_out
+    return q_out if k_rot is None else (q_out, k_rot)
 
 
-def rope_and_cache_fp8(q, k, v, positions, freq_cache, k_cache, v_cache, k_scale, v_scale, slot_mapping, *, out=None):
+def rope_and_cache_fp8(q, k, v, positions, freq_cache, k_cache, v_cache, k_scale, v_scale, slot_mapping, *, out=None,
+                       k_out=None):
     """rope_and_cache into an fp8-e4m3 cache: k_cache, v_cache (num_blocks,Hkv,16,D) uint8 (or
     float8_e4m3fn), k_scale, v_scale (num_blocks,Hkv) fp32, all updated in place.  A block's scale is
     kept equal to absmax/448 of its valid rows; rows already in a block are re-expressed when new rows
     raise the scale.  Tokens that share a block must be adjacent with consecutive slots, one such run
-    per block and call (what a prefill or a decode step produces).  Returns the rotated q."""
+    per block and call (what a prefill or a decode step produces).  Returns the rotated q, or, with
+    `k_out` (True or a tensor to fill), (rotated q, rotated keys in bf16, packed (T,Hkv,D))."""
     for n, t in (("q", q), ("k", k), ("v", v)):
         _require_gpu_bf16(n, t)
         if t.dim() != 3 or t.stride(2) != 1 or t.stride(1) != t.shape[2]:
@@ -517,15 +598,17 @@ def rope_and_cache_fp8(q, k, v, positions, freq_cache, k_cache, v_cache, k_scale
         if q_out.shape != q.shape or q_out.stride(2) != 1 or q_out.stride(1) != D or q_out.stride(0) % 8 != 0 \
                 or q_out.data_ptr() % 16 != 0:
             raise ValueError("out must have q's shape with contiguous heads, 16-byte aligned")
+    k_rot = _packed_k_out(k_out, k)
     if T == 0:
-        return q_out
-    with _on(q, k, v, q_out, freq_cache, positions, slot_mapping, k_cache, v_cache, k_scale, v_scale) as stream:
+        return q_out if k_rot is None else (q_out, k_rot)
+    with _on(q, k, v, q_out, freq_cache, positions, slot_mapping, k_cache, v_cache, k_scale, v_scale, k_rot) as stream:
         rc = _lib.load().mi355_rope_and_cache_fp8(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
             k_scale.data_ptr(), v_scale.data_ptr(), freq_cache.data_ptr(), positions.data_ptr(), slot_mapping.data_ptr(),
-            nb, T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0), stream)
+            nb, T, Hq, Hkv, D, freq_cache.shape[1], q.stride(0), k.stride(0), v.stride(0), q_out.stride(0),
+            None if k_rot is None else k_rot.data_ptr(), 0 if k_rot is None else k_rot.stride(0), stream)
     _lib.check(rc, "mi355_rope_and_cache_fp8")
-    return q_out
+    return q_out if k_rot is None else (q_out, k_rot)
 
 
 def quantize_kv_cache_fp8(cache, *, out=None):

@@ -223,6 +223,23 @@ def paged_decode_reference(q, k_cache, v_cache, block_tables, context_lens, *,
     return out
 
 
+def paged_prefill_reference(q, k_cache, v_cache, cu_seqlens_q, block_tables, context_lens, *, softmax_scale=None):
+    """Chunked-prefill oracle: q (T,Hq,D) packed; sequence b's chunk = rows [cu[b], cu[b+1]) attends to the
+    context_lens[b] cached tokens of that sequence (its own included) under the bottom-right aligned causal
+    mask -- prefill_reference on the gathered cache rows.  Returns (T,Hq,D) fp32."""
+    out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=torch.float32)
+    cq = [int(x) for x in cu_seqlens_q]
+    for b in range(len(cq) - 1):
+        if cq[b + 1] == cq[b]:
+            continue
+        kk = gather_paged_kv(k_cache, block_tables[b], context_lens[b]).unsqueeze(0)        # (1,Hkv,ctx,D)
+        vv = gather_paged_kv(v_cache, block_tables[b], context_lens[b]).unsqueeze(0)
+        qb = q[cq[b]:cq[b + 1]].transpose(0, 1).unsqueeze(0)
+        ob = prefill_reference(qb, kk, vv, causal=True, softmax_scale=softmax_scale)
+        out[cq[b]:cq[b + 1]] = ob[0].transpose(0, 1)
+    return out
+
+
 def quantize_kv_fp8(cache):
     """Per-(block, kv-head) absmax quantisation to OCP fp8-e4m3 (max 448).
 

@@ -130,3 +130,78 @@ def test_decode_with_full_batch_at_long_context_lengths(ctx_len):
     ref = orc.prefill_reference(q_rot[None], k_rot[None], v_all.transpose(0, 1)[None], causal=True)[0, :, 0]
     err = (out2[0] - ref).abs()
     assert bool((err <= 2e-2 + 1e-2 * ref.abs()).all()), float(err.max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D", [128, 64])
+def test_prompt_admitted_in_three_chunks_equals_one_shot_prefill(D):
+    """A prompt fed through plan_prefill in three ragged chunks (the second and third on top of cached
+    tokens, read back through the block tables) must give the attention rows of a one-shot prefill of
+    the same prompt: both within the bf16 tolerance of the oracle, and close to each other."""
+    import mi355_attn
+    print(f"case: engine chunked prefill D={D}", flush=True)
+    Hq, Hkv, ctx = 8, 2, 1024
+    fc = orc.build_rope_cache(ctx, D)
+    n = 700
+    q, k, v = rnd(n, Hq, D, seed=31), rnd(n, Hkv, D, seed=32), rnd(n, Hkv, D, seed=33)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+
+    one = mi355_attn.PagedAttentionEngine(num_blocks=64, n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D,
+                                          context_length=ctx, max_batch=4)
+    one.add_sequence(0)
+    whole = one.prefill([0], [n], qg, kg, vg).float().cpu()
+
+    eng = mi355_attn.PagedAttentionEngine(num_blocks=64, n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D,
+                                          context_length=ctx, max_batch=4)
+    eng.add_sequence(7)
+    eng.add_sequence(8)                  # a second, new sequence rides along with the last chunk
+    cuts = [0, 203, 460, n]              # ragged: none of the boundaries is a multiple of 16 or 64
+    parts = []
+    for c0, c1 in zip(cuts[:-1], cuts[1:]):
+        if c1 == n:
+            q2, k2, v2 = rnd(90, Hq, D, seed=41), rnd(90, Hkv, D, seed=42), rnd(90, Hkv, D, seed=43)
+            out = eng.prefill([7, 8], [c1 - c0, 90], torch.cat([qg[c0:c1], q2.cuda()]),
+                              torch.cat([kg[c0:c1], k2.cuda()]), torch.cat([vg[c0:c1], v2.cuda()])).float().cpu()
+            parts.append(out[:c1 - c0])
+            other = out[c1 - c0:]
+        else:
+            parts.append(eng.prefill([7], [c1 - c0], qg[c0:c1], kg[c0:c1], vg[c0:c1]).float().cpu())
+    chunked = torch.cat(parts)
+    assert eng.lengths[7] == n and eng.lengths[8] == 90
+    # the caches hold the same rows either way
+    blocks = one.blocks[0]
+    assert torch.equal(one.k_cache[blocks], eng.k_cache[eng.blocks[7]])
+    assert torch.equal(one.v_cache[blocks], eng.v_cache[eng.blocks[7]])
+
+    def oracle(qq, kk, vv):
+        p = torch.arange(qq.shape[0])
+        q_rot = orc.rope_reference(qq.float().transpose(0, 1), p, fc).to(torch.bfloat16)
+        k_rot = orc.rope_reference(kk.float().transpose(0, 1), p, fc).to(torch.bfloat16)
+        return orc.prefill_reference(q_rot[None], k_rot[None], vv.transpose(0, 1)[None], causal=True)[0].transpose(0, 1)
+
+    ref = oracle(q, k, v)
+    for name, got in (("one-shot", whole), ("chunked", chunked)):
+        err = (got - ref).abs()
+        assert bool((err <= 2e-2 + 1e-2 * ref.abs()).all()), (name, float(err.max()))
+    assert float((chunked - whole).abs().max()) <= 2e-2
+    ref2 = oracle(q2, k2, v2)
+    err = (other - ref2).abs()
+    assert bool((err <= 2e-2 + 1e-2 * ref2.abs()).all()), float(err.max())
+    # decoding continues from the chunked cache
+    qd, kd, vd = rnd(1, Hq, D, seed=51), rnd(1, Hkv, D, seed=52), rnd(1, Hkv, D, seed=53)
+    step = eng.decode_step([7], qd.cuda(), kd.cuda(), vd.cuda()).float().cpu()
+    full = oracle(torch.cat([q, qd]), torch.cat([k, kd]), torch.cat([v, vd]))[-1:]
+    err = (step - full).abs()
+    assert bool((err <= 2e-2 + 1e-2 * full.abs()).all()), float(err.max())
+
+
+@pytest.mark.gpu
+def test_chunked_prefill_needs_a_bf16_cache():
+    import mi355_attn
+    eng = mi355_attn.PagedAttentionEngine(num_blocks=16, n_q_heads=4, n_kv_heads=2, head_dim=64, context_length=128,
+                                          max_batch=2, kv_dtype="fp8")
+    eng.add_sequence(0)
+    q, k, v = rnd(20, 4, 64, seed=1).cuda(), rnd(20, 2, 64, seed=2).cuda(), rnd(20, 2, 64, seed=3).cuda()
+    eng.prefill([0], [20], q, k, v)
+    with pytest.raises(NotImplementedError):
+        eng.plan_prefill([0], [5])

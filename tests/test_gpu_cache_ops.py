@@ -75,6 +75,43 @@ def test_rope_and_cache_pair_path_and_out_argument(ops):
         ops.rope_and_cache(q, k, v, pos, fcg, kc_b, vc_b, slots, out=torch.empty(T, Hq, D + 8, dtype=torch.bfloat16, device="cuda"))
 
 
+@pytest.mark.parametrize("D,fp8", [(128, False), (64, False), (6, False), (128, True)])
+def test_rope_and_cache_also_returns_the_packed_rotated_keys(ops, D, fp8):
+    """k_out: the same launch that fills the cache hands back the rotated keys in packed form; they equal the
+    rows a separate rotation gives and (bf16 cache) the rows the cache received.  D = 6 takes the pair kernel."""
+    print(f"case: rope_and_cache k_out D={D} fp8={fp8}", flush=True)
+    T, Hq, Hkv, ctx = 50, 6, 2, 64
+    q, k, v = rnd(T, Hq, D, seed=1).cuda(), rnd(T, Hkv, D, seed=2).cuda(), rnd(T, Hkv, D, seed=3).cuda()
+    fcg = ops.build_rope_cache(ctx, D)
+    pos = torch.arange(T, dtype=torch.int32).cuda()
+    slots = (torch.arange(T, dtype=torch.int64) + 32).cuda()
+    k_plain = ops.rope_and_cache(k, k, v, pos, fcg)                     # queries-only call: rotates its first argument
+    q_plain = ops.rope_and_cache(q, k, v, pos, fcg)
+    if fp8:
+        k8 = torch.zeros(8, Hkv, 16, D, dtype=torch.uint8, device="cuda")
+        v8 = torch.zeros_like(k8)
+        ks, vs = torch.ones(8, Hkv, device="cuda"), torch.ones(8, Hkv, device="cuda")
+        k8b, v8b, ksb, vsb = k8.clone(), v8.clone(), ks.clone(), vs.clone()
+        q_rot, k_rot = ops.rope_and_cache_fp8(q, k, v, pos, fcg, k8, v8, ks, vs, slots, k_out=True)
+        ops.rope_and_cache_fp8(q, k, v, pos, fcg, k8b, v8b, ksb, vsb, slots)
+        assert torch.equal(k8, k8b) and torch.equal(v8, v8b) and torch.equal(ks, ksb) and torch.equal(vs, vsb)
+    else:
+        kc = torch.zeros(8, Hkv, 16, D, dtype=torch.bfloat16, device="cuda")
+        vc = torch.zeros_like(kc)
+        q_rot, k_rot = ops.rope_and_cache(q, k, v, pos, fcg, kc, vc, slots, k_out=True)
+        rows = kc.permute(0, 2, 1, 3).reshape(-1, Hkv, D)[32:32 + T]
+        assert torch.equal(rows, k_rot)
+        # without a cache: rotated q and k from one launch
+        q2, k2 = ops.rope_and_cache(q, k, v, pos, fcg, k_out=True)
+        assert torch.equal(q2, q_plain) and torch.equal(k2, k_plain)
+        # into a caller's tensor
+        if D % 8 == 0:
+            buf = torch.empty(T, Hkv, D, dtype=torch.bfloat16, device="cuda")
+            _, k3 = ops.rope_and_cache(q, k, v, pos, fcg, k_out=buf)
+            assert k3 is buf and torch.equal(buf, k_plain)
+    assert torch.equal(q_rot, q_plain) and torch.equal(k_rot, k_plain)
+
+
 def test_rope_and_cache_ignores_slots_outside_the_pool_and_clamps_positions(ops):
     print("case: rope_and_cache bad slots / positions", flush=True)
     T, Hq, Hkv, D, ctx, nb = 8, 2, 2, 64, 32, 3

@@ -338,6 +338,64 @@ def _reference_module_tensors(x_proj, freq, num_heads, amp):
     return Q, K, V
 
 
+@pytest.mark.parametrize("D,Hq,Hkv", [(128, 8, 2), (64, 4, 4), (32, 4, 1)])
+def test_paged_prefill_ragged_chunks_match_the_oracle(ops, D, Hq, Hkv):
+    """Chunks of new tokens over cached context, read through the block table: ragged chunk lengths and
+    contexts (a chunk that IS the whole context, one token over a long context, chunk ends inside a block,
+    several query tiles), garbage in unused blocks, in the tail of the last block and in the table tail."""
+    ctx = [700, 391, 64, 1500, 17, 300]
+    chunk = [203, 391, 1, 1, 17, 299]
+    print(f"case: paged prefill D={D} Hq={Hq} Hkv={Hkv}", flush=True)
+    _, kc, vc, bt, cl = orc.make_paged_case(batch=len(ctx), n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                            context_lens=ctx, pool_factor=1.3, seed=21, dtype=torch.bfloat16)
+    cu = torch.tensor([0] + list(torch.tensor(chunk).cumsum(0)), dtype=torch.int32)
+    q = rnd(int(cu[-1]), Hq, D, seed=22)
+    ref = orc.paged_prefill_reference(q, kc, vc, cu, bt, cl)
+    used = torch.zeros(kc.shape[0], dtype=torch.bool)
+    bt2 = bt.clone()
+    kc2, vc2 = kc.clone(), vc.clone()
+    for b, c in enumerate(ctx):
+        nb = (c + 15) // 16
+        used[bt[b, :nb].long()] = True
+        bt2[b, nb:] = 2 ** 30
+        if c % 16:
+            last = int(bt[b, (c - 1) // 16])
+            kc2[last, :, c % 16:] = float("nan")
+            vc2[last, :, c % 16:] = float("inf")
+    kc2[~used] = float("nan")
+    vc2[~used] = float("nan")
+    dev = "cuda:0"
+    got = ops.flash_attn_paged_prefill(q.to(dev), kc2.to(dev), vc2.to(dev), cu.to(dev), bt2.to(dev), cl.to(dev), max(chunk))
+    torch.cuda.synchronize()
+    check(got, ref, what="paged prefill")
+    # a strided q (a slice of a fused projection) and a caller-provided output
+    wide = torch.zeros(q.shape[0], Hq + 2, D, dtype=torch.bfloat16, device=dev)
+    wide[:, :Hq] = q.to(dev)
+    out = torch.empty_like(got)
+    ret = ops.flash_attn_paged_prefill(wide[:, :Hq], kc2.to(dev), vc2.to(dev), cu.to(dev), bt2.to(dev), cl.to(dev),
+                                       max(chunk), out=out)
+    assert ret is out and torch.equal(out, got)
+
+
+def test_paged_prefill_equals_dense_prefill_on_the_gathered_rows(ops):
+    """The paged walk changes where keys come from, not the arithmetic: same bits as the packed kernel fed with
+    the gathered rows (head_dim 64: both calls run the same kernel)."""
+    print("case: paged prefill vs packed", flush=True)
+    Hq, Hkv, D = 4, 2, 64
+    ctx, chunk = [333, 130], [100, 130]
+    _, kc, vc, bt, cl = orc.make_paged_case(batch=2, n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                            context_lens=ctx, seed=5, dtype=torch.bfloat16)
+    cu_q = torch.tensor([0, 100, 230], dtype=torch.int32)
+    cu_k = torch.tensor([0, 333, 463], dtype=torch.int32)
+    q = rnd(230, Hq, D, seed=6)
+    kk = torch.cat([orc.gather_paged_kv(kc, bt[b], ctx[b]).transpose(0, 1) for b in range(2)]).to(torch.bfloat16)
+    vv = torch.cat([orc.gather_paged_kv(vc, bt[b], ctx[b]).transpose(0, 1) for b in range(2)]).to(torch.bfloat16)
+    dev = "cuda:0"
+    a = ops.flash_attn_paged_prefill(q.to(dev), kc.to(dev), vc.to(dev), cu_q.to(dev), bt.to(dev), cl.to(dev), 130)
+    b = ops.flash_attn_varlen_prefill(q.to(dev), kk.to(dev), vv.to(dev), cu_q.to(dev), cu_k.to(dev), 130, 333, causal=True)
+    assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("amp", [True, False])
 def test_sdpa_slot_takes_the_reference_modules_tensors(ops, amp):
     """The swap at model.py:382 with the tensors the reference really passes there: float32 Q/K + strided bf16 V

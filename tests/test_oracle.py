@@ -494,3 +494,22 @@ def test_backward_oracle_closed_forms():
     k2 = torch.randn(1, 1, 5, 8, generator=g)
     dq, dk, _, _ = orc.prefill_backward_reference(q, k2, v2, dout, causal=False)
     assert dq.abs().max() < 1e-5 and dk.abs().max() < 1e-5
+
+
+def test_paged_prefill_reference_is_the_tail_of_a_whole_prefill():
+    """A chunk attending to its cached context gives rows [c0, c1) of the causal prefill of the first c1 tokens."""
+    Hq, Hkv, D = 4, 2, 16
+    ctx = [45, 23]
+    chunk = [13, 23]
+    _, kc, vc, bt, cl = orc.make_paged_case(batch=2, n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                            context_lens=ctx, pool_factor=1.5, seed=3)
+    g = torch.Generator().manual_seed(4)
+    q_full = [torch.randn(c, Hq, D, generator=g) for c in ctx]
+    q = torch.cat([qf[c - n:] for qf, c, n in zip(q_full, ctx, chunk)])
+    cu = torch.tensor([0, 13, 36])
+    got = orc.paged_prefill_reference(q, kc, vc, cu, bt, cl)
+    for b in range(2):
+        kk = orc.gather_paged_kv(kc, bt[b], ctx[b])[None]
+        vv = orc.gather_paged_kv(vc, bt[b], ctx[b])[None]
+        whole = orc.prefill_reference(q_full[b].transpose(0, 1)[None], kk, vv, causal=True)[0].transpose(0, 1)
+        torch.testing.assert_close(got[int(cu[b]):int(cu[b + 1])], whole[ctx[b] - chunk[b]:], rtol=1e-5, atol=1e-6)
