@@ -13,7 +13,7 @@ The CPU baseline is the oracle (a restatement of the reference's PyTorch attenti
 timed on the host cores over a bounded sample of the same inputs; its outputs also
 check the GPU results of that sample.
 
-usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|fp8|backward|producers|layer|loop]
+usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|few|fp8|backward|producers|layer|loop]
                        [--no-cpu]
 """
 from __future__ import annotations
@@ -429,6 +429,48 @@ def bench_prefill(cfg, args):
     return res, (case, holder["out"])
 
 
+def bench_prefill_few_sequences(args):
+    """Prefill of ONE sequence (what a per-request prefill of `generate` produces): whole long prompts, where the
+    launch of one workgroup per pair of query tiles still fills the GPU, and a chunk of a prompt over a long cached
+    context, where it does not and the keys are split over workgroups (mi355_prefill_fwd_splitkv)."""
+    import torch
+    import mi355_attn
+
+    Hq, Hkv, D = 32, 8, 128
+    g = torch.Generator(device="cuda").manual_seed(args.seed + 7)
+
+    def rnd(*shape):
+        return (torch.randn(*shape, generator=g, device="cuda") * 0.5).to(torch.bfloat16)
+
+    out = {}
+    steps, warmup = max(1, args.steps // 2), args.warmup
+    for name, Sq, Sk in (("prompt_8192", 8192, 8192), ("prompt_16384", 16384, 16384), ("prompt_2048", 2048, 2048),
+                         ("chunk_256_over_16384", 256, 16384)):
+        q, k, v = rnd(1, Hq, Sq, D), rnd(1, Hkv, Sk, D), rnd(1, Hkv, Sk, D)
+        flops = 4.0 * Hq * D * (Sq * (Sk - Sq) + Sq * Sq / 2.0)          # causal convention, bottom-right diagonal
+        n_split = mi355_attn.suggest_kv_splits(1, Hq, D, Sq, Sk, Sq, True, q.device)
+        ws = mi355_attn.prefill_splitkv_workspace(Sq, Hq, D, n_split, q.device) if n_split > 1 else None
+        wall_ms, dev_ms = timed(lambda: mi355_attn.flash_attn_prefill(q, k, v, causal=True, kv_splits=n_split, workspace=ws),
+                                steps, warmup, BURN_IN)
+        res = {
+            "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
+            "algorithmic_flops": flops, "kv_splits": n_split,
+            "config": {"workload": "causal prefill forward of one sequence, %d query rows over %d keys, 32 q / 8 kv heads, "
+                                   "head_dim 128, dense layout" % (Sq, Sk)},
+            "roofline": {"bound": "mfma",
+                         "kernel": "prefill_fwd_w64_kernel<causal>" if n_split == 1 else
+                                   "prefill_fwd_kernel<128, causal> (keys split %d ways) + prefill_merge_kernel" % n_split,
+                         "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms, "traffic": None},
+        }
+        if n_split > 1:
+            _, one_ms = timed(lambda: mi355_attn.flash_attn_prefill(q, k, v, causal=True, kv_splits=1), steps, warmup)
+            res["unsplit_device_ms"] = one_ms
+            res["speedup_over_unsplit"] = one_ms / dev_ms
+        out[name] = res
+    return out
+
+
 def cpu_prefill(case, gpu_out, cfg, n_heads=8):
     import torch
     from oracle import attention_oracle as orc
@@ -466,7 +508,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", choices=["decode", "prefill", "fp8", "backward", "producers", "layer", "loop"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "few", "fp8", "backward", "producers", "layer", "loop"], default=None)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the 1 GiB plain copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
@@ -523,6 +565,8 @@ def main():
         if args.only == "prefill":
             line.update({"value": pre["value"], "unit": "TFLOP/s", "ms_per_step": pre["ms_per_step"], "dtype": "bf16",
                          "config": pre["config"], "roofline": pre["roofline"]})
+    if args.only in (None, "few"):
+        line["prefill_few_sequences"] = bench_prefill_few_sequences(args)
     if args.only in (None, "backward"):
         line["prefill_backward"] = bench_prefill_backward(2, args)
     if args.only in (None, "fp8"):

@@ -104,13 +104,51 @@ int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out
  * Same mathematics as mi355_prefill_fwd (model.py:308-325 / :382) -- the reference has no cache,
  * so it has no counterpart of the table walk; what it replaces is re-running the whole prefix at
  * model.py:218 when a prompt arrives in pieces.
+ * n_split > 1 splits every sequence's keys over n_split workgroups (see mi355_prefill_fwd_splitkv:
+ * a short chunk over a long context would otherwise occupy a handful of compute units); it then needs
+ * total_q_rows = cu_seqlens_q[B] and a workspace of mi355_prefill_splitkv_workspace_bytes().
+ * n_split <= 1: workspace may be NULL.
  */
 int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
                             int64_t q_token_stride, int64_t out_token_stride,
                             const int32_t* cu_seqlens_q, const int32_t* block_tables, int64_t table_stride,
                             const int32_t* context_lens, int B, int Hq, int Hkv, int Sq_max, int D,
                             int block_size, int64_t num_blocks, float softmax_scale, int kv_dtype,
+                            int n_split, int64_t total_q_rows, void* workspace, size_t workspace_bytes,
                             void* stream);
+
+/*
+ * mi355_prefill_fwd with the keys of every sequence split over n_split workgroups (flash-decoding for
+ * prefill): share c of a query tile's K/V tiles yields a normalised fp32 partial result and its
+ * log-sum-exp per query row, and a second kernel merges them,
+ *   out = sum_c w_c O_c / sum_c w_c,   w_c = exp(lse_c - max lse).
+ * For few or short query sequences over long key sequences (one long prompt, a short chunk over a
+ * long context), where one workgroup per pair of query tiles leaves most compute units idle.  The
+ * partials cost 4 (D + 1) n_split bytes of traffic per query row and head each way, so splitting pays
+ * when queries are few.  Same arguments as mi355_prefill_fwd (mask modes NONE / CAUSAL), plus:
+ *   n_split       1..64 (1: plain mi355_prefill_fwd, no workspace needed)
+ *   total_q_rows  B * Sq_max (dense) or the packed number of query rows
+ *   workspace     >= mi355_prefill_splitkv_workspace_bytes(total_q_rows, Hq, D, n_split), 16-byte aligned
+ * No reference counterpart beyond the mathematics of model.py:308-325.
+ */
+size_t mi355_prefill_splitkv_workspace_bytes(int64_t total_q_rows, int Hq, int D, int n_split);
+/*
+ * A good n_split for a forward prefill of this shape (1 = do not split): a host-side cost model fitted to
+ * timings on an MI355X -- a share of the keys must save more tile-loop time than its fp32 partial rows cost in
+ * traffic, so few query rows over many keys split 4..16 ways and a launch that fills the GPU is left alone.
+ * Sq_max / Sk_max: longest query / key sequence; causal: non-zero for MI355_MASK_CAUSAL;
+ * n_compute_units <= 0: ask the current device (the only case that touches the GPU runtime).
+ */
+int mi355_prefill_suggest_kv_splits(int B, int Hq, int D, int Sq_max, int Sk_max, int64_t total_q_rows,
+                                    int causal, int n_compute_units);
+int mi355_prefill_fwd_splitkv(const void* q, const void* k, const void* v, void* out,
+                              const int64_t q_strides[3], const int64_t k_strides[3],
+                              const int64_t v_strides[3], const int64_t o_strides[3],
+                              const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                              int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
+                              float softmax_scale, int mask_mode, int dtype,
+                              int n_split, int64_t total_q_rows, void* workspace, size_t workspace_bytes,
+                              void* stream);
 
 /*
  * Prefill backward: dq, dk, dv of out = softmax(q k^T * softmax_scale [causal]) v given dout,

@@ -65,6 +65,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     const int n_wg = gridDim.x;
     int lid = blockIdx.x;
     if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
+    const int split = blockIdx.y;                    // share of the keys this workgroup serves (gridDim.y = n_split)
     const int pair0 = lid % p.n_pairs;
     const int h = (lid / p.n_pairs) % p.Hq;
     const int b = lid / (p.n_pairs * p.Hq);
@@ -74,6 +75,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     const __bf16 *qb, *kb, *vb;
     __bf16* ob;
     float* lb;
+    int64_t part_row0 = (int64_t)b * p.Sq;          // first row of this sequence in the partial buffers
+    if (PAGED || p.cu_q) part_row0 = p.cu_q[b];
     if constexpr (PAGED) {
         const int q_start = p.cu_q[b];
         sq = p.cu_q[b + 1] - q_start;
@@ -215,10 +218,17 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
         int kv_end = sk;
         if (causal) kv_end = max(0, min(sk, min(sq, q0 + kBM) + coff));
         const int n_tiles = (kv_end + kBN - 1) / kBN;
+        int t0 = 0, t1 = n_tiles;                  // this workgroup's tiles
+        if (p.n_split > 1) {
+            const int per = (n_tiles + p.n_split - 1) / p.n_split;
+            t0 = min(n_tiles, split * per);
+            t1 = min(n_tiles, t0 + per);
+        }
 
         // the first K/V tile is requested before the query rows, so that the two latencies overlap
+        // (tile t lives in buffer t % 2)
         __syncthreads();                     // the previous query tile's readers are done with the LDS buffers
-        if (n_tiles > 0) issue_tile(0, 0);
+        if (t1 > t0) issue_tile(t0, t0 & 1);
 
         // ---- Q^T fragments: step s covers d = 16s + 8kg + j ----------------------
         // rows come in whole (CPR lanes per row) and go through the wavefront's slab (private, and LDS operations
@@ -282,7 +292,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
             __syncthreads();                 // ... and everybody's; also: all are done reading the other buffer
 
             // The next tile's direct-to-LDS loads go out first: a whole tile of work hides their latency.
-            if (tile + 1 < n_tiles) issue_tile(tile + 1, (tile + 1) & 1);
+            if (tile + 1 < t1) issue_tile(tile + 1, (tile + 1) & 1);
 
             const int k0 = tile * kBN;
             if (causal && MASKED && k0 > qw0 + 31 + coff) return false;
@@ -384,12 +394,34 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
             }
         };
 
-        run_tiles(std::false_type{}, 0, n_plain);
-        run_tiles(std::true_type{}, n_plain, n_tiles);
-        if (n_tiles & 1) flip();             // leave the offsets pointing at buffer 0 for the next query tile
+        if (t1 > t0 && (t0 & 1)) flip();     // the offsets start at the first tile's buffer ...
+        run_tiles(std::false_type{}, t0, min(n_plain, t1));
+        run_tiles(std::true_type{}, max(n_plain, t0), t1);
+        if (t1 > t0 && (t1 & 1)) flip();     // ... and are left pointing at buffer 0 for the next query tile
 
         // ---- normalise and store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4 ---
         l_run = xor32_sum(l_run);
+        if (p.n_split > 1) {
+            // partial result of this share of the keys: normalised fp32 rows and their log-sum-exp (-inf and
+            // zeros when the share kept no key for the row); the merge kernel weighs them
+            const float inv_p = l_run > 0.f ? 1.0f / l_run : 0.f;
+            if (q_ok) {
+                const int64_t prow = ((int64_t)split * p.Hq + h) * p.part_rows + part_row0 + qi;
+                if (kg == 0)
+                    p.part_lse[prow] = l_run > 0.f ? 0.69314718056f * (m_ref * p.scale_log2 + __log2f(l_run)) : -INFINITY;
+                float* po = p.part_o + prow * D + 4 * kg;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        f32x4 w;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) w[e] = o[dt][4 * g + e] * inv_p;
+                        *reinterpret_cast<f32x4*>(po + 32 * dt + 8 * g) = w;
+                    }
+            }
+            continue;
+        }
         const float inv = 1.0f / l_run;          // l == 0 (no key kept) -> NaN row, like the reference softmax
         // sum_j exp(scale * s_j) = 2^(m_ref * scale_log2) * l  ->  lse = ln2 * (m_ref * scale_log2 + log2 l)
         if (lb && q_ok && kg == 0)
@@ -422,7 +454,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
 
 template <int D>
 static int launch_prefill(const PrefillParams& p, hipStream_t stream) {
-    dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B));    // one workgroup per PAIR of query tiles, 1-D (see the id remap)
+    // one workgroup per PAIR of query tiles, 1-D in x (see the id remap); y = share of the keys
+    dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B), (unsigned)(p.n_split > 1 ? p.n_split : 1));
     dim3 block(kPfWaves * 64);
     if (p.mask_mode == MI355_MASK_CAUSAL)
         hipLaunchKernelGGL((prefill_fwd_kernel<D, MI355_MASK_CAUSAL>), grid, block, 0, stream, p);
@@ -433,9 +466,60 @@ static int launch_prefill(const PrefillParams& p, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// Merge of the split-key partials: one wavefront per (query row, head).
+//   out = sum_c w_c O_c / sum_c w_c,  w_c = exp(lse_c - max_c lse_c);  no share kept a key -> NaN, like the reference
+struct MergeParams {
+    const float* part_o;
+    const float* part_lse;
+    __bf16* out;
+    int64_t os[3];
+    int64_t part_rows;
+    int n_split, Hq, D, Sq_dense;        // Sq_dense: rows per batch entry of the dense layout, 0 = packed
+};
+__global__ __launch_bounds__(256) void prefill_merge_kernel(MergeParams p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (w >= p.part_rows * p.Hq) return;
+    const int h = (int)(w % p.Hq);
+    const int64_t row = w / p.Hq;
+    float m = -INFINITY;
+    for (int c = 0; c < p.n_split; ++c) m = fmaxf(m, p.part_lse[((int64_t)c * p.Hq + h) * p.part_rows + row]);
+    __bf16* dst = p.Sq_dense ? p.out + (row / p.Sq_dense) * p.os[0] + (int64_t)h * p.os[1] + (row % p.Sq_dense) * p.os[2]
+                             : p.out + row * p.os[2] + (int64_t)h * p.os[1];
+    for (int d = lane; d < p.D; d += 64) {
+        float num = 0.f, den = 0.f;
+        for (int c = 0; c < p.n_split; ++c) {
+            const int64_t prow = ((int64_t)c * p.Hq + h) * p.part_rows + row;
+            const float l = p.part_lse[prow];
+            if (l == -INFINITY) continue;                 // (its rows may never have been written)
+            const float wgt = __expf(l - m);
+            num += wgt * p.part_o[prow * p.D + d];
+            den += wgt;
+        }
+        dst[d] = (__bf16)(m == -INFINITY ? __builtin_nanf("") : num / den);
+    }
+}
+
+static int launch_merge(const PrefillParams& p, int D, hipStream_t stream) {
+    MergeParams m;
+    m.part_o = p.part_o;
+    m.part_lse = p.part_lse;
+    m.out = p.out;
+    for (int i = 0; i < 3; ++i) m.os[i] = p.os[i];
+    m.part_rows = p.part_rows;
+    m.n_split = p.n_split;
+    m.Hq = p.Hq;
+    m.D = D;
+    m.Sq_dense = (p.cu_q || p.block_table) ? 0 : p.Sq;
+    const int64_t wgs = (p.part_rows * p.Hq + 3) / 4;
+    if (wgs > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(prefill_merge_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, m);
+    return (int)hipGetLastError();
+}
+
 template <int D>
 static int launch_prefill_paged(const PrefillParams& p, hipStream_t stream) {
-    dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B));
+    dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B), (unsigned)(p.n_split > 1 ? p.n_split : 1));
     hipLaunchKernelGGL((prefill_fwd_kernel<D, MI355_MASK_CAUSAL, true>), grid, dim3(kPfWaves * 64), 0, stream, p);
     return (int)hipGetLastError();
 }
@@ -444,12 +528,39 @@ static int launch_prefill_paged(const PrefillParams& p, hipStream_t stream) {
 
 using namespace mi355;
 
+static size_t split_workspace_bytes(int64_t total_q_rows, int Hq, int D, int n_split) {
+    return (size_t)n_split * (size_t)Hq * (size_t)total_q_rows * (size_t)(D + 1) * sizeof(float);
+}
+
+// Split-key fields of the parameters (n_split <= 1: none).  `expected_rows` >= 0: what total_q_rows must equal.
+static int set_split(PrefillParams& p, int D, int n_split, int64_t total_q_rows, void* workspace, size_t workspace_bytes,
+                     int64_t expected_rows) {
+    p.n_split = 1;
+    p.part_o = nullptr;
+    p.part_lse = nullptr;
+    p.part_rows = 0;
+    if (n_split <= 1) return 0;
+    if (n_split > 64) return set_error(MI355_EINVAL, "prefill: n_split must be at most 64");
+    if (total_q_rows <= 0 || (expected_rows >= 0 && total_q_rows != expected_rows))
+        return set_error(MI355_EINVAL, "prefill: total_q_rows must be the number of query rows (B * Sq, or the packed total)");
+    if (!workspace || ((uintptr_t)workspace & 15))
+        return set_error(MI355_EINVAL, "prefill: split keys need a 16-byte aligned workspace");
+    if (workspace_bytes < split_workspace_bytes(total_q_rows, p.Hq, D, n_split))
+        return set_error(MI355_EWORKSPACE, "prefill: workspace smaller than mi355_prefill_splitkv_workspace_bytes()");
+    p.n_split = n_split;
+    p.part_rows = total_q_rows;
+    p.part_o = (float*)workspace;
+    p.part_lse = p.part_o + (size_t)n_split * p.Hq * total_q_rows * D;
+    return 0;
+}
+
 static int prefill_common(const void* q, const void* k, const void* v, void* out, const int64_t q_strides[3],
                           const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
                           const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const uint8_t* mask,
                           const int64_t mask_strides[3], int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
                           float softmax_scale, int mask_mode, int dtype, float* lse, const int64_t* lse_strides,
-                          void* stream) {
+                          void* stream, int n_split = 1, int64_t total_q_rows = 0, void* workspace = nullptr,
+                          size_t workspace_bytes = 0) {
     if (!q || !k || !v || !out || !q_strides || !k_strides || !v_strides || !o_strides)
         return set_error(MI355_EINVAL, "prefill: null pointer argument");
     if (dtype != MI355_BF16) return set_error(MI355_EDTYPE, "prefill: dtype must be MI355_BF16");
@@ -503,10 +614,18 @@ static int prefill_common(const void* q, const void* k, const void* v, void* out
     p.ctx_lens = nullptr;
     p.table_stride = 0;
     p.num_blocks = 0;
+    if (int e = set_split(p, D, n_split, total_q_rows, workspace, workspace_bytes, cu_seqlens_q ? -1 : (int64_t)B * Sq_max))
+        return e;
     if ((int64_t)p.n_pairs * Hq * B > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill: too many workgroups");
 
     hipStream_t s = (hipStream_t)stream;
     int rc;
+    if (p.n_split > 1) {
+        rc = D == 128 ? launch_prefill<128>(p, s) : (D == 64 ? launch_prefill<64>(p, s) : launch_prefill<32>(p, s));
+        if (rc == 0) rc = launch_merge(p, D, s);
+        if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
+        return MI355_OK;
+    }
     // head_dim 128 without an explicit mask and without lse: the kernel with 64 queries per wavefront and a
     // hand-scheduled tile loop
     if (D == 128 && mask_mode != MI355_MASK_BOOL && !lse) rc = launch_prefill_w64(p, s);
@@ -545,7 +664,8 @@ extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const
                                        int64_t q_token_stride, int64_t out_token_stride, const int32_t* cu_seqlens_q,
                                        const int32_t* block_tables, int64_t table_stride, const int32_t* context_lens,
                                        int B, int Hq, int Hkv, int Sq_max, int D, int block_size, int64_t num_blocks,
-                                       float softmax_scale, int kv_dtype, void* stream) {
+                                       float softmax_scale, int kv_dtype, int n_split, int64_t total_q_rows,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !k_cache || !v_cache || !out || !cu_seqlens_q || !block_tables || !context_lens)
         return set_error(MI355_EINVAL, "prefill_paged: null pointer argument");
     if (kv_dtype != MI355_BF16) return set_error(MI355_EDTYPE, "prefill_paged: the cache must be MI355_BF16");
@@ -584,9 +704,73 @@ extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const
     p.ctx_lens = context_lens;
     p.table_stride = table_stride;
     p.num_blocks = (int)num_blocks;
+    if (int e = set_split(p, D, n_split, total_q_rows, workspace, workspace_bytes, -1)) return e;
     if ((int64_t)p.n_pairs * Hq * B > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill_paged: too many workgroups");
     hipStream_t s = (hipStream_t)stream;
-    const int rc = D == 128 ? launch_prefill_paged<128>(p, s) : (D == 64 ? launch_prefill_paged<64>(p, s) : launch_prefill_paged<32>(p, s));
+    int rc = D == 128 ? launch_prefill_paged<128>(p, s) : (D == 64 ? launch_prefill_paged<64>(p, s) : launch_prefill_paged<32>(p, s));
+    if (rc == 0 && p.n_split > 1) rc = launch_merge(p, D, s);
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;
+}
+
+extern "C" size_t mi355_prefill_splitkv_workspace_bytes(int64_t total_q_rows, int Hq, int D, int n_split) {
+    if (total_q_rows <= 0 || Hq <= 0 || D <= 0 || n_split <= 1) return 0;
+    return split_workspace_bytes(total_q_rows, Hq, D, n_split);
+}
+
+// Cost model behind mi355_prefill_suggest_kv_splits, in microseconds, from timings on an MI355X (32 and 8 query
+// heads, head_dim 128, 64..2048 query rows over 1.5K..32K keys): a workgroup spends about 1.5 us per K/V tile of 64
+// keys (1.6 us in the split kernel) and 5 us per query tile outside the tile loop; the partial rows cost their bytes
+// twice (written, then read by the merge) at about 2.5 TB/s, plus 8 us for the second launch.
+extern "C" int mi355_prefill_suggest_kv_splits(int B, int Hq, int D, int Sq_max, int Sk_max, int64_t total_q_rows,
+                                               int causal, int n_compute_units) {
+    if (B <= 0 || Hq <= 0 || D <= 0 || Sq_max <= 0 || Sk_max <= 0 || total_q_rows <= 0) return 1;
+    int n_cu = n_compute_units;
+    if (n_cu <= 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0)
+            return 1;
+    }
+    const int nq = (Sq_max + kBM - 1) / kBM, n_pairs = (nq + 1) / 2;
+    const double jobs = (double)n_pairs * Hq * B;
+    // K/V tiles and query tiles of the heaviest workgroup (a pair of query tiles; causal: bottom-right diagonal)
+    const double halves = nq >= 2 ? 2.0 : 1.0;
+    double keys = halves * Sk_max;
+    if (causal) {
+        const int over = Sk_max > Sq_max ? Sk_max - Sq_max : 0;         // keys every query sees
+        keys = nq >= 2 ? 2.0 * over + Sq_max + kBM : (double)over + (Sq_max < kBM ? Sq_max : kBM);
+        if (keys > halves * Sk_max) keys = halves * Sk_max;
+    }
+    const double tiles = keys / kBN;
+    const auto rounds = [&](double wgs) { return (double)(int64_t)((wgs + n_cu - 1) / n_cu); };
+    const double plain = rounds(jobs) * (tiles * 1.5 + 5.0 * halves);
+    double best = plain * 0.85;                       // a split must win clearly
+    int best_n = 1;
+    static const int kCandidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
+    for (int n : kCandidates) {
+        if (tiles / n < 2.0 * halves) break;          // at least two tiles per share and query tile
+        const double bytes = (double)total_q_rows * Hq * (D + 1) * 4.0 * n;
+        const double t = rounds(jobs * n) * (tiles / n * 1.6 + 5.0 * halves) + 8.0 + 2.0 * bytes / 2.5e6;
+        if (t < best) {
+            best = t;
+            best_n = n;
+        }
+    }
+    return best_n;
+}
+
+extern "C" int mi355_prefill_fwd_splitkv(const void* q, const void* k, const void* v, void* out,
+                                         const int64_t q_strides[3], const int64_t k_strides[3],
+                                         const int64_t v_strides[3], const int64_t o_strides[3],
+                                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int B, int Hq, int Hkv,
+                                         int Sq_max, int Sk_max, int D, float softmax_scale, int mask_mode, int dtype,
+                                         int n_split, int64_t total_q_rows, void* workspace, size_t workspace_bytes,
+                                         void* stream) {
+    if (mask_mode == MI355_MASK_BOOL)
+        return set_error(MI355_EINVAL, "prefill_fwd_splitkv: mask_mode must be MI355_MASK_NONE or MI355_MASK_CAUSAL");
+    if (n_split < 1) return set_error(MI355_EINVAL, "prefill_fwd_splitkv: n_split must be at least 1");
+    return prefill_common(q, k, v, out, q_strides, k_strides, v_strides, o_strides, cu_seqlens_q, cu_seqlens_k, nullptr,
+                          nullptr, B, Hq, Hkv, Sq_max, Sk_max, D, softmax_scale, mask_mode, dtype, nullptr, nullptr, stream,
+                          n_split, total_q_rows, workspace, workspace_bytes);
 }

@@ -28,6 +28,14 @@ struct PrefillParams {
     const int32_t* ctx_lens;
     int64_t table_stride;
     int num_blocks;
+    // split keys (n_split > 1): workgroup (.., split c) serves the c-th share of every query tile's K/V tiles and
+    // writes, instead of `out`, a normalised fp32 partial result and its log-sum-exp per query row:
+    //   part_o  (n_split, Hq, part_rows, D)    part_lse (n_split, Hq, part_rows)
+    // row = packed row, or b * Sq + i in the dense layout; a second kernel merges the partials into `out`
+    int n_split;
+    float* part_o;
+    float* part_lse;
+    int64_t part_rows;
 };
 
 // The 64-queries-per-wavefront kernel (head_dim 128, no mask or causal, no lse): prefill_fwd_w64.hip.

@@ -28,6 +28,8 @@ from .ops import (  # noqa: F401
     flash_attn_varlen_prefill,
     paged_attention_decode,
     paged_decode_workspace,
+    prefill_splitkv_workspace,
+    suggest_kv_splits,
     scaled_dot_product_attention,
     sdpa_slot,
 )

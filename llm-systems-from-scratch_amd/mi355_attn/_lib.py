@@ -26,6 +26,9 @@ EXPORTS = (
     "mi355_paged_decode_workspace_bytes",
     "mi355_paged_decode_chunk_tokens",
     "mi355_prefill_paged_fwd",
+    "mi355_prefill_fwd_splitkv",
+    "mi355_prefill_splitkv_workspace_bytes",
+    "mi355_prefill_suggest_kv_splits",
     "mi355_rope_and_cache",
     "mi355_rope_and_cache_fp8",
     "mi355_quantize_kv_fp8",
@@ -63,7 +66,14 @@ def load():
                                                                  i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
     lib.mi355_prefill_paged_fwd.restype = i32
     lib.mi355_prefill_paged_fwd.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, i64, vp,
-                                            i32, i32, i32, i32, i32, i32, i64, f32, i32, vp]
+                                            i32, i32, i32, i32, i32, i32, i64, f32, i32, i32, i64, vp, sz, vp]
+    lib.mi355_prefill_fwd_splitkv.restype = i32
+    lib.mi355_prefill_fwd_splitkv.argtypes = [vp, vp, vp, vp, _i64x3, _i64x3, _i64x3, _i64x3, vp, vp,
+                                              i32, i32, i32, i32, i32, i32, f32, i32, i32, i32, i64, vp, sz, vp]
+    lib.mi355_prefill_splitkv_workspace_bytes.restype = sz
+    lib.mi355_prefill_splitkv_workspace_bytes.argtypes = [i64, i32, i32, i32]
+    lib.mi355_prefill_suggest_kv_splits.restype = i32
+    lib.mi355_prefill_suggest_kv_splits.argtypes = [i32, i32, i32, i32, i32, i64, i32, i32]
     lib.mi355_paged_decode_fwd.restype = i32
     lib.mi355_paged_decode_fwd.argtypes = [vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, sz,
                                            i32, i32, i32, i32, i32, i64, i32, f32, i32, vp]

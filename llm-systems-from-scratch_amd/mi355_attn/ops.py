@@ -81,8 +81,52 @@ def _packed_or_dense_strides(t, packed):
     return (0, t.stride(1), t.stride(0)) if packed else t.stride()[:3]
 
 
-def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode, lse=None):
+_N_CU = {}
+
+
+def suggest_kv_splits(B, Hq, D, sq_max, sk_max, total_rows, causal, device):
+    """The library's suggestion for this shape (mi355_prefill_suggest_kv_splits: a cost model of tile-loop time
+    saved against the traffic of the partial rows); 1 = do not split."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx not in _N_CU:
+        _N_CU[idx] = torch.cuda.get_device_properties(idx).multi_processor_count
+    return _lib.load().mi355_prefill_suggest_kv_splits(int(B), int(Hq), int(D), int(sq_max), int(sk_max),
+                                                       int(total_rows), 1 if causal else 0, _N_CU[idx])
+
+
+def prefill_splitkv_workspace(total_q_rows, n_q_heads, head_dim, kv_splits, device):
+    """Scratch tensor for a prefill call with kv_splits > 1 (fp32 partial rows and their log-sum-exps)."""
+    n = _lib.load().mi355_prefill_splitkv_workspace_bytes(int(total_q_rows), n_q_heads, head_dim, int(kv_splits))
+    return torch.empty(max(int(n), 16), dtype=torch.uint8, device=device)
+
+
+def _split_args(kv_splits, workspace, B, Hq, D, sq_max, sk_max, total_rows, causal, device):
+    """(n_split, workspace) for a forward-only prefill call; kv_splits None = choose."""
+    n = suggest_kv_splits(B, Hq, D, sq_max, sk_max, total_rows, causal, device) if kv_splits is None else int(kv_splits)
+    if n < 1 or n > 64:
+        raise ValueError("kv_splits must be in 1..64")
+    if n == 1:
+        return 1, None
+    if workspace is None:
+        workspace = prefill_splitkv_workspace(total_rows, Hq, D, n, device)
+    return n, workspace
+
+
+def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode, lse=None, n_split=1, workspace=None,
+             total_rows=0):
     lib = _lib.load()
+    if n_split > 1:
+        packed = cu_q is not None
+        qs, ks, vs, os_ = (_packed_or_dense_strides(x, packed) for x in (q, k, v, out))
+        with _on(q, k, v, out, cu_q, cu_k, workspace) as stream:
+            rc = lib.mi355_prefill_fwd_splitkv(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
+                None if cu_q is None else cu_q.data_ptr(), None if cu_k is None else cu_k.data_ptr(),
+                B, Hq, Hkv, Sq, Sk, D, float(scale), mode, _lib.MI355_BF16, int(n_split), int(total_rows),
+                workspace.data_ptr(), workspace.numel() * workspace.element_size(), stream)
+        _lib.check(rc, "mi355_prefill_fwd_splitkv")
+        return
     if lse is not None:
         packed = cu_q is not None
         qs, ks, vs, os_ = (_packed_or_dense_strides(x, packed) for x in (q, k, v, out))
@@ -110,7 +154,7 @@ def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode,
     _lib.check(rc, "mi355_prefill_fwd")
 
 
-def _dense(q, k, v, mask, mode, softmax_scale, want_lse=False):
+def _dense(q, k, v, mask, mode, softmax_scale, want_lse=False, kv_splits=1, workspace=None):
     for n, t in (("q", q), ("k", k), ("v", v)):
         _require_gpu_bf16(n, t)
         if t.dim() != 4:
@@ -131,7 +175,9 @@ def _dense(q, k, v, mask, mode, softmax_scale, want_lse=False):
         return (out, lse) if want_lse else out
     if Sk == 0:
         raise ValueError("attention over zero keys is undefined")
-    _prefill(q, k, v, out, None, None, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode, lse)
+    n_split, workspace = (1, None) if (want_lse or mask is not None) else _split_args(
+        kv_splits, workspace, B, Hq, D, Sq, Sk, B * Sq, mode == _lib.MASK_CAUSAL, q.device)
+    _prefill(q, k, v, out, None, None, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode, lse, n_split, workspace, B * Sq)
     return (out, lse) if want_lse else out
 
 
@@ -208,7 +254,7 @@ def _needs_grad(*tensors):
     return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
 
 
-def flash_attn_prefill(q, k, v, *, causal=True, softmax_scale=None):
+def flash_attn_prefill(q, k, v, *, causal=True, softmax_scale=None, kv_splits=None, workspace=None):
     """Prefill forward.  q (B,Hq,Sq,D); k, v (B,Hkv,Sk,D) -> (B,Hq,Sq,D).
 
     Fills the slot of torch.nn.functional.scaled_dot_product_attention(Q, K, V,
@@ -218,12 +264,17 @@ def flash_attn_prefill(q, k, v, *, causal=True, softmax_scale=None):
     float32 only for three float32 inputs outside autocast, bfloat16 otherwise).
     Differentiable: when an input requires grad, dq/dk/dv come from the HIP backward kernels
     (what autograd computes behind model.py:382 during train.py's loss.backward()).
+    kv_splits (forward-only calls): split every sequence's keys over that many workgroups and merge the
+    partial results (mi355_prefill_fwd_splitkv) -- for few query rows over many keys, where one workgroup
+    per pair of 256-row query tiles would leave most of the GPU idle.  None chooses (1 whenever the plain
+    launch already fills the GPU); `workspace` may carry a prefill_splitkv_workspace() tensor to reuse.
     """
     q, k, v, out_dtype = _to_bf16(q, k, v)
     if _needs_grad(q, k, v):
         out = _DensePrefillFn.apply(q, k, v, bool(causal), softmax_scale)
     else:
-        out = _dense(q, k, v, None, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, softmax_scale)
+        out = _dense(q, k, v, None, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, softmax_scale,
+                     kv_splits=kv_splits, workspace=workspace)
     return out if out.dtype == out_dtype else out.to(out_dtype)
 
 
@@ -277,11 +328,12 @@ def scaled_dot_product_attention(Q, K, V, mask=None):
         if m4.stride(-1) != 1:
             m4 = m4.contiguous()
         mode = _lib.MASK_BOOL
-    out = _dense(q4, k4, v4, m4, mode, None)
+    out = _dense(q4, k4, v4, m4, mode, None, kv_splits=None)
     return out.reshape(*lead, nq, d).to(out_dtype)
 
 
-def _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale, want_lse=False):
+def _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale, want_lse=False,
+            kv_splits=1, workspace=None):
     for n, t in (("q", q), ("k", k), ("v", v)):
         _require_gpu_bf16(n, t)
         if t.dim() != 3:
@@ -307,23 +359,27 @@ def _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, cau
     out = torch.empty(Tq, Hq, D, dtype=q.dtype, device=q.device)
     lse = torch.empty(Hq, Tq, dtype=torch.float32, device=q.device) if want_lse else None
     if Tq and max_seqlen_q:
+        n_split, workspace = (1, None) if want_lse else _split_args(
+            kv_splits, workspace, B, Hq, D, max_seqlen_q, max_seqlen_k, Tq, causal, q.device)
         _prefill(q, k, v, out, cu_seqlens_q, cu_seqlens_k, None, B, Hq, Hkv, int(max_seqlen_q), int(max_seqlen_k),
-                 D, scale, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, lse)
+                 D, scale, _lib.MASK_CAUSAL if causal else _lib.MASK_NONE, lse, n_split, workspace, Tq)
     return (out, lse) if want_lse else out
 
 
 def flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, *,
-                              causal=True, softmax_scale=None):
+                              causal=True, softmax_scale=None, kv_splits=None, workspace=None):
     """Packed ("varlen") prefill.  q (Tq,Hq,D); k, v (Tk,Hkv,D) bf16; cu_seqlens int32 (B+1,), cu[0]=0.
 
-    Sequence b owns rows [cu[b], cu[b+1]).  Returns (Tq,Hq,D) bf16.  Differentiable like flash_attn_prefill.
+    Sequence b owns rows [cu[b], cu[b+1]).  Returns (Tq,Hq,D) bf16.  Differentiable like flash_attn_prefill;
+    kv_splits / workspace as there.
     """
     q, k, v, out_dtype = _to_bf16(q, k, v)
     if _needs_grad(q, k, v):
         out = _VarlenPrefillFn.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, bool(causal),
                                      softmax_scale)
     else:
-        out = _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale)
+        out = _varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, softmax_scale,
+                      kv_splits=kv_splits, workspace=workspace)
     return out if out.dtype == out_dtype else out.to(out_dtype)
 
 
@@ -420,7 +476,7 @@ def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, s
 
 
 def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, context_lens, max_seqlen_q, *,
-                             softmax_scale=None, out=None):
+                             softmax_scale=None, out=None, max_context=None, kv_splits=None, workspace=None):
     """Causal prefill of a chunk of new tokens over context that already sits in a paged bf16 cache.
 
     q (T,Hq,D) bf16, packed, contiguous heads (token stride free): sequence b owns rows
@@ -428,6 +484,8 @@ def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, co
     context_lens[b] tokens of sequence b -- the chunk's own too (write them first with rope_and_cache) --
     addressed through block_tables (B,max_blocks) int32.  Query i of the chunk keeps key j iff
     j <= i + (context_lens[b] - chunk length).  max_seqlen_q = longest chunk.  Returns (T,Hq,D) bf16.
+    max_context bounds context_lens (default: what block_tables can address) and only guides the choice of
+    kv_splits (see flash_attn_prefill): a short chunk over a long context is split over many workgroups.
     The mathematics is that of llm-core/llm_core/model.py:308-325 with the mask of :384; the reference
     itself would re-run the whole prefix (model.py:218)."""
     _require_gpu_bf16("q", q)
@@ -470,11 +528,17 @@ def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, co
     if T == 0 or B == 0:
         return out
     scale = 1.0 / math.sqrt(D) if softmax_scale is None else softmax_scale
-    with _on(q, k_cache, v_cache, out, cu_seqlens_q, block_tables, context_lens) as stream:
+    if max_context is None:
+        max_context = block_tables.shape[1] * _BLOCK
+    n_split, workspace = _split_args(kv_splits, workspace, B, Hq, D, int(max_seqlen_q), int(max_context), T, True,
+                                     q.device)
+    with _on(q, k_cache, v_cache, out, cu_seqlens_q, block_tables, context_lens, workspace) as stream:
         rc = _lib.load().mi355_prefill_paged_fwd(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), q.stride(0), out.stride(0),
             cu_seqlens_q.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
-            B, Hq, Hkv, int(max_seqlen_q), D, _BLOCK, k_cache.shape[0], float(scale), _lib.MI355_BF16, stream)
+            B, Hq, Hkv, int(max_seqlen_q), D, _BLOCK, k_cache.shape[0], float(scale), _lib.MI355_BF16,
+            n_split, T, None if workspace is None else workspace.data_ptr(),
+            0 if workspace is None else workspace.numel() * workspace.element_size(), stream)
     _lib.check(rc, "mi355_prefill_paged_fwd")
     return out
 

@@ -83,6 +83,48 @@ def test_prefill_rejects_bad_arguments_without_a_gpu(lib):
     assert call(q=ptr + 2) == -1 and b"aligned" in lib.mi355_last_error()
 
 
+def test_prefill_split_keys_rejects_bad_arguments_without_a_gpu(lib):
+    s3 = _lib.strides3((8, 8, 8))
+    buf = C.create_string_buffer(64)
+    ptr = (C.addressof(buf) + 15) & ~15
+    need = lib.mi355_prefill_splitkv_workspace_bytes(8, 2, 64, 4)
+    assert need == 4 * 2 * 8 * (64 + 1) * 4
+    assert lib.mi355_prefill_splitkv_workspace_bytes(8, 2, 64, 1) == 0
+
+    def call(n_split=4, rows=8, ws=ptr, ws_bytes=need, mode=_lib.MASK_CAUSAL):
+        return lib.mi355_prefill_fwd_splitkv(ptr, ptr, ptr, ptr, s3, s3, s3, s3, None, None, 1, 2, 2, 8, 8, 64, 0.125,
+                                             mode, _lib.MI355_BF16, n_split, rows, ws, ws_bytes, None)
+
+    assert call(n_split=65) == -1 and b"n_split" in lib.mi355_last_error()
+    assert call(n_split=0) == -1
+    assert call(rows=7) == -1 and b"total_q_rows" in lib.mi355_last_error()
+    assert call(ws=None) == -1 and b"workspace" in lib.mi355_last_error()
+    assert call(ws=ptr + 4) == -1
+    assert call(ws_bytes=need - 1) == -2 and b"workspace" in lib.mi355_last_error()
+    assert call(mode=_lib.MASK_BOOL) == -1
+
+
+def test_suggested_key_splits_follow_the_measured_cases(lib):
+    """The cost model against timings taken on an MI355X (256 compute units): few query rows over many keys are
+    split, a launch that fills the GPU is not, and the suggestion never leaves a share fewer than two K/V tiles."""
+    def n(B, Hq, Sq, Sk, causal=1):
+        return lib.mi355_prefill_suggest_kv_splits(B, Hq, 128, Sq, Sk, B * Sq, causal, 256)
+
+    assert n(8, 32, 4096, 4096) == 1                    # configs[2]: 768 workgroups
+    assert n(1, 32, 2048, 2048) == 1                    # measured: 66 us unsplit, 81 us split in two
+    assert n(8, 32, 128, 2048) == 1                     # measured: 60 us unsplit, 85 us split in two
+    assert 6 <= n(1, 32, 256, 16384) <= 8               # measured best 8 (359 -> 85 us)
+    assert 6 <= n(1, 32, 256, 8192) <= 8                # measured best 8 (191 -> 57 us)
+    assert 3 <= n(1, 32, 1024, 8192) <= 4               # measured best 4 (352 -> 155 us)
+    assert 8 <= n(1, 8, 512, 16384) <= 24               # measured best 16 (711 -> 88 us)
+    assert 3 <= n(8, 8, 128, 2048) <= 4                 # measured best 4 (55 -> 32 us)
+    assert n(1, 8, 64, 32768) >= 16                     # measured best 32 (712 -> 67 us)
+    for Sq, Sk in ((1, 1), (64, 64), (256, 300), (100, 128)):
+        assert n(1, 1, Sq, Sk) == 1 and n(1, 1, Sq, Sk, causal=0) == 1
+    assert n(1, 1, 64, 100000, causal=0) == 64
+    assert lib.mi355_prefill_suggest_kv_splits(0, 8, 128, 64, 64, 0, 1, 256) == 1
+
+
 def test_decode_rejects_bad_arguments_without_a_gpu(lib):
     buf = C.create_string_buffer(64)
     ptr = C.addressof(buf)

@@ -284,12 +284,14 @@ def test_prefill_unmasked_head_dim_128_long_and_ragged(ops, Sq, Sk):
     B, Hq, Hkv, D = 2, 4, 2, 128
     q, k, v = rnd(B, Hq, Sq, D, seed=81, scale=0.5), rnd(B, Hkv, Sk, D, seed=82, scale=0.5), rnd(B, Hkv, Sk, D, seed=83, scale=0.5)
     ref = orc.prefill_reference(q, k, v, causal=False)
-    got = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=False)
+    got = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=False, kv_splits=1)
     torch.cuda.synchronize()
     check(got, ref, what=f"unmasked D128 {Sq}x{Sk}")
-    # the reference's own signature (no GQA there: first kv head only) lands on the same kernel
+    # the default may split the keys of so small a launch over several workgroups (another kernel and a merge)
+    check(ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=False), ref, what=f"unmasked D128 {Sq}x{Sk}, default")
+    # the reference's own signature (no GQA there: first kv head only)
     got2 = ops.scaled_dot_product_attention(q[:, :2].cuda(), k[:, :1].cuda(), v[:, :1].cuda())
-    assert torch.equal(got[:, :2], got2)
+    check(got2, ref[:, :2], what=f"unmasked D128 {Sq}x{Sk}, reference signature")
 
 
 def test_prefill_unmasked_scores_that_outgrow_the_reference(ops):
@@ -312,6 +314,78 @@ def test_prefill_unmasked_scores_that_outgrow_the_reference(ops):
     # the same through the 8-wavefront kernel (an all-true explicit mask takes that path): both must agree with the oracle
     keep = torch.ones(Sq, Sk, dtype=torch.bool, device="cuda")
     check(ops.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), keep), ref, what="reference moves, masked path")
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("splits", [2, 5, 64])
+def test_prefill_split_keys_dense(ops, D, splits):
+    """Every sequence's keys split over several workgroups whose fp32 partial rows a second kernel merges: causal
+    (early rows see no key of the later shares: those partials are empty), rectangular, unmasked, GQA, more shares
+    than K/V tiles, a ragged last query tile."""
+    print(f"case: prefill split keys D={D} splits={splits}", flush=True)
+    B, Hq, Hkv, Sq, Sk = 2, 4, 2, 333, 1500
+    q, k, v = rnd(B, Hq, Sq, D, seed=91, scale=0.5), rnd(B, Hkv, Sk, D, seed=92, scale=0.5), rnd(B, Hkv, Sk, D, seed=93, scale=0.5)
+    for causal in (True, False):
+        ref = orc.prefill_reference(q, k, v, causal=causal)
+        got = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=causal, kv_splits=splits)
+        torch.cuda.synchronize()
+        check(got, ref, what=f"split keys D{D} x{splits} causal={causal}")
+    # square causal: the first query tile's later shares hold no tile at all
+    ref = orc.prefill_reference(q, k[:, :, :Sq], v[:, :, :Sq], causal=True)
+    ws = ops.prefill_splitkv_workspace(B * Sq, Hq, D, splits, "cuda:0")
+    got = ops.flash_attn_prefill(q.cuda(), k[:, :, :Sq].cuda(), v[:, :, :Sq].cuda(), causal=True, kv_splits=splits, workspace=ws)
+    check(got, ref, what=f"split keys square D{D} x{splits}")
+
+
+def test_prefill_split_keys_is_chosen_for_few_long_sequences(ops):
+    """A chunk of one prompt over a long context (one workgroup per pair of query tiles would occupy 8 of 256
+    compute units): the default splits the keys; the result agrees with the unsplit kernel to rounding and with
+    the oracle to tolerance."""
+    print("case: prefill split keys, automatic", flush=True)
+    B, Hq, Hkv, Sq, Sk, D = 1, 8, 2, 512, 4096, 128
+    q, k, v = rnd(B, Hq, Sq, D, seed=94, scale=0.5), rnd(B, Hkv, Sk, D, seed=95, scale=0.5), rnd(B, Hkv, Sk, D, seed=96, scale=0.5)
+    assert ops.suggest_kv_splits(B, Hq, D, Sq, Sk, B * Sq, True, torch.device("cuda:0")) > 1
+    ref = orc.prefill_reference(q, k, v, causal=True)
+    auto = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=True)
+    one = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=True, kv_splits=1)
+    torch.cuda.synchronize()
+    check(auto, ref, what="auto split")
+    check(one, ref, what="unsplit")
+    assert not torch.equal(auto, one)            # (another kernel, another order of summation)
+    assert (auto.float() - one.float()).abs().max().item() <= 2e-2
+    with pytest.raises(ValueError):
+        ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=True, kv_splits=65)
+
+
+@pytest.mark.parametrize("splits", [3, 16])
+def test_prefill_split_keys_varlen_and_paged(ops, splits):
+    """Packed sequences of ragged lengths (one of them empty of keys for some shares, one a single token) and chunks
+    over a paged cache, keys split."""
+    print(f"case: prefill split keys varlen/paged splits={splits}", flush=True)
+    Hq, Hkv, D = 8, 2, 128
+    lens = [1000, 3, 517, 1]
+    T = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q, k, v = rnd(T, Hq, D, seed=97, scale=0.5), rnd(T, Hkv, D, seed=98, scale=0.5), rnd(T, Hkv, D, seed=99, scale=0.5)
+    ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True)
+    got = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens),
+                                        causal=True, kv_splits=splits)
+    check(got, ref, what="split keys varlen")
+
+    ctx = [700, 391, 64, 1500, 17, 300]
+    chunk = [203, 391, 1, 1, 17, 299]
+    _, kc, vc, bt, cl = orc.make_paged_case(batch=len(ctx), n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                            context_lens=ctx, pool_factor=1.3, seed=23, dtype=torch.bfloat16)
+    cu = torch.tensor([0] + list(torch.tensor(chunk).cumsum(0)), dtype=torch.int32)
+    q = rnd(int(cu[-1]), Hq, D, seed=24)
+    ref = orc.paged_prefill_reference(q, kc, vc, cu, bt, cl)
+    dev = "cuda:0"
+    got = ops.flash_attn_paged_prefill(q.to(dev), kc.to(dev), vc.to(dev), cu.to(dev), bt.to(dev), cl.to(dev), max(chunk),
+                                       kv_splits=splits)
+    check(got, ref, what="split keys paged")
+    unsplit = ops.flash_attn_paged_prefill(q.to(dev), kc.to(dev), vc.to(dev), cu.to(dev), bt.to(dev), cl.to(dev),
+                                           max(chunk), kv_splits=1)
+    assert (got.float() - unsplit.float()).abs().max().item() <= 2e-2
 
 
 def _reference_module_tensors(x_proj, freq, num_heads, amp):
