@@ -2,76 +2,96 @@
 """Writes prefill_w64_asm.inc: the hand-scheduled tile loop of prefill_fwd_w64.hip as inline-assembly text.
 
 Why assembly: with one wavefront per SIMD and 64 query columns per wavefront the output accumulators (128 registers)
-must live in AGPRs while the score accumulators must live in VGPRs (the exponentials read them), and the vector and
-LDS instructions must sit in the shadow of the MFMAs at a fixed rhythm.  The compiler offers neither (it picks one
-register form for every MFMA of a function and clusters the vector work), so the loop over the K/V tiles of a query
-tile is generated here, instruction by instruction, and included by the kernel as a string.  What stays ordinary HIP
-C++: prologue, epilogue, ragged ends, and the rare tile in which a row maximum outgrows its exponent reference.
+and the query fragments (64) must live in AGPRs while the score accumulators must live in VGPRs (the exponentials read
+them), and the vector and LDS instructions must sit in the shadow of the MFMAs at a fixed rhythm.  The compiler offers
+neither (it picks one register form for every MFMA of a function and clusters the vector work), so the loop over the
+K/V tiles of a query tile is generated here, instruction by instruction, and included by the kernel as a string.
+What stays ordinary HIP C++: prologue, epilogue, ragged ends, and moving a row's exponent reference.
 
-One tile (64 keys) of one wavefront (64 queries = column blocks A and B, head_dim 128):
-  phase 1   S(.,0) = K[0:32] . Q^T               16 MFMA 32x32x16 (8 per block), K fragments one step ahead
-  phase 2   S(.,1) = K[32:64] . Q^T              16 MFMA | P(.,0) = bf16(2^(S(.,0) * scale + nb)): 32 v_fma, 32 v_exp,
-                                                           16 cvt, 8 or3 (a masked tile adds a compare and a select
-                                                           per score: key index against a per-lane threshold)
-  check     some weight >= 2 (top exponent bit of its bf16 pattern)?  -> leave, status 1 (nothing of the tile accumulated)
-  phase 3   O += V[0:32]^T . P(.,0), l += sums   16 MFMA + 4 row-sum MFMA 16x16x32 | P(.,1) likewise from S(.,1)
-  check     -> leave, status 2 (keys 0..31 of the tile are accumulated, 32..63 are not)
-  phase 4a  O += V[32:48]^T . P(.,1)             8 + 2 MFMA (fragments already in registers)
-  hand-over every wavefront is done reading the tile; the next tile has landed; the tile after it is requested
-            (direct-to-LDS loads into the buffer just freed) and the next tile's first K fragments are read
-  phase 4b  O += V[48:64]^T . P(.,1)             8 + 2 MFMA: covers the latency of those reads
+One tile = 64 keys; a wavefront owns 64 queries = column blocks A and B of 32; head_dim 128.  Per 32-key half h of
+tile t there are three pieces of work (each for both blocks):
+  S(t,h)  scores   = K[t][32h:32h+32] . Q^T         16 MFMA 32x32x16 (8 per block), K fragments from LDS
+  E(t,h)  weights  = bf16(2^(S * scale + nb))       32 v_fma, 32 v_exp, 16 cvt, 8 or3 (a masked tile adds a compare
+                                                    and a select per score)
+  O(t,h)  O^T     += V[t][32h:32h+32]^T . P, l += row sums   16 MFMA + 4 row-sum MFMA 16x16x32, V^T fragments from LDS
+With one wavefront per SIMD the vector work of a half hides only behind MFMAs of the same wavefront that do not
+depend on it.  Unmasked tiles therefore run as a software pipeline across tiles, two half-steps per tile:
+  H0(t):  S(t,1)   | E(t,0) | O(t-1,1)
+  H1(t):  S(t+1,0) | E(t,1) | O(t,0)
+so every half-step carries 36 MFMAs and one half's vector work.  The pipeline is filled by a prologue (S(t,0), then
+H0 without its O part) and emptied by an epilogue (H1 without its S part, then O(t,1)).  Masked tiles (the causal
+diagonal) run one at a time: S(t,0); S(t,1) | E(t,0); O(t,0) | E(t,1); O(t,1).
+
+Tile hand-over ("boundary") -- the protocol every wavefront of the workgroup follows once per tile, here and in the
+C++ steps of the kernel.  K[t] and V[t] live in LDS buffers t % 2 (one pair of buffers for K, one for V).
+  when tile t starts: K[t] has landed and the workgroup has met since; K[t+1] and V[t] are in flight
+  boundary(t):        this wavefront has read all it needs of K[t] and V[t-1]; it waits for its own shares of
+                      K[t+1] and V[t], meets the others at a barrier, and requests K[t+2] and V[t+1] into the
+                      buffers just freed
+  afterwards:         it reads V[t] (and K[t+1])
+In the pipeline the boundary sits inside H0(t), behind three quarters of its MFMAs; the last quarter (whose
+fragments are in registers by then) covers the latency of the first reads of K[t+1] and V[t], and the requests are
+issued between its MFMAs.
+
+Weights are 2^(score * scale + nb) with nb preset by the caller (see the kernel); nothing here looks at row maxima.
+Each tile ORs its packed weights together, and a weight >= 2 (top exponent bit of a bf16 pattern) ends the block
+after that tile with status 1: the caller lowers nb of the rows that need it, rescales, and re-enters.
+
 Tiles come in three kinds, by index: [0, n_plain) every key visible to every query; [n_plain, n_mask) masked (causal
 diagonal: key <= threshold of the lane's query; the threshold moves down by 64 per tile); [n_mask, n_end) nothing
-visible for this wavefront -- it only takes part in the hand-over.  When the diagonal is aligned with the tiles
+visible for this wavefront -- it only takes part in the boundary.  When the diagonal is aligned with the tiles
 (operand `aligned`: query i of the wavefront sees key j of the one masked tile iff j <= i) that tile takes a cheaper
 body: only the two triangular 32x32 sub-blocks get mask code, and the invisible one is neither scored nor accumulated.
 
 Register map (physical, fixed; the block loads them itself from its operands, see entry()):
-  v[0:31] Q^T fragments of block A (step s = v[4s:4s+3]), v[32:63] block B
-  v[64:95]  S(A,0), S(B,0); dead after the first check: v[64:79] then hold P(.,1), v[80:95] V^T fragments
-  v[96:127] S(A,1), S(B,1)
-  v128 / v129 nb (the additive term of the exponent) of this lane's query in block A / B
-  v130 -inf, v131 / v132 mask threshold of the lane's query in block A / B (key index inside the tile, minus 4*(lane/32))
-  v[134:149] P(.,0): A slices 0,1 then B slices 0,1
-  v[150:165] K fragments (4 in flight), v[166:181] V^T fragments (4 d-tiles of one 16-key slice)
-  v[182:185] A operand of the row-sum MFMA
-  v[186:193] K fragment LDS addresses per step, v[194:201] V^T LDS addresses [half][d-tile] (both for buffer 0; the
+  v[0:31]   S(A,0), S(B,0)     v[32:63]  S(A,1), S(B,1)
+  v[64:79]  P(.,0): A slices 0,1 then B slices 0,1 (a slice = 16 keys = 4 registers)     v[80:95] P(.,1)
+  v[96:111] K fragments (4 in flight)    v[112:143] V^T fragments (8: 2 slices x 4 d-tiles)
+  v144 / v145 nb (the additive term of the exponent) of this lane's query in block A / B
+  v146 -inf, v147 / v148 mask threshold of the lane's query in block A / B (key index inside the tile, minus 4*(lane/32))
+  v[150:153] A operand of the row-sum MFMA
+  v[154:161] K fragment LDS addresses per step, v[162:169] V^T LDS addresses [half][d-tile] (both for buffer 0; the
   buffer and the position inside the tile are immediates; V tiles sit two tile sizes behind the K tiles),
-  v[202:209] lane offsets of the direct-to-LDS loads (K steps 0..3, V steps 0..3)
+  v[170:177] lane offsets of the direct-to-LDS loads (K steps 0..3, V steps 0..3)
   twelve more registers, wherever the compiler puts the block's vector operands: after entry() they serve as scratch
   (collected weight bits, exponentials on their way to packing)
   a[0:63] O^T of block A (d-tile dt = a[16dt:16dt+15]), a[64:127] block B, a[128:131] / a[132:135] row sums:
   these live in the AGPRs for a whole query tile and are touched only by the assembly snippets below (the kernel
   is compiled with its builtin MFMAs in VGPR form, so the compiler has no use for AGPRs of its own)
-  s[36:37] / s[38:39] global address of the wavefront's first DMA row of the K / V tile after next (advanced per tile),
-  s[40:41] scratch; every other scalar is a named operand
+  a[136:167] Q^T fragments of block A (step s = a[136+4s:139+4s]), a[168:199] block B: loaded by entry()
+  s[36:37] / s[38:39] global address of the wavefront's first DMA row of K[t+2] / V[t+1] (advanced per tile),
+  s[40:41] scratch, s42 "a weight reached 2"; every other scalar is a named operand
 """
 import os
 
-ABL = os.environ.get("W64_ABL", "").split(",")       # timing experiments only (results wrong): nobarrier, nodma, nocheck
+# timing experiments only (results wrong): nobarrier, nodma, nocheck, noexp, novalu, nosum
+ABL = os.environ.get("W64_ABL", "").split(",")
 
-QA, QB = 0, 32
-S = {("A", 0): 64, ("B", 0): 80, ("A", 1): 96, ("B", 1): 112}
-NB = {"A": 128, "B": 129}
-NEGINF = 130
-THR = {"A": 131, "B": 132}
-PW0 = {"A": 134, "B": 142}          # + 4*slice
-PW1 = {"A": 64, "B": 72}            # aliases S(A,0)
-VF1 = 80                            # aliases S(B,0): 4 d-tiles x 4 registers
-KF = 150
-VF0 = 166
-SUMA = 182
-KOFF, VOFF, DMAOFF = 186, 194, 202
-N_FIXED_VGPRS = 210
+EXP = "v_mov_b32" if "noexp" in ABL else "v_exp_f32"
+S = {("A", 0): 0, ("B", 0): 16, ("A", 1): 32, ("B", 1): 48}
+P = {0: {"A": 64, "B": 72}, 1: {"A": 80, "B": 88}}          # + 4 * slice inside the half
+KF = 96
+VF = 112                            # fragment j (slice j // 4 of the half, d-tile j % 4) at VF + 4j
+NB = {"A": 144, "B": 145}
+NEGINF = 146
+THR = {"A": 147, "B": 148}
+SUMA = 150                          # (register tuples of MFMA operands start at even registers)
+KOFF, VOFF, DMAOFF = 154, 162, 170
+N_FIXED_VGPRS = 178
 # Scratch registers are the block's vector operands themselves: each is read once by entry() and is free from then on
-# (the operands are declared in/out), so the block needs no register beyond v[0:209] and its operands.
+# (the operands are declared in/out), so the block needs no register beyond v[0:177] and its operands.
 ETMP = ["%[nb0]", "%[nb1]", "%[suma]", "%[k0]", "%[vlo0]", "%[vhi0]", "%[rowk]", "%[rowv]"]   # exponentials on their way to packing
 ANY, TMP = "%[c0s]", "%[qaddr]"     # collected weight bits; scratch
-OA, OB, LA, LB = 0, 64, 128, 132
-KPTR, VPTR, PTMP = 36, 38, 40       # SGPR pairs: global address of this wavefront's share of the tile after next (K, V); scratch
+OREG = {"A": 0, "B": 64}
+LREG = {"A": 128, "B": 132}
+QREG = {"A": 136, "B": 168}
+N_ACC = 136                         # a[0:135]: what ordinary code reaches through the snippets
+N_AGPRS = 200
+KPTR, VPTR, PTMP, FLAG = 36, 38, 40, 42
 Q_SLAB_ROW = 272                    # bytes per row of the query staging slab (256 + 16 of padding)
 K_TILE = 16384                      # bytes of one K (or V) tile in LDS: 64 rows x 256 bytes
 ROW = 256
+NONE = {"A": False, "B": False}
 
 
 def rng(base, n):
@@ -113,137 +133,184 @@ class Emitter:
             self.pending = []
 
 
-def mfma32_v(dst, a, b, c):
-    cs = "0" if c is None else f"v{rng(c, 16)}"
-    return f"v_mfma_f32_32x32x16_bf16 v{rng(dst, 16)}, v{rng(a, 4)}, v{rng(b, 4)}, {cs}"
+def mfma_s(c, h, slot, s):
+    """S(c,h) (+)= K fragment in `slot` . Q^T fragment of step s."""
+    dst = S[(c, h)]
+    cs = "0" if s == 0 else f"v{rng(dst, 16)}"
+    return f"v_mfma_f32_32x32x16_bf16 v{rng(dst, 16)}, v{rng(KF + 4 * slot, 4)}, a{rng(QREG[c] + 4 * s, 4)}, {cs}"
 
 
-def mfma32_a(acc, a, b):
-    return f"v_mfma_f32_32x32x16_bf16 a{rng(acc, 16)}, v{rng(a, 4)}, v{rng(b, 4)}, a{rng(acc, 16)}"
+def mfma_o(c, j, p):
+    """O^T(c, d-tile j % 4) += V^T fragment j . P words at p."""
+    acc = OREG[c] + 16 * (j % 4)
+    return f"v_mfma_f32_32x32x16_bf16 a{rng(acc, 16)}, v{rng(VF + 4 * j, 4)}, v{rng(p, 4)}, a{rng(acc, 16)}"
 
 
-def mfma16_a(acc, a, b):
-    return f"v_mfma_f32_16x16x32_bf16 a{rng(acc, 4)}, v{rng(a, 4)}, v{rng(b, 4)}, a{rng(acc, 4)}"
+def mfma_sum(c, p):
+    if "nosum" in ABL:
+        return "s_nop 0"
+    acc = LREG[c]
+    return f"v_mfma_f32_16x16x32_bf16 a{rng(acc, 4)}, v{rng(SUMA, 4)}, v{rng(p, 4)}, a{rng(acc, 4)}"
 
 
-def k_read(e, buf, t, s, slot):
-    e.lds_read(f"ds_read_b128 v{rng(KF + 4 * slot, 4)}, v{KOFF + s} offset:{buf * K_TILE + t * 32 * ROW}", KF + 4 * slot)
+def k_read(e, buf, h, s, slot):
+    e.lds_read(f"ds_read_b128 v{rng(KF + 4 * slot, 4)}, v{KOFF + s} offset:{buf * K_TILE + h * 32 * ROW}", KF + 4 * slot)
 
 
-def v_read(e, buf, u, dt, base):
-    """V^T fragment of 16-key slice u, d-tile dt into registers base..base+3 (two transposed 64-bit reads)."""
-    off = buf * K_TILE + 16 * u * ROW
+def v_read(e, buf, h, j):
+    """V^T fragment j of half h (16-key slice 2h + j // 4, d-tile j % 4) into its registers (two transposed 64-bit reads)."""
+    off = buf * K_TILE + 16 * (2 * h + j // 4) * ROW
+    base, dt = VF + 4 * j, j % 4
     e.lds_read(f"ds_read_b64_tr_b16 v{rng(base, 2)}, v{VOFF + dt} offset:{off}", base)
     e.lds_read(f"ds_read_b64_tr_b16 v{rng(base + 2, 2)}, v{VOFF + 4 + dt} offset:{off}", base + 2)
 
 
-def exp_ops(t, dst, mask, blocks="AB"):
-    """Vector work that turns S(c,t), c in `blocks`, into packed bf16 weights in dst[c] (+ slice * 4).  The result of
-    a transcendental may not feed the next vector instruction, so the packing of a pair trails its exponentials.
-    Accumulator register i of a lane holds key 32t + 8(i/4) + 4(lane/32) + i%4 of the tile; where mask[c] is set the
-    score is kept only if that index is <= the lane's threshold (the lane part of the index is folded into the
-    threshold)."""
+def vneeds(j):
+    return (VF + 4 * j, VF + 4 * j + 2)
+
+
+def exp_ops(h, mask, blocks="AB"):
+    """Vector work that turns S(c,h), c in `blocks`, into packed bf16 weights P(c,h).  The result of a transcendental
+    may not feed the next vector instruction, so the packing of a pair trails its exponentials.  Accumulator register
+    i of a lane holds key 32h + 8(i/4) + 4(lane/32) + i%4 of the tile; where mask[c] is set the score is kept only if
+    that index is <= the lane's threshold (the lane part of the index is folded into the threshold)."""
+    if "novalu" in ABL:
+        return []
     ops, pend = [], []
     i = 0
     for c in blocks:
+        dst = P[h][c]
         for w in range(8):                      # packed word w of the block: accumulator registers 2w, 2w+1
             t0, t1 = ETMP[2 * (i % 4)], ETMP[2 * (i % 4) + 1]
             for tmp, r in ((t0, 2 * w), (t1, 2 * w + 1)):
-                ops.append(f"v_fma_f32 {tmp}, v{S[(c, t)] + r}, %[scale], v{NB[c]}")
+                ops.append(f"v_fma_f32 {tmp}, v{S[(c, h)] + r}, %[scale], v{NB[c]}")
                 if mask[c]:
-                    ops.append(f"v_cmp_le_i32_e64 vcc, {32 * t + 8 * (r // 4) + r % 4}, v{THR[c]}")
+                    ops.append(f"v_cmp_le_i32_e64 vcc, {32 * h + 8 * (r // 4) + r % 4}, v{THR[c]}")
                     ops.append(f"v_cndmask_b32 {tmp}, v{NEGINF}, {tmp}, vcc")
-            ops.append(f"v_exp_f32 {t0}, {t0}")
-            ops.append(f"v_exp_f32 {t1}, {t1}")
+            ops.append(f"{EXP} {t0}, {t0}")
+            ops.append(f"{EXP} {t1}, {t1}")
             ops += pend
-            pend = [f"v_cvt_pk_bf16_f32 v{dst[c] + w}, {t0}, {t1}"]
+            pend = [f"v_cvt_pk_bf16_f32 v{dst + w}, {t0}, {t1}"]
             if w % 2 == 1:
-                pend.append(f"v_or3_b32 {ANY}, {ANY}, v{dst[c] + w - 1}, v{dst[c] + w}")
+                pend.append(f"v_or3_b32 {ANY}, {ANY}, v{dst + w - 1}, v{dst + w}")
             i += 1
     ops += ["s_nop 0"] + pend
     return ops
 
 
-def spread(e, mfmas, valu, hold=0):
-    """Emit the MFMAs in order with the vector instructions spread evenly behind them, none behind the first
-    `hold` MFMAs: the vector work reads accumulators that the MFMAs just before this phase wrote, and the hardware
-    does not interlock that dependency (a result is visible 8 passes after its MFMA started; `hold` MFMAs of other
-    chains in between cover that).  `mfmas` entries are (text, needs, post): registers whose LDS reads must have
-    returned, and a callback run right after the MFMA (it issues the LDS reads that refill the registers the MFMA
-    has just consumed)."""
+def plan(mfmas, valu, hold=0):
+    """Distributes the vector instructions evenly behind the MFMAs, none behind the first `hold` MFMAs: the vector
+    work reads accumulators that the MFMAs just before it wrote, and the hardware does not interlock that dependency
+    (a result is visible 8 passes after its MFMA started; `hold` MFMAs of other chains in between cover that).
+    `mfmas` entries are (text, needs, post): registers whose LDS reads must have returned, and a callback run right
+    after the MFMA (it issues the LDS reads that refill the registers the MFMA has just consumed).
+    Returns entries (text, needs, post, vector instructions that follow)."""
     n, nv, vi = len(mfmas), len(valu), 0
+    out = []
     for i, (text, needs, post) in enumerate(mfmas):
+        upto = (i + 1 - hold) * nv // (n - hold) if i >= hold else 0
+        out.append((text, needs, post, valu[vi:upto]))
+        vi = max(vi, upto)
+    assert vi == nv
+    return out
+
+
+def emit(e, entries, extras=()):
+    """Emits planned entries; `extras` (groups of instructions that must stay together, e.g. the m0 write and its
+    direct-to-LDS load) are spread evenly behind the MFMAs as well."""
+    extras = list(extras)
+    n, ne, xi = len(entries), len(extras), 0
+    for i, (text, needs, post, valu) in enumerate(entries):
         if needs:
             e.need(*needs)
         e.raw(text)
         if post:
             post()
-        upto = (i + 1 - hold) * nv // (n - hold) if i >= hold else 0
-        while vi < upto:
-            e.raw(valu[vi])
-            vi += 1
+        for v in valu:
+            e.raw(v)
+        upto = (i + 1) * ne // n
+        while xi < upto:
+            for x in extras[xi]:
+                e.raw(x)
+            xi += 1
 
 
-def check(e, label):
+def check_weights(e, flagged_label):
+    """End of a tile: did one of its weights reach 2?  Then control goes to `flagged_label`."""
     e.raw(f"v_and_b32 {TMP}, 0x40004000, {ANY}")
     e.raw(f"v_cmp_ne_u32 vcc, 0, {TMP}")
     e.raw(f"v_mov_b32 {ANY}, 0")
     e.raw("s_nop 1")
     if "nocheck" not in ABL:
-        e.raw(f"s_cbranch_vccnz {label}")
+        e.raw(f"s_cbranch_vccnz {flagged_label}")
 
 
-def hand_over(e, buf, tag):
-    """End of the LDS reads of the tile in buffer `buf`: count the tile, meet the other wavefronts once the own share
-    of the next tile has landed, request the tile after next into this buffer, read the next tile's first K fragments."""
-    nxt = buf ^ 1
-    e.raw("; tile hand-over")
+def dma_chunks(which, buf):
+    """Instruction groups that request K[t+2] into K buffer `buf` ("k" in which) and V[t+1] into V buffer buf ^ 1
+    ("v" in which), and advance the pointers by a tile."""
+    chunks = []
+    for name, j0, ptr, lds0 in (("v", 4, VPTR, 2 * K_TILE + (buf ^ 1) * K_TILE), ("k", 0, KPTR, buf * K_TILE)):
+        if name not in which:
+            continue
+        chunks.append([f"s_mov_b64 s[{PTMP}:{PTMP + 1}], s[{ptr}:{ptr + 1}]"])
+        for j in range(4):
+            c = [f"s_add_u32 m0, %[ldsdst], {lds0 + j * 1024}", "s_nop 0"]
+            if "nodma" not in ABL:
+                c.append(f"global_load_lds_dwordx4 v{DMAOFF + j0 + j}, s[{PTMP}:{PTMP + 1}]")
+            if j < 3:
+                c += [f"s_add_u32 s{PTMP}, s{PTMP}, %[{name}step]", f"s_addc_u32 s{PTMP + 1}, s{PTMP + 1}, 0"]
+            chunks.append(c)
+        chunks.append([f"s_lshl_b32 %[t2], %[{name}step], 4",          # a tile is 64 rows = 16 DMA steps of 4 rows
+                       f"s_add_u32 s{ptr}, s{ptr}, %[t2]",
+                       f"s_addc_u32 s{ptr + 1}, s{ptr + 1}, 0"])
+    return chunks
+
+
+def wait_and_meet(e):
+    """First half of a boundary: all LDS reads of this wavefront have returned, its shares of K[t+1] and V[t] have
+    landed, and every wavefront of the workgroup is here."""
+    e.raw("; boundary")
     e.drain()
-    e.raw("s_add_u32 %[tile], %[tile], 1")
-    e.raw("s_cmp_ge_u32 %[tile], %[n_tiles]")          # no next tile: nothing to wait for, nobody to meet
-    e.raw(f"s_cbranch_scc1 7{tag}f")
     e.raw("s_waitcnt vmcnt(0)")
     if "nobarrier" not in ABL:
         e.raw("s_barrier")
+
+
+def boundary_plain(e, buf, tag, after):
+    """A whole boundary with nothing to interleave: the requests are jumped over when their tiles do not exist.
+    `after` emits what follows the barrier and precedes the requests (LDS reads of the data that has just landed)."""
+    wait_and_meet(e)
+    after()
     e.raw("s_add_u32 %[t2], %[tile], 1")
     e.raw("s_cmp_ge_u32 %[t2], %[n_tiles]")
+    e.raw(f"s_cbranch_scc1 6{tag}f")                       # no tile t+1: nothing to request
+    for c in dma_chunks("v", buf):
+        for x in c:
+            e.raw(x)
+    e.raw("s_add_u32 %[t2], %[tile], 2")
+    e.raw("s_cmp_ge_u32 %[t2], %[n_tiles]")
     e.raw(f"s_cbranch_scc1 6{tag}f")
-    for name, j0, ptr, lds0 in (("k", 0, KPTR, 0), ("v", 4, VPTR, 2 * K_TILE)):
-        e.raw(f"s_mov_b64 s[{PTMP}:{PTMP + 1}], s[{ptr}:{ptr + 1}]")
-        for j in range(4):
-            e.raw(f"s_add_u32 m0, %[ldsdst], {lds0 + buf * K_TILE + j * 1024}")
-            e.raw("s_nop 0")
-            if "nodma" not in ABL:
-                e.raw(f"global_load_lds_dwordx4 v{DMAOFF + j0 + j}, s[{PTMP}:{PTMP + 1}]")
-            if j < 3:
-                e.raw(f"s_add_u32 s{PTMP}, s{PTMP}, %[{name}step]")
-                e.raw(f"s_addc_u32 s{PTMP + 1}, s{PTMP + 1}, 0")
-        e.raw(f"s_lshl_b32 %[t2], %[{name}step], 4")          # a tile is 64 rows = 16 DMA steps of 4 rows
-        e.raw(f"s_add_u32 s{ptr}, s{ptr}, %[t2]")
-        e.raw(f"s_addc_u32 s{ptr + 1}, s{ptr + 1}, 0")
+    for c in dma_chunks("k", buf):
+        for x in c:
+            e.raw(x)
     e.raw(f"6{tag}:")
-    for s in range(4):
-        k_read(e, nxt, 0, s, s)
-    e.raw(f"7{tag}:")
 
 
-KINDS = {"plain": 0, "masked": 1, "diag": 3}
+KINDS = {"masked": 1, "diag": 3}
 
 
-def tile_body(e, buf, kind):
-    """kind: "plain" no mask; "masked" every score against its threshold; "diag" the tile on an ALIGNED causal
-    diagonal (query i of the wavefront sees key j of the tile iff j <= i): S(A,0) and S(B,1) are triangular, S(B,0)
-    is fully visible, and S(A,1) is not computed at all -- block A neither scores nor accumulates keys 32..63."""
+def single_tile(e, buf, kind, start):
+    """A masked tile on its own (no pipelining across tiles).  kind: "masked" every score against its threshold;
+    "diag" the tile on an ALIGNED causal diagonal (query i of the wavefront sees key j of the tile iff j <= i):
+    S(A,0) and S(B,1) are triangular, S(B,0) is fully visible, and S(A,1) is not computed at all -- block A neither
+    scores nor accumulates keys 32..63.  Arrives with K fragments 0..3 of half 0 in flight; leaves likewise for the
+    next tile."""
     tag = f"{buf}{KINDS[kind]}"
     diag = kind == "diag"
-    t1_blocks = "B" if diag else "AB"
-    mask0 = {"A": kind != "plain", "B": kind == "masked"}
-    mask1 = {"A": kind == "masked", "B": kind != "plain"}
-    qreg = {"A": QA, "B": QB}
-    oreg = {"A": OA, "B": OB}
-    lreg = {"A": LA, "B": LB}
-    # ---- phase 1: scores of keys 0..31.  K fragments 0..3 of this tile are in flight (or in registers) ----
-    e.raw(f"; ---- {kind} tile in buffer {buf}: phase 1")
+    h1_blocks = "B" if diag else "AB"
+    mask0 = {"A": True, "B": kind == "masked"}
+    mask1 = {"A": kind == "masked", "B": True}
+    e.raw(f"; ---- {kind} tile in buffers {buf}: S(.,0)")
     m = []
     for s in range(8):
         slot = s % 4
@@ -253,11 +320,10 @@ def tile_body(e, buf, kind):
                 k_read(e, buf, 0, s + 4, slot)
             else:
                 k_read(e, buf, 1, s - 4, slot)
-        m.append((mfma32_v(S[("A", 0)], KF + 4 * slot, QA + 4 * s, None if s == 0 else S[("A", 0)]), (KF + 4 * slot,), None))
-        m.append((mfma32_v(S[("B", 0)], KF + 4 * slot, QB + 4 * s, None if s == 0 else S[("B", 0)]), None, refill))
-    spread(e, m, [])
-    # ---- phase 2: scores of keys 32..63 | weights of keys 0..31; V^T fragments of slice 0 requested ----
-    e.raw("; phase 2")
+        m.append((mfma_s("A", 0, slot, s), (KF + 4 * slot,), None))
+        m.append((mfma_s("B", 0, slot, s), None, refill))
+    emit(e, plan(m, []))
+    e.raw("; S(.,1) | E(.,0)")
     m = []
     for s in range(8):
         slot = s % 4
@@ -265,58 +331,198 @@ def tile_body(e, buf, kind):
         def refill(s=s, slot=slot):
             if s < 4:
                 k_read(e, buf, 1, s + 4, slot)
-            else:
-                dt = s - 4
-                v_read(e, buf, 0, dt, VF0 + 4 * dt)
-        for ci, c in enumerate(t1_blocks):
-            m.append((mfma32_v(S[(c, 1)], KF + 4 * slot, qreg[c] + 4 * s, None if s == 0 else S[(c, 1)]),
-                      (KF + 4 * slot,) if ci == 0 else None, refill if ci == len(t1_blocks) - 1 else None))
-    spread(e, m, exp_ops(0, PW0, mask0), hold=1 if diag else 3)
-    check(e, "91f")
-    # ---- phase 3: values of keys 0..31 | weights of keys 32..63 ----
-    e.raw("; phase 3")
-    e.need(VF0, VF0 + 2)                         # (keeps the number of reads in flight countable)
-    for dt in range(4):                          # slice 1 goes into the registers S(B,0) has just vacated
-        v_read(e, buf, 1, dt, VF1 + 4 * dt)
+        for ci, c in enumerate(h1_blocks):
+            m.append((mfma_s(c, 1, slot, s), (KF + 4 * slot,) if ci == 0 else None,
+                      refill if ci == len(h1_blocks) - 1 else None))
+    emit(e, plan(m, exp_ops(0, mask0), hold=1 if diag else 3))
+
+    def first_v_reads():
+        for j in range(8):
+            v_read(e, buf, 0, j)
+    boundary_plain(e, buf, tag, first_v_reads)
+    e.raw("; O(.,0) | E(.,1)")
     m = []
-    for u, vf in ((0, VF0), (1, VF1)):
-        m.append((mfma16_a(LA, SUMA, PW0["A"] + 4 * u), None, None))
-        m.append((mfma16_a(LB, SUMA, PW0["B"] + 4 * u), None, None))
-        for dt in range(4):
-            def refill(u=u, dt=dt, vf=vf):
-                v_read(e, buf, u + 2, dt, vf + 4 * dt)
-            m.append((mfma32_a(OA + 16 * dt, vf + 4 * dt, PW0["A"] + 4 * u), (vf + 4 * dt, vf + 4 * dt + 2), None))
-            m.append((mfma32_a(OB + 16 * dt, vf + 4 * dt, PW0["B"] + 4 * u), None, refill))
-    spread(e, m, exp_ops(1, PW1, mask1, t1_blocks), hold=3)
-    check(e, "92f")
-    # ---- phase 4a: values of keys 32..47 (fragments are in registers or about to arrive) ----
-    e.raw("; phase 4a")
-    m = [(mfma16_a(lreg[c], SUMA, PW1[c]), None, None) for c in t1_blocks]
-    for dt in range(4):
-        for ci, c in enumerate(t1_blocks):
-            m.append((mfma32_a(oreg[c] + 16 * dt, VF0 + 4 * dt, PW1[c]), (VF0 + 4 * dt, VF0 + 4 * dt + 2) if ci == 0 else None, None))
-    spread(e, m, [])
-    if kind != "plain":                          # the next tile's keys are 64 further along: thresholds move down
-        e.raw(f"v_subrev_u32 v{THR['A']}, 64, v{THR['A']}")
-        e.raw(f"v_subrev_u32 v{THR['B']}, 64, v{THR['B']}")
-    hand_over(e, buf, tag)
-    # ---- phase 4b: values of keys 48..63 ----
-    e.raw("; phase 4b")
-    m = [(mfma16_a(lreg[c], SUMA, PW1[c] + 4), None, None) for c in t1_blocks]
-    for dt in range(4):
-        for c in t1_blocks:
-            m.append((mfma32_a(oreg[c] + 16 * dt, VF1 + 4 * dt, PW1[c] + 4), None, None))
-    spread(e, m, [])
+    for j in range(8):
+        if j % 4 == 0:
+            m.append((mfma_sum("A", P[0]["A"] + 4 * (j // 4)), None, None))
+            m.append((mfma_sum("B", P[0]["B"] + 4 * (j // 4)), None, None))
+
+        def refill(j=j):
+            v_read(e, buf, 1, j)
+        m.append((mfma_o("A", j, P[0]["A"] + 4 * (j // 4)), vneeds(j), None))
+        m.append((mfma_o("B", j, P[0]["B"] + 4 * (j // 4)), None, refill))
+    emit(e, plan(m, exp_ops(1, mask1, h1_blocks), hold=3))
+    e.raw("s_nop 1")
+    e.raw("; O(.,1); the next tile's first K fragments are requested half way")
+    m = []
+    for j in range(8):
+        if j % 4 == 0:
+            for c in h1_blocks:
+                m.append((mfma_sum(c, P[1][c] + 4 * (j // 4)), None, None))
+
+        def next_k(j=j):
+            if j == 3:
+                for s in range(4):
+                    k_read(e, buf ^ 1, 0, s, s)
+        for ci, c in enumerate(h1_blocks):
+            m.append((mfma_o(c, j, P[1][c] + 4 * (j // 4)), vneeds(j) if ci == 0 else None,
+                      next_k if ci == len(h1_blocks) - 1 else None))
+    emit(e, plan(m, []))
+    e.raw(f"v_subrev_u32 v{THR['A']}, 64, v{THR['A']}")     # the next tile's keys are 64 further along
+    e.raw(f"v_subrev_u32 v{THR['B']}, 64, v{THR['B']}")
+    e.raw("s_add_u32 %[tile], %[tile], 1")
+    assert e.pending == start, (e.pending, start)
+    check_weights(e, "80f")
     e.raw("s_branch 20b")
+
+
+def half_step(e, *, s_part, o_part, valu, hold):
+    """The MFMAs of one pipeline half-step as planned entries.
+    s_part: (K buffer, half, k_next(i, slot) called after step i >= 4) -- S(., half) of the tile in that buffer; the
+            fragments of steps 0..3 are in flight, those of steps 4..7 are requested as the slots come free
+    o_part: (P half, v_next(j) called after fragment j is consumed) -- O += V^T fragments 0..7 (already requested)
+            . P(., half)
+    Order: per step i the two score MFMAs (blocks A, B), then the two (with row sums: four) accumulations of
+    fragment i."""
+    m = []
+    for i in range(8):
+        slot = i % 4
+        if s_part:
+            kbuf, kh, k_next = s_part
+
+            def k_refill(i=i, slot=slot, kbuf=kbuf, kh=kh, k_next=k_next):
+                if i < 4:
+                    k_read(e, kbuf, kh, i + 4, slot)
+                elif k_next:
+                    k_next(i, slot)
+            m.append((mfma_s("A", kh, slot, i), (KF + 4 * slot,), None))
+            m.append((mfma_s("B", kh, slot, i), None, k_refill))
+        if o_part:
+            ph, v_next = o_part
+            if i % 4 == 0:
+                m.append((mfma_sum("A", P[ph]["A"] + 4 * (i // 4)), None, None))
+                m.append((mfma_sum("B", P[ph]["B"] + 4 * (i // 4)), None, None))
+
+            def v_refill(i=i, v_next=v_next):
+                if v_next:
+                    v_next(i)
+            m.append((mfma_o("A", i, P[ph]["A"] + 4 * (i // 4)), vneeds(i), None))
+            m.append((mfma_o("B", i, P[ph]["B"] + 4 * (i // 4)), None, v_refill))
+    return plan(m, valu, hold)
+
+
+def pipeline(e, b, start, h0_start, dry=False):
+    """The software pipeline over unmasked tiles for tiles whose buffers are `b` (code for both parities is
+    generated; a tile step ends by jumping to the other parity's H0).  Returns the reads H1 leaves in flight."""
+    o = b ^ 1
+    # After the barrier of boundary(t): K[t+1] half 0 fragments 0, 1 and V[t] half 0 fragments 0..5 are requested at
+    # once (their registers are free); slots 2, 3 and fragments 6, 7 follow as steps 6, 7 of H0 consume them.
+    def k_after(i, slot):
+        if i >= 6:
+            k_read(e, o, 0, slot, slot)
+
+    def k_after_pro(i, slot):               # the prologue has no O part: fragments 6, 7 follow the K refills
+        if i >= 6:
+            k_read(e, o, 0, slot, slot)
+            v_read(e, b, 0, i)
+
+    def v_after(j):
+        if j >= 6:
+            v_read(e, b, 0, j)
+
+    def first_reads():
+        k_read(e, o, 0, 0, 0)
+        k_read(e, o, 0, 1, 1)
+        for j in range(6):
+            v_read(e, b, 0, j)
+
+    def tail_variants(entries, tagbase, join_label):
+        """boundary(t) and the rest of the half-step, in three variants by which requests exist."""
+        wait_and_meet(e)
+        first_reads()
+        e.raw("s_add_u32 %[t2], %[tile], 2")
+        e.raw("s_cmp_lt_u32 %[t2], %[n_tiles]")
+        e.raw(f"s_cbranch_scc1 {tagbase}2f")               # K[t+2] and V[t+1] exist
+        e.raw("s_add_u32 %[t2], %[tile], 1")
+        e.raw("s_cmp_lt_u32 %[t2], %[n_tiles]")
+        e.raw(f"s_cbranch_scc1 {tagbase}1f")               # only V[t+1]
+        saved, result = list(e.pending), None
+        for vi, which in ((0, ""), (1, "v"), (2, "kv")):
+            e.pending = list(saved)
+            if vi:
+                e.raw(f"{tagbase}{vi}:")
+            emit(e, entries, dma_chunks(which, b))
+            e.raw(f"s_branch {join_label}")
+            assert result is None or result == e.pending
+            result = list(e.pending)
+        return result
+
+    # ---------------- prologue: S(t,0), then H0 without its O part ----------------
+    e.pending = list(start)
+    e.raw(f"4{b}0:")
+    e.raw(f"; ---- pipeline prologue, tile in buffers {b}: S(t,0)")
+    emit(e, half_step(e, s_part=(b, 0, lambda i, slot: k_read(e, b, 1, i - 4, slot)), o_part=None, valu=[], hold=0))
+    e.raw("; S(t,1) | E(t,0), boundary inside")
+    pro = half_step(e, s_part=(b, 1, k_after_pro), o_part=None, valu=exp_ops(0, NONE), hold=3)
+    emit(e, pro[:12])                                      # steps 0..5
+    at_m = tail_variants(pro[12:], f"5{b}0", f"4{b}4f")
+
+    # ---------------- H0(t): S(t,1) | E(t,0) | O(t-1,1) ----------------
+    e.raw(f"4{b}1:")
+    e.raw(f"; ---- H0, tile in buffers {b}: S(t,1) | E(t,0) | O(t-1,1), boundary inside")
+    e.pending = list(h0_start)
+    h0 = half_step(e, s_part=(b, 1, k_after), o_part=(1, v_after), valu=exp_ops(0, NONE), hold=0)
+    emit(e, h0[:28])                                       # steps 0..5
+    at_m2 = tail_variants(h0[28:], f"5{b}1", f"4{b}4f")
+    assert dry or at_m == at_m2, (at_m, at_m2)
+
+    # ---------------- H1 ----------------
+    e.raw(f"4{b}4:")
+    e.pending = list(at_m2)
+    e.raw("s_add_u32 %[t2], %[tile], 1")
+    e.raw("s_cmp_ge_u32 %[t2], %[n_pipe]")
+    e.raw(f"s_cbranch_scc1 4{b}6f")
+    e.raw(f"; ---- H1, tile in buffers {b}: S(t+1,0) | E(t,1) | O(t,0)")
+    emit(e, half_step(e, s_part=(o, 0, lambda i, slot: k_read(e, o, 1, i - 4, slot)),
+                      o_part=(0, lambda j: v_read(e, b, 1, j)), valu=exp_ops(1, NONE), hold=0))
+    leaves = list(e.pending)
+    check_weights(e, f"4{b}7f")
+    e.raw("s_add_u32 %[tile], %[tile], 1")
+    e.raw(f"s_branch 4{o}1b" if o < b else f"s_branch 4{o}1f")
+    e.raw(f"4{b}7:")                                       # a weight reached 2: finish this tile, then leave
+    e.raw(f"s_mov_b32 s{FLAG}, 1")
+    e.raw(f"s_branch 4{b}5f")
+    # ---------------- H1 without its S part (the last unmasked tile the block may run) ----------------
+    e.raw(f"4{b}6:")
+    e.pending = list(at_m2)
+    e.raw(f"; ---- H1 tail, tile in buffers {b}: E(t,1) | O(t,0)")
+    emit(e, half_step(e, s_part=None, o_part=(0, lambda j: v_read(e, b, 1, j)), valu=exp_ops(1, NONE), hold=0))
+    check_weights(e, f"4{b}9f")
+    e.raw(f"s_branch 4{b}5f")
+    e.raw(f"4{b}9:")
+    e.raw(f"s_mov_b32 s{FLAG}, 1")
+    # ---------------- epilogue: O(t,1); the next tile's first K fragments are requested first ----------------
+    e.raw(f"4{b}5:")
+    e.raw("; ---- pipeline epilogue: O(t,1)")
+    e.raw("s_waitcnt lgkmcnt(0)")
+    e.pending = []
+    for s in range(4):
+        k_read(e, o, 0, s, s)
+    epi = half_step(e, s_part=None, o_part=(1, None), valu=[], hold=0)
+    emit(e, [(t, None, p_, v) for (t, _, p_, v) in epi])
+    e.raw("s_add_u32 %[tile], %[tile], 1")
+    assert e.pending == start, (e.pending, start)
+    e.raw("s_branch 20b")
+    return leaves
 
 
 def entry(e):
     """Loads the fixed registers from the block's operands: the Q^T fragments from the staging slab, nb, the row-sum
     operand, LDS read addresses (the address of step s / d-tile dt is the one of step 0 / d-tile 0 with s << 5 /
     dt << 6 XORed in: the swizzle XORs exactly those bits), DMA lane offsets and pointers, mask thresholds."""
-    for c, q in ((0, QA), (1, QB)):
+    for c in "AB":
         for s_ in range(8):
-            e.lines.append(f"ds_read_b128 v{rng(q + 4 * s_, 4)}, %[qaddr] offset:{c * 32 * Q_SLAB_ROW + 32 * s_}")
+            e.lines.append(f"ds_read_b128 a{rng(QREG[c] + 4 * s_, 4)}, %[qaddr] offset:{(c == 'B') * 32 * Q_SLAB_ROW + 32 * s_}")
     e.raw(f"v_mov_b32 v{NB['A']}, %[nb0]")
     e.raw(f"v_mov_b32 v{NB['B']}, %[nb1]")
     e.raw(f"v_mov_b32 v{NEGINF}, 0xff800000")
@@ -338,6 +544,7 @@ def entry(e):
     e.raw(f"s_mov_b32 s{KPTR + 1}, %[khi]")
     e.raw(f"s_mov_b32 s{VPTR}, %[vlo]")
     e.raw(f"s_mov_b32 s{VPTR + 1}, %[vhi]")
+    e.raw(f"s_mov_b32 s{FLAG}, 0")
     e.raw(f"v_mov_b32 {ANY}, 0")
 
 
@@ -358,6 +565,8 @@ def generate():
     assert e.pending == start
     # ---- loop head: which kind of tile, which buffer.  Every path arrives here with those four reads in flight. ----
     e.raw("20:")
+    e.raw(f"s_cmp_lg_u32 s{FLAG}, 0")
+    e.raw("s_cbranch_scc1 91f")
     e.raw("s_cmp_ge_u32 %[tile], %[n_end]")
     e.raw("s_cbranch_scc1 90f")
     e.raw("s_bitcmp1_b32 %[tile], 0")
@@ -365,34 +574,43 @@ def generate():
     for buf, lab in ((0, None), (1, "21")):
         if lab:
             e.raw(f"{lab}:")
-        e.raw("s_cmp_lt_u32 %[tile], %[n_plain]")
-        e.raw(f"s_cbranch_scc1 3{buf}0f")
+        e.raw("s_cmp_lt_u32 %[tile], %[n_pipe]")
+        e.raw(f"s_cbranch_scc1 4{buf}0f")
         e.raw("s_cmp_ge_u32 %[tile], %[n_mask]")
         e.raw(f"s_cbranch_scc1 3{buf}2f")
         e.raw("s_cmp_lg_u32 %[aligned], 0")              # masked: on an aligned diagonal the cheaper body
         e.raw(f"s_cbranch_scc1 3{buf}3f")
         e.raw(f"s_branch 3{buf}1f")
+    # what H1 leaves in flight for H0 (the same for both parities): from a dry run
+    dry = Emitter()
+    h0_start = pipeline(dry, 0, start, [], dry=True)
     for buf in (0, 1):
-        for kind in ("plain", "masked", "diag"):
+        leaves = pipeline(e, buf, start, h0_start)
+        assert leaves == h0_start, (leaves, h0_start)
+        for kind in ("masked", "diag"):
             e.pending = list(start)
             e.raw(f"3{buf}{KINDS[kind]}:")
-            tile_body(e, buf, kind)
-            assert e.pending == start, (e.pending, start)
-        # nothing visible in this tile: the wavefront only takes part in the hand-over
+            single_tile(e, buf, kind, start)
+        # nothing visible in this tile: the wavefront only takes part in the boundary
         e.pending = list(start)
         e.raw(f"3{buf}2:")
-        hand_over(e, buf, f"{buf}2")
+
+        def next_k(buf=buf):
+            for s in range(4):
+                k_read(e, buf ^ 1, 0, s, s)
+        boundary_plain(e, buf, f"{buf}2", next_k)
+        e.raw("s_add_u32 %[tile], %[tile], 1")
         assert e.pending == start
         e.raw("s_branch 20b")
     # exits
+    e.raw("80:")                                       # a masked tile saw a weight reach 2
+    e.raw(f"s_mov_b32 s{FLAG}, 1")
+    e.raw("s_branch 20b")
     e.raw("90:")
     e.raw("s_mov_b32 %[t2], 0")                        # %[t2] doubles as the status the block returns
     e.raw("s_branch 99f")
     e.raw("91:")
     e.raw("s_mov_b32 %[t2], 1")
-    e.raw("s_branch 99f")
-    e.raw("92:")
-    e.raw("s_mov_b32 %[t2], 2")
     e.raw("99:")
     e.raw("s_waitcnt lgkmcnt(0)")
     e.raw("s_nop 15")                                  # the last MFMA results are read by ordinary code next
@@ -400,13 +618,13 @@ def generate():
 
 
 def acc_of(c, dt):
-    return (OA, OB)[c] + 16 * dt
+    return (OREG["A"], OREG["B"])[c] + 16 * dt
 
 
 def snippets():
     """Small assembly statements through which ordinary code reaches the accumulators in the AGPRs."""
     out = {}
-    out["W64_ZERO"] = [f"v_accvgpr_write_b32 a{i}, 0" for i in range(LB + 4)]
+    out["W64_ZERO"] = [f"v_accvgpr_write_b32 a{i}, 0" for i in range(N_ACC)]
     for c in range(2):
         for dt in range(4):
             a = acc_of(c, dt)
@@ -416,7 +634,7 @@ def snippets():
                                        f"v_mfma_f32_32x32x16_bf16 a{rng(a, 16)}, %0, %1, a{rng(a, 16)}"]
             # 16 outputs %0..%15 <- the accumulator (after the last MFMA on it has finished)
             out[f"W64_READ_{c}_{dt}"] = ["s_nop 15"] + [f"v_accvgpr_read_b32 %{i}, a{a + i}" for i in range(16)]
-        la = (LA, LB)[c]
+        la = (LREG["A"], LREG["B"])[c]
         out[f"W64_SUM_{c}"] = ["s_nop 1", f"v_mfma_f32_16x16x32_bf16 a{rng(la, 4)}, %0, %1, a{rng(la, 4)}"]
         out[f"W64_READL_{c}"] = ["s_nop 15", f"v_accvgpr_read_b32 %0, a{la}", f"v_accvgpr_read_b32 %1, a{la + 1}"]
         # operands: %0 scratch (early-clobber output), %1 alpha of the lane's query, %2 / %3 alpha of queries c and c+16
@@ -433,9 +651,9 @@ def snippets():
 
 
 HEADER = '''// GENERATED by gen_prefill_w64_loop.py -- do not edit; change the generator and run it again.
-// Assembly of prefill_fwd_w64.hip: W64_LOOP is the hand-scheduled loop over the K/V tiles (register map and
-// phases: see the generator); the other macros are the small statements through which ordinary code reaches the
-// accumulators that live in the AGPRs.
+// Assembly of prefill_fwd_w64.hip: W64_LOOP is the hand-scheduled loop over the K/V tiles (register map, pipeline
+// and hand-over protocol: see the generator); the other macros are the small statements through which ordinary
+// code reaches the accumulators that live in the AGPRs.
 '''
 
 
@@ -452,11 +670,11 @@ def main():
         f.write(as_macro("W64_LOOP", lines))
         for name, body in snippets().items():
             f.write(as_macro(name, body))
-        acc = ", ".join('"a%d"' % i for i in range(LB + 4))
+        acc = ", ".join('"a%d"' % i for i in range(N_AGPRS))
         f.write(f"#define W64_CLOBBER_ACC {acc}\n")
         f.write("#define W64_CLOBBER_LOOP_VGPRS " + ", ".join('"v%d"' % i for i in range(N_FIXED_VGPRS)) + "\n")
     n_mfma = sum(1 for l in lines if l.startswith("v_mfma"))
-    print(f"wrote prefill_w64_asm.inc: loop of {len(lines)} lines, {n_mfma} MFMAs (four tile bodies)")
+    print(f"wrote prefill_w64_asm.inc: loop of {len(lines)} lines, {n_mfma} MFMAs")
 
 
 if __name__ == "__main__":

@@ -11,22 +11,27 @@
 // work out of the loop: row sums come from a 16x16x32 MFMA against a 0/1 operand instead of adds, and the exponent
 // reference is looked at only through the weights themselves.  A query tile starts with the reference preset to 0
 // (nb = -32: the weight of a score x is 2^(x - 32)) and the loop watches for a weight that reaches 2 (the top exponent
-// bit of its bf16 pattern): only then ordinary code moves the reference of that row up to its maximum, rescales and
+// bit of its bf16 pattern): only then ordinary code moves the reference of that row up, rescales and
 // resumes.  For scores between -60 and +33 binary orders -- anything a trained model produces -- no row maximum is
-// ever computed.  A row whose scores are all so negative that its sum stays below 2^-92 may have lost terms to
-// underflow; the workgroup then computes the whole query tile again with references taken from the data.
+// ever computed.  The loop notices a weight >= 2 at the end of its tile: the tile is already accumulated (weights up
+// to 2^40 are harmless in fp32 sums), the reference of every row is then moved by the exponent of its row sum, a
+// rescaling by an exact power of two.  A row whose sum left [2^-92, 2^40] may have lost terms to underflow or
+// overflow; the workgroup then computes the whole query tile again with references taken from the data.
 // (Folding the scale into the Q fragments would save the fma too, but rounds Q once more: the error of a score then
 // grows with the score, and outlier keys came out 3x less accurate.  Not done.)
 //
 // What differs most from prefill_fwd.hip is who schedules the instructions.  The loop over the K/V tiles of a query
 // tile is hand-scheduled assembly (prefill_w64_asm.inc, written by gen_prefill_w64_loop.py: vector and LDS
-// instructions sit at fixed places in the shadow of the MFMAs, which one wavefront per SIMD cannot leave to chance);
-// it covers unmasked tiles, the tiles on the causal diagonal and the tiles above it.  Ragged ends, reference moves and
-// the recomputation go through step_cxx below, ordinary HIP code on the same state.
+// instructions sit at fixed places in the shadow of the MFMAs, which one wavefront per SIMD cannot leave to chance,
+// and unmasked tiles run as a software pipeline across tiles); it covers unmasked tiles, the tiles on the causal
+// diagonal and the tiles above it.  Ragged ends and the recomputation go through step_cxx below, ordinary HIP code
+// on the same state.
 //
-// Hand-over protocol between the two (and between tiles): when a tile step starts, its tile has landed in LDS, the
-// workgroup has met at a barrier after that, and the next tile's loads are in flight.  A step ends by waiting for its
-// own share of the next tile, meeting the others at the barrier and requesting the tile after next.
+// Hand-over protocol between the two (and between tiles), one "boundary" per tile t and wavefront: K[t] and V[t]
+// live in LDS buffers t % 2.  When tile t starts, K[t] has landed and the workgroup has met since; K[t+1] and V[t]
+// are in flight.  At boundary(t) the wavefront has read what it needs of K[t] and V[t-1]; it waits for its own
+// shares of K[t+1] and V[t], meets the others at the barrier and requests K[t+2] and V[t+1] into the buffers just
+// freed.  Only after boundary(t) may it read V[t].
 #include <type_traits>
 
 #include "common.hpp"
@@ -105,6 +110,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     constexpr int D = kWD, NS = D / 16, NDT = D / 32, CPR = D / 8;
     constexpr float kBias = 32.0f;             // the largest weight sits at 2^-kBias when a reference is set
     constexpr float kUnderflow = 0x1p-92f;     // a row sum below this may have lost terms (see the file header)
+    constexpr float kOverflow = 0x1p40f;       // a row sum above this (or NaN) may have overflowed somewhere
 
     // K buffers 0,1 then V buffers 0,1 (the assembly loop addresses all four relative to one base)
     __shared__ __attribute__((aligned(1024))) unsigned char kv_lds[4 * kWTile];
@@ -184,29 +190,30 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const uint32_t dma_row_k = (uint32_t)(ld_q * (int)p.ks[2] * 2), dma_row_v = (uint32_t)(ld_q * (int)p.vs[2] * 2);
     const uint32_t lds_dst = __builtin_amdgcn_readfirstlane(lds_address(kv_lds + wave * 4096));
     const uint32_t k_step = (uint32_t)(4 * p.ks[2] * 2), v_step = (uint32_t)(4 * p.vs[2] * 2);   // 4 rows, in bytes
-    auto issue_tile = [&](const Job& jb, int tile, int buf) {
-        const unsigned char* kbase = reinterpret_cast<const unsigned char*>(jb.kb + ((int64_t)tile * kWBN + 16 * wave) * p.ks[2]);
-        const unsigned char* vbase = reinterpret_cast<const unsigned char*>(jb.vb + ((int64_t)tile * kWBN + 16 * wave) * p.vs[2]);
+    // K (which == 0) or V (which == 1) rows of tile `tile` into that tensor's LDS buffer `buf`
+    auto issue_rows = [&](const Job& jb, int which, int tile, int buf) {
+        const __bf16* src = which ? jb.vb : jb.kb;
+        const int64_t stride = which ? p.vs[2] : p.ks[2];
+        const uint32_t step = which ? v_step : k_step, dma_row = which ? dma_row_v : dma_row_k;
+        const uint32_t dst = lds_dst + (2 * which + buf) * kWTile;
         if (tile * kWBN + kWBN <= jb.sk) {
+            const unsigned char* base = reinterpret_cast<const unsigned char*>(src + ((int64_t)tile * kWBN + 16 * wave) * stride);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                dma_to_lds_16_m0(kbase + (size_t)j * k_step, dma_row_k + ((ld_c0 ^ j) << 4), lds_dst + buf * kWTile + j * 1024);
-                dma_to_lds_16_m0(vbase + (size_t)j * v_step, dma_row_v + ((ld_c0 ^ j) << 4), lds_dst + (2 + buf) * kWTile + j * 1024);
-            }
+            for (int j = 0; j < 4; ++j)
+                dma_to_lds_16_m0(base + (size_t)j * step, dma_row + ((ld_c0 ^ j) << 4), dst + j * 1024);
         } else {
             // last, partial tile: rows past the end re-read the last row (finite; their scores are masked)
             const int last = jb.sk - 1 - tile * kWBN;
-            const unsigned char* kt0 = reinterpret_cast<const unsigned char*>(jb.kb + (int64_t)tile * kWBN * p.ks[2]);
-            const unsigned char* vt0 = reinterpret_cast<const unsigned char*>(jb.vb + (int64_t)tile * kWBN * p.vs[2]);
+            const unsigned char* t0 = reinterpret_cast<const unsigned char*>(src + (int64_t)tile * kWBN * stride);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int row = min(16 * wave + 4 * j + ld_q, last);                 // row inside the tile
-                const int col = (ld_c0 ^ j) << 4;
-                dma_to_lds_16_m0(kt0, (uint32_t)(row * (int)p.ks[2] * 2 + col), lds_dst + buf * kWTile + j * 1024);
-                dma_to_lds_16_m0(vt0, (uint32_t)(row * (int)p.vs[2] * 2 + col), lds_dst + (2 + buf) * kWTile + j * 1024);
+                dma_to_lds_16_m0(t0, (uint32_t)(row * (int)stride * 2 + ((ld_c0 ^ j) << 4)), dst + j * 1024);
             }
         }
     };
+    auto issue_k = [&](const Job& jb, int tile, int buf) { issue_rows(jb, 0, tile, buf); };
+    auto issue_v = [&](const Job& jb, int tile, int buf) { issue_rows(jb, 1, tile, buf); };
     // number of K/V tiles of a job (the same for the four wavefronts)
     auto tiles_of = [&](const Job& jb) {
         int kv_end = jb.sk;
@@ -251,25 +258,51 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const int c16 = lane % CPR, r0 = lane / CPR;
 
     // What a job needs before it can start is requested as early as possible -- for the first job right here, for
-    // every other one while the job before it normalises and stores its output: K/V tiles 0 and 1 (direct-to-LDS)
-    // and the wavefront's query rows (into registers; rows past the end of the sequence are zero).
+    // every other one while the job before it normalises and stores its output: K[0] (direct-to-LDS), the wavefront's
+    // query rows (into registers; rows past the end of the sequence are zero), then K[1] and V[0].
     u32x4 q_rows[64 / kRowsPerPass];
     auto prefetch = [&](const Job& jb) {
         const int nt = tiles_of(jb);
-        if (nt > 0) issue_tile(jb, 0, 0);
-        if (nt > 1) issue_tile(jb, 1, 1);
+        if (nt > 0) issue_k(jb, 0, 0);
         const int qw0 = jb.q0 + 64 * wave;
 #pragma unroll
         for (int i = 0; i < 64 / kRowsPerPass; ++i) {
             const int r = i * kRowsPerPass + r0;
             q_rows[i] = u32x4{0u, 0u, 0u, 0u};
-            if (qw0 + r < jb.sq) q_rows[i] = *reinterpret_cast<const u32x4*>(jb.qb + (int64_t)(qw0 + r) * p.qs[2] + c16 * 8);
+            if (qw0 + i * kRowsPerPass < jb.sq) {          // (wave-uniform: see row_passes)
+                if (qw0 + r < jb.sq) q_rows[i] = *reinterpret_cast<const u32x4*>(jb.qb + (int64_t)(qw0 + r) * p.qs[2] + c16 * 8);
+            }
+        }
+        if (nt > 1) issue_k(jb, 1, 1);
+        if (nt > 0) issue_v(jb, 0, 0);
+    };
+    // number of row instructions (loads of query rows, stores of output rows: four rows each) a job issues: a pass
+    // whose four rows all lie past the end of the sequence is jumped over, so the count is known here
+    auto row_passes = [&](const Job& jb) {
+        return min(max((jb.sq - (jb.q0 + 64 * wave) + kRowsPerPass - 1) / kRowsPerPass, 0), 64 / kRowsPerPass);
+    };
+    // waits until at most `young` (rounded down to a multiple of 4) of this wavefront's vector-memory operations
+    // are in flight; they complete in order, so everything older than the youngest `young` has then arrived
+    auto wait_all_but = [&](int young) {
+        switch (young >> 2) {
+            case 0: wait_vmcnt<0>(); break;
+            case 1: wait_vmcnt<4>(); break;
+            case 2: wait_vmcnt<8>(); break;
+            case 3: wait_vmcnt<12>(); break;
+            case 4: wait_vmcnt<16>(); break;
+            case 5: wait_vmcnt<20>(); break;
+            case 6: wait_vmcnt<24>(); break;
+            case 7: wait_vmcnt<28>(); break;
+            case 8: wait_vmcnt<32>(); break;
+            case 9: wait_vmcnt<36>(); break;
+            default: wait_vmcnt<40>(); break;
         }
     };
 
     Job cur{}, nxt{};
     bool have = next_job(cur);
     if (have) prefetch(cur);
+    int prev_stores = 0;                                   // output row stores of the job before `cur`
     while (have) {
         const int sq = cur.sq, sk = cur.sk, q0 = cur.q0;
         const int coff = sk - sq;                          // bottom-right aligned causal diagonal
@@ -288,6 +321,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         // the assembly loop requests tile+2 with whole-tile loads: it may run tile t only if tile t+2 is a whole tile
         // (or does not exist), so it stops three tiles before a partial last tile
         const int n_asm = n_tiles > sk / kWBN ? max(0, n_tiles - 3) : n_tiles;
+        const int young_rows = row_passes(cur) + prev_stores;
 
         // query rows: registers -> slab (the previous job has read its output rows back from the slab by now: LDS
         // operations of a wavefront execute in order)
@@ -296,32 +330,33 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             *reinterpret_cast<u32x4*>(slab + (i * kRowsPerPass + r0) * kWORow + c16 * 16) = q_rows[i];
 
         // Two attempts at most: the first with the references preset to 0, the second -- only if some row's sum came
-        // out suspiciously small -- entirely in ordinary code with references taken from the data.
+        // out suspiciously small or large -- entirely in ordinary code with references taken from the data.
         bool have_next = false;
         for (int attempt = 0; attempt < 2; ++attempt) {
         const bool preset = attempt == 0;
+        const int young_dma = (n_tiles > 1 ? 4 : 0) + (n_tiles > 0 ? 4 : 0);      // requests of K[1] and V[0]
         if (!preset) {                        // start over: the buffers are free (everybody passed the vote below)
-            if (n_tiles > 0) issue_tile(cur, 0, 0);
-            if (n_tiles > 1) issue_tile(cur, 1, 1);
+            if (n_tiles > 0) issue_k(cur, 0, 0);
+            if (n_tiles > 1) issue_k(cur, 1, 1);
+            if (n_tiles > 0) issue_v(cur, 0, 0);
         }
         asm volatile(W64_ZERO : : : W64_CLOBBER_ACC);               // O^T and the row sums
         // per column block: r_ref exponent reference in the log2 domain (-inf: none yet), nb = -r_ref - kBias
         float r_ref[2], nb[2];
         r_ref[0] = r_ref[1] = preset ? 0.f : -INFINITY;
         nb[0] = nb[1] = preset ? -kBias : 0.f;
+        bool redo = false;                    // a row sum left the range in which no term can have been lost
 
-        // Wait for tile 0 and meet the others.  First attempt: the tiles were requested before the query rows, which
-        // have arrived (they are in the slab), and only the previous job's 16 output stores may be younger.  Second
-        // attempt: this wavefront's 8 loads of tile 1 may stay in flight.
-        if (preset) wait_vmcnt<16>(); else if (n_tiles > 1) wait_vmcnt<8>(); else wait_vmcnt<0>();
+        // Wait for K[0] and meet the others.  Younger than its request are: on the first attempt this job's query row
+        // loads and the previous job's output row stores (each issued once per four rows that exist), and on both
+        // the requests of K[1] and V[0].
+        wait_all_but(young_dma + (preset ? young_rows : 0));
         __syncthreads();
 
-        // One 32-key half of a tile for one column block, in ordinary code: scores, mask, reference move, weights,
-        // accumulation.  (Rare: ragged end, a row maximum that outgrew its reference, the second attempt.)
-        auto sub_block = [&](auto c_c, int tile, int t, bool masked) {
+        // Scores of one 32-key half of a tile for one column block, in ordinary code (reads K[tile]).
+        auto scores = [&](auto c_c, int tile, int t) {
             constexpr int c = decltype(c_c)::value;
             const int buf = tile & 1;
-            const int k0 = tile * kWBN + 32 * t;
             f32x16 s_acc;
 #pragma unroll
             for (int j = 0; j < 16; ++j) s_acc[j] = 0.f;
@@ -335,6 +370,13 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             }
 #pragma unroll
             for (int s = 0; s < NS; ++s) s_acc = mfma32(as_bf16x8(kf[s]), qf[s], s_acc);
+            return s_acc;
+        };
+        // The rest of that half: mask, reference move, weights, accumulation (reads V[tile]).
+        auto finish = [&](auto c_c, int tile, int t, bool masked, f32x16 s_acc) {
+            constexpr int c = decltype(c_c)::value;
+            const int buf = tile & 1;
+            const int k0 = tile * kWBN + 32 * t;
             const int qi = qw0 + 32 * c + n;
             float mx = -INFINITY;
 #pragma unroll
@@ -378,36 +420,63 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 acc_pv<c, 3>(vf[3], pf);
             }
         };
-        // the end of every tile step: own share of the next tile landed, everybody done with this one, tile+2 requested
-        auto hand_over = [&](int tile) {
-            if (tile + 1 < n_tiles) {
-                wait_vmcnt<0>();
-                __syncthreads();
-                if (tile + 2 < n_tiles) issue_tile(cur, tile + 2, tile & 1);
+        // boundary(tile): see the protocol in the file header
+        auto boundary = [&](int tile) {
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (tile + 1 < n_tiles) issue_v(cur, tile + 1, (tile + 1) & 1);
+            if (tile + 2 < n_tiles) issue_k(cur, tile + 2, tile & 1);
+        };
+        // a whole tile in ordinary code: scores from K[tile], boundary, everything else from V[tile]
+        // (a tile past n_mask has nothing for this wavefront: it only takes part in the boundary)
+        auto step_cxx = [&](int tile) {
+            const bool visible = tile < n_mask, masked = tile >= n_plain;
+            constexpr std::integral_constant<int, 0> A{};
+            constexpr std::integral_constant<int, 1> B{};
+            f32x16 sa0{}, sb0{}, sa1{}, sb1{};
+            if (visible) {
+                sa0 = scores(A, tile, 0);
+                sb0 = scores(B, tile, 0);
+                sa1 = scores(A, tile, 1);
+                sb1 = scores(B, tile, 1);
+            }
+            boundary(tile);
+            if (visible) {
+                finish(A, tile, 0, masked, sa0);
+                finish(B, tile, 0, masked, sb0);
+                finish(A, tile, 1, masked, sa1);
+                finish(B, tile, 1, masked, sb1);
             }
         };
-        auto step_cxx = [&](int tile, int t_first) {
-            if (tile < n_mask) {                      // (a tile past n_mask has nothing for this wavefront)
-                const bool masked = tile >= n_plain;
-                for (int t = t_first; t < 2; ++t) {
-                    sub_block(std::integral_constant<int, 0>{}, tile, t, masked);
-                    sub_block(std::integral_constant<int, 1>{}, tile, t, masked);
-                }
-            }
-            hand_over(tile);
+        // The assembly loop saw a weight reach 2: every row's reference moves up by the exponent of its sum (the sum,
+        // and with it every weight so far, lands in [2^-32, 2^-31)); an exact rescaling by a power of two.
+        auto move_references = [&](auto c_c) {
+            constexpr int c = decltype(c_c)::value;
+            float s_lo, s_hi;
+            acc_read_sums<c>(s_lo, s_hi);
+            const float l_lo = __shfl(s_lo, lane & 15, 64), l_hi = __shfl(s_hi, lane & 15, 64);
+            const float l = (n & 16) ? l_hi : l_lo;
+            if (!(l <= kOverflow)) redo = true;
+            const int expo = (int)((__builtin_bit_cast(uint32_t, l) >> 23) & 0xffu) - 127;
+            const int k = min(max(expo + (int)kBias, 0), 126);
+            const float alpha = __builtin_bit_cast(float, (uint32_t)(127 - k) << 23);      // 2^-k
+            if (__builtin_amdgcn_ballot_w64(k != 0) != 0)
+                acc_scale<c>(alpha, __shfl(alpha, lane & 15, 64), __shfl(alpha, (lane & 15) + 16, 64));
+            r_ref[c] += (float)k;
+            nb[c] -= (float)k;
         };
 
         int tile = 0;
         const int n_loop = preset ? n_asm : 0;
         while (tile < n_tiles) {
             if (tile >= n_loop) {
-                step_cxx(tile, 0);
+                step_cxx(tile);
                 ++tile;
                 continue;
             }
-            // ---- the hand-scheduled loop over tiles [tile, n_loop); leaves early when a weight reaches 2 ----
+            // ---- the hand-scheduled loop over tiles [tile, n_loop); leaves after a tile in which a weight reached 2 ----
             const uint64_t kptr = (uint64_t)(uintptr_t)(cur.kb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.ks[2]);
-            const uint64_t vptr = (uint64_t)(uintptr_t)(cur.vb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.vs[2]);
+            const uint64_t vptr = (uint64_t)(uintptr_t)(cur.vb + ((int64_t)(tile + 1) * kWBN + 16 * wave) * p.vs[2]);
             // mask thresholds for the first masked tile the loop will meet: a key at index j of that tile is kept by
             // query i of the wavefront iff j <= i + (qw0 + coff - k0) and j < sk - k0 (the lane part 4*kg of a key's
             // index is folded in)
@@ -426,19 +495,18 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                   [vhi0] "+v"(v_vhi), [rowk] "+v"(v_rowk), [rowv] "+v"(v_rowv), [c0s] "+v"(v_c0s), [qaddr] "+v"(v_q),
                   [thr0] "+v"(v_thr0), [thr1] "+v"(v_thr1)
                 : [n_tiles] "s"(__builtin_amdgcn_readfirstlane(n_tiles)), [n_end] "s"(__builtin_amdgcn_readfirstlane(n_loop)),
-                  [n_plain] "s"(__builtin_amdgcn_readfirstlane(n_plain)), [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)),
+                  [n_pipe] "s"(__builtin_amdgcn_readfirstlane(min(n_plain, n_loop))), [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)),
                   [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)),
                   [kstep] "s"(__builtin_amdgcn_readfirstlane(k_step)), [vstep] "s"(__builtin_amdgcn_readfirstlane(v_step)),
                   [ldsdst] "s"(lds_dst), [scale] "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, p.scale_log2))),
                   [klo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)kptr)), [khi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kptr >> 32))),
                   [vlo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)vptr)), [vhi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(vptr >> 32)))
-                : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
+                : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
             tile = tile_s;
-            // status 0: tiles up to n_loop done.  1: a weight of tile `tile` reached 2, nothing of that tile is
-            // accumulated.  2: likewise for its keys 32..63; keys 0..31 are accumulated.
+            // status 0: tiles up to n_loop done.  1: tiles up to `tile` done, and in the last of them a weight reached 2.
             if (status != 0) {
-                step_cxx(tile, status == 2 ? 1 : 0);
-                ++tile;
+                move_references(std::integral_constant<int, 0>{});
+                move_references(std::integral_constant<int, 1>{});
             }
         }
 
@@ -455,9 +523,10 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         read_sums(std::integral_constant<int, 0>{});
         read_sums(std::integral_constant<int, 1>{});
         if (preset) {
-            // (rows past the end of the sequence count too: their sums are sk * 2^-32, far above the limit)
-            const bool small = !(l_row[0] >= kUnderflow) || !(l_row[1] >= kUnderflow);
-            if (__syncthreads_or(small ? 1 : 0)) continue;
+            // (rows past the end of the sequence count too: their sums are sk * 2^-32, far above the lower limit)
+            const bool bad = redo || !(l_row[0] >= kUnderflow) || !(l_row[1] >= kUnderflow) || !(l_row[0] <= kOverflow) ||
+                             !(l_row[1] <= kOverflow);
+            if (__syncthreads_or(bad ? 1 : 0)) continue;
         } else {
             __syncthreads();
         }
@@ -497,8 +566,11 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         for (int i = 0; i < 64 / kRowsPerPass; ++i) {
             const int r = i * kRowsPerPass + r0;
             const u32x4 w = *reinterpret_cast<const u32x4*>(slab + r * kWORow + c16 * 16);
-            if (qw0 + r < sq) *reinterpret_cast<u32x4*>(cur.ob + (int64_t)(qw0 + r) * p.os[2] + c16 * 8) = w;
+            if (qw0 + i * kRowsPerPass < sq) {             // (wave-uniform: see row_passes)
+                if (qw0 + r < sq) *reinterpret_cast<u32x4*>(cur.ob + (int64_t)(qw0 + r) * p.os[2] + c16 * 8) = w;
+            }
         }
+        prev_stores = row_passes(cur);
         cur = nxt;
         have = have_next;
     }
