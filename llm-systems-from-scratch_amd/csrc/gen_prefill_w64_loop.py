@@ -64,7 +64,7 @@ Register map (physical, fixed; the block loads them itself from its operands, se
 """
 import os
 
-# timing experiments only (results wrong): nobarrier, nodma, nocheck, noexp, novalu, nosum
+# timing experiments only (results wrong): nobarrier, nodma, nocheck, noexp, novalu, nosum, nofma, noor
 ABL = os.environ.get("W64_ABL", "").split(",")
 
 EXP = "v_mov_b32" if "noexp" in ABL else "v_exp_f32"
@@ -183,15 +183,20 @@ def exp_ops(h, mask, blocks="AB"):
         for w in range(8):                      # packed word w of the block: accumulator registers 2w, 2w+1
             t0, t1 = ETMP[2 * (i % 4)], ETMP[2 * (i % 4) + 1]
             for tmp, r in ((t0, 2 * w), (t1, 2 * w + 1)):
-                ops.append(f"v_fma_f32 {tmp}, v{S[(c, h)] + r}, %[scale], v{NB[c]}")
+                if "nofma" not in ABL or mask[c]:
+                    ops.append(f"v_fma_f32 {tmp}, v{S[(c, h)] + r}, %[scale], v{NB[c]}")
                 if mask[c]:
                     ops.append(f"v_cmp_le_i32_e64 vcc, {32 * h + 8 * (r // 4) + r % 4}, v{THR[c]}")
                     ops.append(f"v_cndmask_b32 {tmp}, v{NEGINF}, {tmp}, vcc")
-            ops.append(f"{EXP} {t0}, {t0}")
-            ops.append(f"{EXP} {t1}, {t1}")
+            if "nofma" in ABL and not mask[c]:
+                ops.append(f"{EXP} {t0}, v{S[(c, h)] + 2 * w}")
+                ops.append(f"{EXP} {t1}, v{S[(c, h)] + 2 * w + 1}")
+            else:
+                ops.append(f"{EXP} {t0}, {t0}")
+                ops.append(f"{EXP} {t1}, {t1}")
             ops += pend
             pend = [f"v_cvt_pk_bf16_f32 v{dst + w}, {t0}, {t1}"]
-            if w % 2 == 1:
+            if w % 2 == 1 and "noor" not in ABL:
                 pend.append(f"v_or3_b32 {ANY}, {ANY}, v{dst + w - 1}, v{dst + w}")
             i += 1
     ops += ["s_nop 0"] + pend
