@@ -11,8 +11,8 @@ What stays ordinary HIP C++: prologue, epilogue, ragged ends, and moving a row's
 One tile = 64 keys; a wavefront owns 64 queries = column blocks A and B of 32; head_dim 128.  Per 32-key half h of
 tile t there are three pieces of work (each for both blocks):
   S(t,h)  scores   = K[t][32h:32h+32] . Q^T         16 MFMA 32x32x16 (8 per block), K fragments from LDS
-  E(t,h)  weights  = bf16(2^(S * scale + nb))       32 v_fma, 32 v_exp, 16 cvt, 8 or3 (a masked tile adds a compare
-                                                    and a select per score)
+  E(t,h)  weights  = bf16(2^(S * scale + nb))       32 v_fma, 32 v_exp, 16 cvt (a masked tile adds a compare and a
+                                                    select per score)
   O(t,h)  O^T     += V[t][32h:32h+32]^T . P, l += row sums   16 MFMA + 4 row-sum MFMA 16x16x32, V^T fragments from LDS
 With one wavefront per SIMD the vector work of a half hides only behind MFMAs of the same wavefront that do not
 depend on it.  Unmasked tiles therefore run as a software pipeline across tiles, two half-steps per tile:
@@ -34,8 +34,8 @@ fragments are in registers by then) covers the latency of the first reads of K[t
 issued between its MFMAs.
 
 Weights are 2^(score * scale + nb) with nb preset by the caller (see the kernel); nothing here looks at row maxima.
-Each tile ORs its packed weights together, and a weight >= 2 (top exponent bit of a bf16 pattern) ends the block
-after that tile with status 1: the caller lowers nb of the rows that need it, rescales, and re-enters.
+At the end of each tile the row sums are looked at, and a sum >= 2 ends the block after that tile with status 1: the
+caller lowers nb of the rows that need it, rescales, and re-enters.
 
 Tiles come in three kinds, by index: [0, n_plain) every key visible to every query; [n_plain, n_mask) masked (causal
 diagonal: key <= threshold of the lane's query; the threshold moves down by 64 per tile); [n_mask, n_end) nothing
@@ -54,17 +54,17 @@ Register map (physical, fixed; the block loads them itself from its operands, se
   buffer and the position inside the tile are immediates; V tiles sit two tile sizes behind the K tiles),
   v[170:177] lane offsets of the direct-to-LDS loads (K steps 0..3, V steps 0..3)
   twelve more registers, wherever the compiler puts the block's vector operands: after entry() they serve as scratch
-  (collected weight bits, exponentials on their way to packing)
+  (exponentials on their way to packing)
   a[0:63] O^T of block A (d-tile dt = a[16dt:16dt+15]), a[64:127] block B, a[128:131] / a[132:135] row sums:
   these live in the AGPRs for a whole query tile and are touched only by the assembly snippets below (the kernel
   is compiled with its builtin MFMAs in VGPR form, so the compiler has no use for AGPRs of its own)
   a[136:167] Q^T fragments of block A (step s = a[136+4s:139+4s]), a[168:199] block B: loaded by entry()
   s[36:37] / s[38:39] global address of the wavefront's first DMA row of K[t+2] / V[t+1] (advanced per tile),
-  s[40:41] scratch, s42 "a weight reached 2"; every other scalar is a named operand
+  s[40:41] scratch, s42 "a row sum reached 2"; every other scalar is a named operand
 """
 import os
 
-# timing experiments only (results wrong): nobarrier, nodma, nocheck, noexp, novalu, nosum, nofma, noor
+# timing experiments only (results wrong): nobarrier, nodma, nocheck, noexp, novalu, nosum, nofma
 ABL = os.environ.get("W64_ABL", "").split(",")
 
 EXP = "v_mov_b32" if "noexp" in ABL else "v_exp_f32"
@@ -81,7 +81,7 @@ N_FIXED_VGPRS = 178
 # Scratch registers are the block's vector operands themselves: each is read once by entry() and is free from then on
 # (the operands are declared in/out), so the block needs no register beyond v[0:177] and its operands.
 ETMP = ["%[nb0]", "%[nb1]", "%[suma]", "%[k0]", "%[vlo0]", "%[vhi0]", "%[rowk]", "%[rowv]"]   # exponentials on their way to packing
-ANY, TMP = "%[c0s]", "%[qaddr]"     # collected weight bits; scratch
+TMP = "%[qaddr]"                    # scratch
 OREG = {"A": 0, "B": 64}
 LREG = {"A": 128, "B": 132}
 QREG = {"A": 136, "B": 168}
@@ -196,8 +196,6 @@ def exp_ops(h, mask, blocks="AB"):
                 ops.append(f"{EXP} {t1}, {t1}")
             ops += pend
             pend = [f"v_cvt_pk_bf16_f32 v{dst + w}, {t0}, {t1}"]
-            if w % 2 == 1 and "noor" not in ABL:
-                pend.append(f"v_or3_b32 {ANY}, {ANY}, v{dst + w - 1}, v{dst + w}")
             i += 1
     ops += ["s_nop 0"] + pend
     return ops
@@ -240,11 +238,18 @@ def emit(e, entries, extras=()):
             xi += 1
 
 
-def check_weights(e, flagged_label):
-    """End of a tile: did one of its weights reach 2?  Then control goes to `flagged_label`."""
-    e.raw(f"v_and_b32 {TMP}, 0x40004000, {ANY}")
-    e.raw(f"v_cmp_ne_u32 vcc, 0, {TMP}")
-    e.raw(f"v_mov_b32 {ANY}, 0")
+def check_sums(e, flagged_label):
+    """End of a tile: has a row sum reached 2 (or become NaN)?  Then control goes to `flagged_label`.  Lanes 0..15 of
+    the first two registers of each row-sum accumulator hold the sums, everything else there is zero; the last
+    row-sum MFMA was issued at least eight MFMAs ago."""
+    t = ETMP
+    e.raw(f"v_accvgpr_read_b32 {t[0]}, a{LREG['A']}")
+    e.raw(f"v_accvgpr_read_b32 {t[1]}, a{LREG['A'] + 1}")
+    e.raw(f"v_accvgpr_read_b32 {t[2]}, a{LREG['B']}")
+    e.raw(f"v_accvgpr_read_b32 {t[3]}, a{LREG['B'] + 1}")
+    e.raw(f"v_max3_f32 {t[0]}, {t[0]}, {t[1]}, {t[2]}")
+    e.raw(f"v_max_f32 {t[0]}, {t[0]}, {t[3]}")
+    e.raw(f"v_cmp_nlt_f32_e64 vcc, {t[0]}, 2.0")
     e.raw("s_nop 1")
     if "nocheck" not in ABL:
         e.raw(f"s_cbranch_vccnz {flagged_label}")
@@ -377,7 +382,7 @@ def single_tile(e, buf, kind, start):
     e.raw(f"v_subrev_u32 v{THR['B']}, 64, v{THR['B']}")
     e.raw("s_add_u32 %[tile], %[tile], 1")
     assert e.pending == start, (e.pending, start)
-    check_weights(e, "80f")
+    check_sums(e, "80f")
     e.raw("s_branch 20b")
 
 
@@ -491,10 +496,10 @@ def pipeline(e, b, start, h0_start, dry=False):
     emit(e, half_step(e, s_part=(o, 0, lambda i, slot: k_read(e, o, 1, i - 4, slot)),
                       o_part=(0, lambda j: v_read(e, b, 1, j)), valu=exp_ops(1, NONE), hold=0))
     leaves = list(e.pending)
-    check_weights(e, f"4{b}7f")
+    check_sums(e, f"4{b}7f")
     e.raw("s_add_u32 %[tile], %[tile], 1")
     e.raw(f"s_branch 4{o}1b" if o < b else f"s_branch 4{o}1f")
-    e.raw(f"4{b}7:")                                       # a weight reached 2: finish this tile, then leave
+    e.raw(f"4{b}7:")                                       # a row sum reached 2: finish this tile, then leave
     e.raw(f"s_mov_b32 s{FLAG}, 1")
     e.raw(f"s_branch 4{b}5f")
     # ---------------- H1 without its S part (the last unmasked tile the block may run) ----------------
@@ -502,7 +507,7 @@ def pipeline(e, b, start, h0_start, dry=False):
     e.pending = list(at_m2)
     e.raw(f"; ---- H1 tail, tile in buffers {b}: E(t,1) | O(t,0)")
     emit(e, half_step(e, s_part=None, o_part=(0, lambda j: v_read(e, b, 1, j)), valu=exp_ops(1, NONE), hold=0))
-    check_weights(e, f"4{b}9f")
+    check_sums(e, f"4{b}9f")
     e.raw(f"s_branch 4{b}5f")
     e.raw(f"4{b}9:")
     e.raw(f"s_mov_b32 s{FLAG}, 1")
@@ -550,7 +555,6 @@ def entry(e):
     e.raw(f"s_mov_b32 s{VPTR}, %[vlo]")
     e.raw(f"s_mov_b32 s{VPTR + 1}, %[vhi]")
     e.raw(f"s_mov_b32 s{FLAG}, 0")
-    e.raw(f"v_mov_b32 {ANY}, 0")
 
 
 def generate():
@@ -608,7 +612,7 @@ def generate():
         assert e.pending == start
         e.raw("s_branch 20b")
     # exits
-    e.raw("80:")                                       # a masked tile saw a weight reach 2
+    e.raw("80:")                                       # a masked tile took a row sum to 2
     e.raw(f"s_mov_b32 s{FLAG}, 1")
     e.raw("s_branch 20b")
     e.raw("90:")
@@ -629,7 +633,10 @@ def acc_of(c, dt):
 def snippets():
     """Small assembly statements through which ordinary code reaches the accumulators in the AGPRs."""
     out = {}
-    out["W64_ZERO"] = [f"v_accvgpr_write_b32 a{i}, 0" for i in range(N_ACC)]
+    # operand %0: four registers of zeros.  The products land long before anything reads the accumulators, and the
+    # wavefront spends ten issue slots instead of 136 register writes.
+    out["W64_ZERO"] = ([f"v_mfma_f32_32x32x16_bf16 a{rng(16 * i, 16)}, %0, %0, 0" for i in range(8)] +
+                       [f"v_mfma_f32_16x16x32_bf16 a{rng(LREG[c], 4)}, %0, %0, 0" for c in "AB"])
     for c in range(2):
         for dt in range(4):
             a = acc_of(c, dt)

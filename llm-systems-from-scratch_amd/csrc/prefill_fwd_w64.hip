@@ -10,10 +10,10 @@
 // lane, weights 2^(s * scale * log2(e) + nb) with one fma and one exp2 per score), with two changes that take vector
 // work out of the loop: row sums come from a 16x16x32 MFMA against a 0/1 operand instead of adds, and the exponent
 // reference is looked at only through the weights themselves.  A query tile starts with the reference preset to 0
-// (nb = -32: the weight of a score x is 2^(x - 32)) and the loop watches for a weight that reaches 2 (the top exponent
-// bit of its bf16 pattern): only then ordinary code moves the reference of that row up, rescales and
+// (nb = -32: the weight of a score x is 2^(x - 32)) and the loop watches for a row sum that reaches 2: only then
+// ordinary code moves the reference of that row up, rescales and
 // resumes.  For scores between -60 and +33 binary orders -- anything a trained model produces -- no row maximum is
-// ever computed.  The loop notices a weight >= 2 at the end of its tile: the tile is already accumulated (weights up
+// ever computed.  The loop notices a row sum >= 2 at the end of a tile: the tile is already accumulated (weights up
 // to 2^40 are harmless in fp32 sums), the reference of every row is then moved by the exponent of its row sum, a
 // rescaling by an exact power of two.  A row whose sum left [2^-92, 2^40] may have lost terms to underflow or
 // overflow; the workgroup then computes the whole query tile again with references taken from the data.
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             if (n_tiles > 1) issue_k(cur, 1, 1);
             if (n_tiles > 0) issue_v(cur, 0, 0);
         }
-        asm volatile(W64_ZERO : : : W64_CLOBBER_ACC);               // O^T and the row sums
+        asm volatile(W64_ZERO : : "v"(as_bf16x8(u32x4{0u, 0u, 0u, 0u})) : W64_CLOBBER_ACC);      // O^T and the row sums
         // per column block: r_ref exponent reference in the log2 domain (-inf: none yet), nb = -r_ref - kBias
         float r_ref[2], nb[2];
         r_ref[0] = r_ref[1] = preset ? 0.f : -INFINITY;
@@ -448,7 +448,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 finish(B, tile, 1, masked, sb1);
             }
         };
-        // The assembly loop saw a weight reach 2: every row's reference moves up by the exponent of its sum (the sum,
+        // The assembly loop saw a row sum reach 2: every row's reference moves up by the exponent of its sum (the sum,
         // and with it every weight so far, lands in [2^-32, 2^-31)); an exact rescaling by a power of two.
         auto move_references = [&](auto c_c) {
             constexpr int c = decltype(c_c)::value;
@@ -474,7 +474,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 ++tile;
                 continue;
             }
-            // ---- the hand-scheduled loop over tiles [tile, n_loop); leaves after a tile in which a weight reached 2 ----
+            // ---- the hand-scheduled loop over tiles [tile, n_loop); leaves after a tile that took a row sum to 2 ----
             const uint64_t kptr = (uint64_t)(uintptr_t)(cur.kb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.ks[2]);
             const uint64_t vptr = (uint64_t)(uintptr_t)(cur.vb + ((int64_t)(tile + 1) * kWBN + 16 * wave) * p.vs[2]);
             // mask thresholds for the first masked tile the loop will meet: a key at index j of that tile is kept by
@@ -503,7 +503,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                   [vlo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)vptr)), [vhi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(vptr >> 32)))
                 : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
             tile = tile_s;
-            // status 0: tiles up to n_loop done.  1: tiles up to `tile` done, and in the last of them a weight reached 2.
+            // status 0: tiles up to n_loop done.  1: tiles up to `tile` done, and the last of them took a row sum to 2.
             if (status != 0) {
                 move_references(std::integral_constant<int, 0>{});
                 move_references(std::integral_constant<int, 1>{});
