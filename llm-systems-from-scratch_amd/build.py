@@ -18,7 +18,10 @@ SOURCES = ["api.hip", "paged_decode.hip", "prefill_fwd.hip", "prefill_fwd_w64.hi
            "layer_ops.hip"]
 # prefill_fwd_w64.hip keeps its output accumulators in AGPRs that only its assembly statements touch: its builtin MFMAs
 # must therefore be selected in VGPR form, so that the compiler allocates no AGPR for them.
-EXTRA_FLAGS = {"prefill_fwd_w64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+# It is also compiled without the machine-code hoisting of loop invariants: hoisted out of the job loop, a few dozen
+# per-lane addresses stayed live across the assembly loop (which owns most vector registers) and pushed the
+# prefetched query rows into scratch memory, whose reloads wait for every load in flight.
+EXTRA_FLAGS = {"prefill_fwd_w64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1", "-mllvm", "-disable-machine-licm"]}
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -46,19 +46,20 @@ body: only the two triangular 32x32 sub-blocks get mask code, and the invisible 
 Register map (physical, fixed; the block loads them itself from its operands, see entry()):
   v[0:31]   S(A,0), S(B,0)     v[32:63]  S(A,1), S(B,1)
   v[64:79]  P(.,0): A slices 0,1 then B slices 0,1 (a slice = 16 keys = 4 registers)     v[80:95] P(.,1)
-  v[96:111] K fragments (4 in flight)    v[112:143] V^T fragments (8: 2 slices x 4 d-tiles)
-  v144 / v145 nb (the additive term of the exponent) of this lane's query in block A / B
-  v146 -inf, v147 / v148 mask threshold of the lane's query in block A / B (key index inside the tile, minus 4*(lane/32))
-  v[150:153] A operand of the row-sum MFMA
-  v[154:161] K fragment LDS addresses per step, v[162:169] V^T LDS addresses [half][d-tile] (both for buffer 0; the
+  v96 / v97 nb (the additive term of the exponent) of this lane's query in block A / B
+  v98 -inf, v99 / v100 mask threshold of the lane's query in block A / B (key index inside the tile, minus 4*(lane/32))
+  v[102:105] A operand of the row-sum MFMA
+  v[106:113] K fragment LDS addresses per step, v[114:121] V^T LDS addresses [half][d-tile] (both for buffer 0; the
   buffer and the position inside the tile are immediates; V tiles sit two tile sizes behind the K tiles),
-  v[170:177] lane offsets of the direct-to-LDS loads (K steps 0..3, V steps 0..3)
+  v[122:129] lane offsets of the direct-to-LDS loads (K steps 0..3, V steps 0..3)
   twelve more registers, wherever the compiler puts the block's vector operands: after entry() they serve as scratch
   (exponentials on their way to packing)
   a[0:63] O^T of block A (d-tile dt = a[16dt:16dt+15]), a[64:127] block B, a[128:131] / a[132:135] row sums:
   these live in the AGPRs for a whole query tile and are touched only by the assembly snippets below (the kernel
   is compiled with its builtin MFMAs in VGPR form, so the compiler has no use for AGPRs of its own)
   a[136:167] Q^T fragments of block A (step s = a[136+4s:139+4s]), a[168:199] block B: loaded by entry()
+  a[200:215] K fragments (4 in flight), a[216:247] V^T fragments (8: 2 slices x 4 d-tiles): LDS reads land in
+  AGPRs directly and the MFMAs take them as A operands, which leaves the vector registers to the compiler
   s[36:37] / s[38:39] global address of the wavefront's first DMA row of K[t+2] / V[t+1] (advanced per tile),
   s[40:41] scratch, s42 "a row sum reached 2"; every other scalar is a named operand
 """
@@ -70,23 +71,23 @@ ABL = os.environ.get("W64_ABL", "").split(",")
 EXP = "v_mov_b32" if "noexp" in ABL else "v_exp_f32"
 S = {("A", 0): 0, ("B", 0): 16, ("A", 1): 32, ("B", 1): 48}
 P = {0: {"A": 64, "B": 72}, 1: {"A": 80, "B": 88}}          # + 4 * slice inside the half
-KF = 96
-VF = 112                            # fragment j (slice j // 4 of the half, d-tile j % 4) at VF + 4j
-NB = {"A": 144, "B": 145}
-NEGINF = 146
-THR = {"A": 147, "B": 148}
-SUMA = 150                          # (register tuples of MFMA operands start at even registers)
-KOFF, VOFF, DMAOFF = 154, 162, 170
-N_FIXED_VGPRS = 178
+KF = 200                            # AGPRs: LDS reads land there directly, the MFMAs take them as A operands
+VF = 216                            # AGPRs: fragment j (slice j // 4 of the half, d-tile j % 4) at VF + 4j
+NB = {"A": 96, "B": 97}
+NEGINF = 98
+THR = {"A": 99, "B": 100}
+SUMA = 102                          # (register tuples of MFMA operands start at even registers)
+KOFF, VOFF, DMAOFF = 106, 114, 122
+N_FIXED_VGPRS = 130
 # Scratch registers are the block's vector operands themselves: each is read once by entry() and is free from then on
-# (the operands are declared in/out), so the block needs no register beyond v[0:177] and its operands.
+# (the operands are declared in/out), so the block needs no register beyond v[0:129] and its operands.
 ETMP = ["%[nb0]", "%[nb1]", "%[suma]", "%[k0]", "%[vlo0]", "%[vhi0]", "%[rowk]", "%[rowv]"]   # exponentials on their way to packing
 TMP = "%[qaddr]"                    # scratch
 OREG = {"A": 0, "B": 64}
 LREG = {"A": 128, "B": 132}
 QREG = {"A": 136, "B": 168}
 N_ACC = 136                         # a[0:135]: what ordinary code reaches through the snippets
-N_AGPRS = 200
+N_AGPRS = 248
 KPTR, VPTR, PTMP, FLAG = 36, 38, 40, 42
 Q_SLAB_ROW = 272                    # bytes per row of the query staging slab (256 + 16 of padding)
 K_TILE = 16384                      # bytes of one K (or V) tile in LDS: 64 rows x 256 bytes
@@ -137,13 +138,13 @@ def mfma_s(c, h, slot, s):
     """S(c,h) (+)= K fragment in `slot` . Q^T fragment of step s."""
     dst = S[(c, h)]
     cs = "0" if s == 0 else f"v{rng(dst, 16)}"
-    return f"v_mfma_f32_32x32x16_bf16 v{rng(dst, 16)}, v{rng(KF + 4 * slot, 4)}, a{rng(QREG[c] + 4 * s, 4)}, {cs}"
+    return f"v_mfma_f32_32x32x16_bf16 v{rng(dst, 16)}, a{rng(KF + 4 * slot, 4)}, a{rng(QREG[c] + 4 * s, 4)}, {cs}"
 
 
 def mfma_o(c, j, p):
     """O^T(c, d-tile j % 4) += V^T fragment j . P words at p."""
     acc = OREG[c] + 16 * (j % 4)
-    return f"v_mfma_f32_32x32x16_bf16 a{rng(acc, 16)}, v{rng(VF + 4 * j, 4)}, v{rng(p, 4)}, a{rng(acc, 16)}"
+    return f"v_mfma_f32_32x32x16_bf16 a{rng(acc, 16)}, a{rng(VF + 4 * j, 4)}, v{rng(p, 4)}, a{rng(acc, 16)}"
 
 
 def mfma_sum(c, p):
@@ -154,15 +155,15 @@ def mfma_sum(c, p):
 
 
 def k_read(e, buf, h, s, slot):
-    e.lds_read(f"ds_read_b128 v{rng(KF + 4 * slot, 4)}, v{KOFF + s} offset:{buf * K_TILE + h * 32 * ROW}", KF + 4 * slot)
+    e.lds_read(f"ds_read_b128 a{rng(KF + 4 * slot, 4)}, v{KOFF + s} offset:{buf * K_TILE + h * 32 * ROW}", KF + 4 * slot)
 
 
 def v_read(e, buf, h, j):
     """V^T fragment j of half h (16-key slice 2h + j // 4, d-tile j % 4) into its registers (two transposed 64-bit reads)."""
     off = buf * K_TILE + 16 * (2 * h + j // 4) * ROW
     base, dt = VF + 4 * j, j % 4
-    e.lds_read(f"ds_read_b64_tr_b16 v{rng(base, 2)}, v{VOFF + dt} offset:{off}", base)
-    e.lds_read(f"ds_read_b64_tr_b16 v{rng(base + 2, 2)}, v{VOFF + 4 + dt} offset:{off}", base + 2)
+    e.lds_read(f"ds_read_b64_tr_b16 a{rng(base, 2)}, v{VOFF + dt} offset:{off}", base)
+    e.lds_read(f"ds_read_b64_tr_b16 a{rng(base + 2, 2)}, v{VOFF + 4 + dt} offset:{off}", base + 2)
 
 
 def vneeds(j):
@@ -635,19 +636,23 @@ def snippets():
     out = {}
     # operand %0: four registers of zeros.  The products land long before anything reads the accumulators, and the
     # wavefront spends ten issue slots instead of 136 register writes.
-    out["W64_ZERO"] = ([f"v_mfma_f32_32x32x16_bf16 a{rng(16 * i, 16)}, %0, %0, 0" for i in range(8)] +
+    # (The s_nop: the compiler may have written the operand in the instruction just before this statement, and
+    # cannot see that an MFMA reads it here.)
+    out["W64_ZERO"] = (["s_nop 3"] + [f"v_mfma_f32_32x32x16_bf16 a{rng(16 * i, 16)}, %0, %0, 0" for i in range(8)] +
                        [f"v_mfma_f32_16x16x32_bf16 a{rng(LREG[c], 4)}, %0, %0, 0" for c in "AB"])
     for c in range(2):
         for dt in range(4):
             a = acc_of(c, dt)
             # operands: %0 V^T fragment (4 registers), %1 P^T fragment (4 registers), both ready when the statement
-            # starts (the compiler waits for the LDS reads behind its operands)
-            out[f"W64_PV_{c}_{dt}"] = ["s_nop 1",
+            # starts (the compiler waits for the LDS reads behind its operands; the s_nop covers a vector
+            # instruction that wrote an operand just before the statement, which the compiler's hazard
+            # bookkeeping cannot relate to an MFMA inside it)
+            out[f"W64_PV_{c}_{dt}"] = ["s_nop 3",
                                        f"v_mfma_f32_32x32x16_bf16 a{rng(a, 16)}, %0, %1, a{rng(a, 16)}"]
             # 16 outputs %0..%15 <- the accumulator (after the last MFMA on it has finished)
             out[f"W64_READ_{c}_{dt}"] = ["s_nop 15"] + [f"v_accvgpr_read_b32 %{i}, a{a + i}" for i in range(16)]
         la = (LREG["A"], LREG["B"])[c]
-        out[f"W64_SUM_{c}"] = ["s_nop 1", f"v_mfma_f32_16x16x32_bf16 a{rng(la, 4)}, %0, %1, a{rng(la, 4)}"]
+        out[f"W64_SUM_{c}"] = ["s_nop 3", f"v_mfma_f32_16x16x32_bf16 a{rng(la, 4)}, %0, %1, a{rng(la, 4)}"]
         out[f"W64_READL_{c}"] = ["s_nop 15", f"v_accvgpr_read_b32 %0, a{la}", f"v_accvgpr_read_b32 %1, a{la + 1}"]
         # operands: %0 scratch (early-clobber output), %1 alpha of the lane's query, %2 / %3 alpha of queries c and c+16
         # as the row-sum accumulator holds them

@@ -202,13 +202,17 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             for (int j = 0; j < 4; ++j)
                 dma_to_lds_16_m0(base + (size_t)j * step, dma_row + ((ld_c0 ^ j) << 4), dst + j * 1024);
         } else {
-            // last, partial tile: rows past the end re-read the last row (finite; their scores are masked)
-            const int last = jb.sk - 1 - tile * kWBN;
+            // last, partial tile: rows past the end re-read the last row (finite; their scores are masked).
+            // (The empty statement keeps the address arithmetic of this rare path inside the branch: hoisted to
+            // the top of the job it occupied two dozen registers that then lived in scratch memory.)
+            int last = jb.sk - 1 - tile * kWBN;
+            asm volatile("" : "+s"(last));
             const unsigned char* t0 = reinterpret_cast<const unsigned char*>(src + (int64_t)tile * kWBN * stride);
+            const uint32_t row_bytes = (uint32_t)stride * 2u;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int row = min(16 * wave + 4 * j + ld_q, last);                 // row inside the tile
-                dma_to_lds_16_m0(t0, (uint32_t)(row * (int)stride * 2 + ((ld_c0 ^ j) << 4)), dst + j * 1024);
+                const uint32_t row = (uint32_t)min(16 * wave + 4 * j + ld_q, last);   // row inside the tile
+                dma_to_lds_16_m0(t0, row * row_bytes + (uint32_t)((ld_c0 ^ j) << 4), dst + j * 1024);
             }
         }
     };
@@ -224,22 +228,27 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     // ---- per-lane LDS read addresses for buffer 0 (absolute: the assembly loop uses them as they are) ----
     // K fragment of step s, key row 32t + n: chunk (2s + kg) ^ swz(n);  V^T fragment of d-tile dt: source lane s16 of
     // group g16 addresses key row 4(g16>>1) + (s16>>2) (+8 for the upper half), d = 32dt + 16(g16&1) + 4(s16&3)..+3
-    uint32_t rd_addr[16];             // [0..7] K per step, [8..11] V^T lower half per d-tile, [12..15] upper half
+    // Only the addresses of step 0 / d-tile 0 are kept: the one of step s / d-tile dt is that with s << 5 / dt << 6
+    // XORed in (the swizzle XORs exactly those bits).  (The empty statements keep the other fifteen from being
+    // computed once and held in registers for the whole kernel, where they pushed other values into scratch memory.)
+    uint32_t rd_k0, rd_vlo0, rd_vhi0;
     {
-        const uint32_t kbase = lds_address(k_lds), vbase = lds_address(v_lds);
-#pragma unroll
-        for (int s = 0; s < NS; ++s) rd_addr[s] = kbase + n * kWRow + (((2 * s + kg) ^ swz<D>(n)) << 4);
         const int g16 = lane >> 4, s16 = lane & 15;
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const int row = 4 * (g16 >> 1) + (s16 >> 2) + 8 * e;
-#pragma unroll
-            for (int dt = 0; dt < NDT; ++dt) {
-                const int d = 32 * dt + 16 * (g16 & 1) + 4 * (s16 & 3);
-                rd_addr[8 + 4 * e + dt] = vbase + row * kWRow + ((((d >> 3)) ^ swz<D>(row)) << 4) + (d & 7) * 2;
-            }
-        }
+        const int row = 4 * (g16 >> 1) + (s16 >> 2), d = 16 * (g16 & 1) + 4 * (s16 & 3);
+        rd_k0 = lds_address(k_lds) + n * kWRow + ((kg ^ swz<D>(n)) << 4);
+        rd_vlo0 = lds_address(v_lds) + row * kWRow + (((d >> 3) ^ swz<D>(row)) << 4) + (d & 7) * 2;
+        rd_vhi0 = lds_address(v_lds) + (row + 8) * kWRow + (((d >> 3) ^ swz<D>(row + 8)) << 4) + (d & 7) * 2;
     }
+    auto rd_k = [&](int s) {
+        uint32_t a = rd_k0;
+        asm volatile("" : "+v"(a));
+        return a ^ (uint32_t)(s << 5);
+    };
+    auto rd_v = [&](int e, int dt) {
+        uint32_t a = e ? rd_vhi0 : rd_vlo0;
+        asm volatile("" : "+v"(a));
+        return a ^ (uint32_t)(dt << 6);
+    };
 
     // A operand of the row-sum MFMA (see prefill_fwd.hip): row 0 sums k = 0..7, 16..23 (query c), row 1 the rest (c + 16)
     uint32_t sum_word;
@@ -265,12 +274,19 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         const int nt = tiles_of(jb);
         if (nt > 0) issue_k(jb, 0, 0);
         const int qw0 = jb.q0 + 64 * wave;
+        // (the row addresses are derived from a value the compiler cannot trace, so that it computes them here and
+        // not at the top of the job, where sixteen 64-bit addresses would have to wait in registers)
+        // (an offset, not the pointer, goes through the empty statement: a pointer would come back without its
+        // address space and the loads would become flat ones, which also count as LDS operations)
+        int64_t my_off = (int64_t)(qw0 + r0) * p.qs[2] + c16 * 8;
+        asm volatile("" : "+v"(my_off));
+        const __bf16* my_rows = jb.qb + my_off;
 #pragma unroll
         for (int i = 0; i < 64 / kRowsPerPass; ++i) {
             const int r = i * kRowsPerPass + r0;
             q_rows[i] = u32x4{0u, 0u, 0u, 0u};
             if (qw0 + i * kRowsPerPass < jb.sq) {          // (wave-uniform: see row_passes)
-                if (qw0 + r < jb.sq) q_rows[i] = *reinterpret_cast<const u32x4*>(jb.qb + (int64_t)(qw0 + r) * p.qs[2] + c16 * 8);
+                if (qw0 + r < jb.sq) q_rows[i] = *reinterpret_cast<const u32x4*>(my_rows + (int64_t)(i * kRowsPerPass) * p.qs[2]);
             }
         }
         if (nt > 1) issue_k(jb, 1, 1);
@@ -365,7 +381,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             bf16x8 qf[NS];
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
-                kf[s] = lds_load_at<u32x4>(rd_addr[s] + buf * kWTile + t * 32 * kWRow);
+                kf[s] = lds_load_at<u32x4>(rd_k(s) + buf * kWTile + t * 32 * kWRow);
                 qf[s] = qfrag(c, s);
             }
 #pragma unroll
@@ -411,8 +427,8 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 bf16x8 vf[NDT];
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt)
-                    vf[dt] = join_bf16x8(lds_read_tr16_at(rd_addr[8 + dt] + buf * kWTile + 16 * u * kWRow),
-                                         lds_read_tr16_at(rd_addr[12 + dt] + buf * kWTile + 16 * u * kWRow));
+                    vf[dt] = join_bf16x8(lds_read_tr16_at(rd_v(0, dt) + buf * kWTile + 16 * u * kWRow),
+                                         lds_read_tr16_at(rd_v(1, dt) + buf * kWTile + 16 * u * kWRow));
                 acc_sum<c>(sum_a, pf);
                 acc_pv<c, 0>(vf[0], pf);
                 acc_pv<c, 1>(vf[1], pf);
@@ -485,7 +501,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             // vector operands: read once when the block starts, scratch registers of the block afterwards
             float v_nb0 = nb[0], v_nb1 = nb[1];
             int v_thr0 = min(n + diag, sk - 1 - k0m) - 4 * kg, v_thr1 = min(n + 32 + diag, sk - 1 - k0m) - 4 * kg;
-            uint32_t v_sum = sum_word, v_k0 = rd_addr[0], v_vlo = rd_addr[8], v_vhi = rd_addr[12];
+            uint32_t v_sum = sum_word, v_k0 = rd_k0, v_vlo = rd_vlo0, v_vhi = rd_vhi0;
             uint32_t v_rowk = dma_row_k, v_rowv = dma_row_v, v_c0s = (uint32_t)(ld_c0 << 4), v_q = q_addr;
             int status;
             int tile_s = __builtin_amdgcn_readfirstlane(tile);
@@ -562,12 +578,15 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         break;
         }   // attempts
         // ---- output rows leave whole, through the slab ----
+        int64_t out_off = (int64_t)(qw0 + r0) * p.os[2] + c16 * 8;
+        asm volatile("" : "+v"(out_off));                  // (as for the query rows: addresses computed here, not earlier)
+        __bf16* my_out = cur.ob + out_off;
 #pragma unroll
         for (int i = 0; i < 64 / kRowsPerPass; ++i) {
             const int r = i * kRowsPerPass + r0;
             const u32x4 w = *reinterpret_cast<const u32x4*>(slab + r * kWORow + c16 * 16);
             if (qw0 + i * kRowsPerPass < sq) {             // (wave-uniform: see row_passes)
-                if (qw0 + r < sq) *reinterpret_cast<u32x4*>(cur.ob + (int64_t)(qw0 + r) * p.os[2] + c16 * 8) = w;
+                if (qw0 + r < sq) *reinterpret_cast<u32x4*>(my_out + (int64_t)(i * kRowsPerPass) * p.os[2]) = w;
             }
         }
         prev_stores = row_passes(cur);
