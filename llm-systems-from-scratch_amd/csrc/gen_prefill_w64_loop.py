@@ -61,7 +61,7 @@ Register map (physical, fixed; the block loads them itself from its operands, se
   a[200:215] K fragments (4 in flight), a[216:247] V^T fragments (8: 2 slices x 4 d-tiles): LDS reads land in
   AGPRs directly and the MFMAs take them as A operands, which leaves the vector registers to the compiler
   s[36:37] / s[38:39] global address of the wavefront's first DMA row of K[t+2] / V[t+1] (advanced per tile),
-  s[40:41] scratch, s42 "a row sum reached 2"; every other scalar is a named operand
+  s40 / s41 bytes from one tile to the next in K / V, s42 "a row sum reached 2"; every other scalar is a named operand
 """
 import os
 
@@ -88,7 +88,7 @@ LREG = {"A": 128, "B": 132}
 QREG = {"A": 136, "B": 168}
 N_ACC = 136                         # a[0:135]: what ordinary code reaches through the snippets
 N_AGPRS = 248
-KPTR, VPTR, PTMP, FLAG = 36, 38, 40, 42
+KPTR, VPTR, FLAG, KSTEP16, VSTEP16 = 36, 38, 42, 40, 41
 Q_SLAB_ROW = 272                    # bytes per row of the query staging slab (256 + 16 of padding)
 K_TILE = 16384                      # bytes of one K (or V) tile in LDS: 64 rows x 256 bytes
 ROW = 256
@@ -258,22 +258,18 @@ def check_sums(e, flagged_label):
 
 def dma_chunks(which, buf):
     """Instruction groups that request K[t+2] into K buffer `buf` ("k" in which) and V[t+1] into V buffer buf ^ 1
-    ("v" in which), and advance the pointers by a tile."""
+    ("v" in which), and advance the pointers by a tile.  The four loads of a tensor share the scalar base: the
+    distance between them (four rows) is part of the lane offsets."""
     chunks = []
-    for name, j0, ptr, lds0 in (("v", 4, VPTR, 2 * K_TILE + (buf ^ 1) * K_TILE), ("k", 0, KPTR, buf * K_TILE)):
+    for name, j0, ptr, step, lds0 in (("v", 4, VPTR, VSTEP16, 2 * K_TILE + (buf ^ 1) * K_TILE), ("k", 0, KPTR, KSTEP16, buf * K_TILE)):
         if name not in which:
             continue
-        chunks.append([f"s_mov_b64 s[{PTMP}:{PTMP + 1}], s[{ptr}:{ptr + 1}]"])
         for j in range(4):
             c = [f"s_add_u32 m0, %[ldsdst], {lds0 + j * 1024}", "s_nop 0"]
             if "nodma" not in ABL:
-                c.append(f"global_load_lds_dwordx4 v{DMAOFF + j0 + j}, s[{PTMP}:{PTMP + 1}]")
-            if j < 3:
-                c += [f"s_add_u32 s{PTMP}, s{PTMP}, %[{name}step]", f"s_addc_u32 s{PTMP + 1}, s{PTMP + 1}, 0"]
+                c.append(f"global_load_lds_dwordx4 v{DMAOFF + j0 + j}, s[{ptr}:{ptr + 1}]")
             chunks.append(c)
-        chunks.append([f"s_lshl_b32 %[t2], %[{name}step], 4",          # a tile is 64 rows = 16 DMA steps of 4 rows
-                       f"s_add_u32 s{ptr}, s{ptr}, %[t2]",
-                       f"s_addc_u32 s{ptr + 1}, s{ptr + 1}, 0"])
+        chunks.append([f"s_add_u32 s{ptr}, s{ptr}, s{step}", f"s_addc_u32 s{ptr + 1}, s{ptr + 1}, 0"])
     return chunks
 
 
@@ -398,6 +394,16 @@ def half_step(e, *, s_part, o_part, valu, hold):
     m = []
     for i in range(8):
         slot = i % 4
+        # the fragments of steps i and i + 1 are waited for together (they were requested long ago: half as many
+        # wait instructions)
+        pair_needs = None
+        if i % 2 == 0:
+            pair_needs = ()
+            for k in (i, i + 1):
+                if s_part:
+                    pair_needs += (KF + 4 * (k % 4),)
+                if o_part:
+                    pair_needs += vneeds(k)
         if s_part:
             kbuf, kh, k_next = s_part
 
@@ -406,7 +412,8 @@ def half_step(e, *, s_part, o_part, valu, hold):
                     k_read(e, kbuf, kh, i + 4, slot)
                 elif k_next:
                     k_next(i, slot)
-            m.append((mfma_s("A", kh, slot, i), (KF + 4 * slot,), None))
+            m.append((mfma_s("A", kh, slot, i), pair_needs, None))
+            pair_needs = None
             m.append((mfma_s("B", kh, slot, i), None, k_refill))
         if o_part:
             ph, v_next = o_part
@@ -417,7 +424,7 @@ def half_step(e, *, s_part, o_part, valu, hold):
             def v_refill(i=i, v_next=v_next):
                 if v_next:
                     v_next(i)
-            m.append((mfma_o("A", i, P[ph]["A"] + 4 * (i // 4)), vneeds(i), None))
+            m.append((mfma_o("A", i, P[ph]["A"] + 4 * (i // 4)), pair_needs, None))
             m.append((mfma_o("B", i, P[ph]["B"] + 4 * (i // 4)), None, v_refill))
     return plan(m, valu, hold)
 
@@ -547,10 +554,17 @@ def entry(e):
         e.raw(f"v_xor_b32 v{VOFF + dt}, {hex(dt << 6)}, %[vlo0]")
         e.raw(f"v_xor_b32 v{VOFF + 4 + dt}, {hex(dt << 6)}, %[vhi0]")
     e.raw("s_waitcnt lgkmcnt(0)")                      # the Q^T fragments are in; %[qaddr] is scratch from here on
-    for j in range(4):
+    for j in range(4):                                 # load j of a tile: swizzled chunk, row part, and j * four rows
         e.raw(f"v_xor_b32 {TMP}, {hex(j << 4)}, %[c0s]")
         e.raw(f"v_add_u32 v{DMAOFF + j}, {TMP}, %[rowk]")
         e.raw(f"v_add_u32 v{DMAOFF + 4 + j}, {TMP}, %[rowv]")
+        if j:
+            e.raw(f"s_mul_i32 s{KSTEP16}, %[kstep], {j}")
+            e.raw(f"s_mul_i32 s{VSTEP16}, %[vstep], {j}")
+            e.raw(f"v_add_u32 v{DMAOFF + j}, s{KSTEP16}, v{DMAOFF + j}")
+            e.raw(f"v_add_u32 v{DMAOFF + 4 + j}, s{VSTEP16}, v{DMAOFF + 4 + j}")
+    e.raw(f"s_lshl_b32 s{KSTEP16}, %[kstep], 4")          # a tile is 64 rows = 16 steps of 4 rows
+    e.raw(f"s_lshl_b32 s{VSTEP16}, %[vstep], 4")
     e.raw(f"s_mov_b32 s{KPTR}, %[klo]")
     e.raw(f"s_mov_b32 s{KPTR + 1}, %[khi]")
     e.raw(f"s_mov_b32 s{VPTR}, %[vlo]")
