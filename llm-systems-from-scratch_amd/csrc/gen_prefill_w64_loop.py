@@ -202,29 +202,63 @@ def exp_ops(h, mask, blocks="AB"):
     return ops
 
 
-def plan(mfmas, valu, hold=0):
-    """Distributes the vector instructions evenly behind the MFMAs, none behind the first `hold` MFMAs: the vector
-    work reads accumulators that the MFMAs just before it wrote, and the hardware does not interlock that dependency
-    (a result is visible 8 passes after its MFMA started; `hold` MFMAs of other chains in between cover that).
+def issue_cost(text):
+    """Issue time of a non-MFMA instruction in cycles, as the microbenchmarks show it next to an MFMA stream."""
+    return 8 if text.startswith("v_exp") else 4
+
+
+def plan(e, mfmas, valu, hold=0, span=None):
+    """Distributes the vector instructions behind the MFMAs so that every gap between two MFMAs carries about the same
+    issue time (a wavefront issues one instruction per four cycles, and what does not fit under an MFMA delays the
+    next one): the LDS reads and waits that belong to fixed MFMAs are counted first, the vector instructions fill
+    up to the average.  None goes behind the first `hold` MFMAs -- the vector work reads accumulators that the MFMAs
+    just before it wrote, and the hardware does not interlock that dependency (a result is visible 8 passes after
+    its MFMA started; `hold` MFMAs of other chains in between cover that) -- and none behind MFMA `span` and later.
     `mfmas` entries are (text, needs, post): registers whose LDS reads must have returned, and a callback run right
     after the MFMA (it issues the LDS reads that refill the registers the MFMA has just consumed).
-    Returns entries (text, needs, post, vector instructions that follow)."""
-    n, nv, vi = len(mfmas), len(valu), 0
-    out = []
+    Returns entries (text, needs, post, vector instructions that follow, issue time of the gap's fixed part --
+    doubled behind the short row-sum MFMAs)."""
+    n = len(mfmas)
+    span = n if span is None else span
+    fixed = [0] * n
     for i, (text, needs, post) in enumerate(mfmas):
-        upto = (i + 1 - hold) * nv // (n - hold) if i >= hold else 0
-        out.append((text, needs, post, valu[vi:upto]))
-        vi = max(vi, upto)
-    assert vi == nv
+        if post:                                   # dry run of the callback: how many instructions does it issue?
+            n0, p0 = len(e.lines), list(e.pending)
+            post()
+            fixed[i] += sum(issue_cost(t) for t in e.lines[n0:])
+            del e.lines[n0:]
+            e.pending = p0
+        if needs and i:
+            fixed[i - 1] += 4                      # the wait in front of this MFMA sits in the previous gap
+    weight = [0.5 if "16x16x32" in t or t.startswith("s_nop") else 1.0 for t, _, _ in mfmas]
+    elig = range(hold, span)
+    total = sum(fixed[i] for i in elig) + sum(issue_cost(v) for v in valu)
+    wsum = sum(weight[i] for i in elig) or 1.0
+    out, vi, cum, wcum = [], 0, 0.0, 0.0
+    for i, (text, needs, post) in enumerate(mfmas):
+        mine = []
+        if hold <= i < span:
+            cum += fixed[i]
+            wcum += weight[i]
+            target = total * wcum / wsum
+            while vi < len(valu) and (i == span - 1 or cum + issue_cost(valu[vi]) / 2 <= target):
+                mine.append(valu[vi])
+                cum += issue_cost(valu[vi])
+                vi += 1
+        out.append((text, needs, post, mine, fixed[i] * (2.0 if weight[i] < 1.0 else 1.0)))
+    assert vi == len(valu)
     return out
 
 
 def emit(e, entries, extras=()):
     """Emits planned entries; `extras` (groups of instructions that must stay together, e.g. the m0 write and its
-    direct-to-LDS load) are spread evenly behind the MFMAs as well."""
+    direct-to-LDS load) go behind the MFMAs too, again so that the gaps carry equal issue time."""
     extras = list(extras)
-    n, ne, xi = len(entries), len(extras), 0
-    for i, (text, needs, post, valu) in enumerate(entries):
+    cost_x = [sum(issue_cost(t) for t in x) for x in extras]
+    gap = [f + sum(issue_cost(v) for v in valu) for (_, _, _, valu, f) in entries]
+    total = sum(gap) + sum(cost_x)
+    n, xi, cum = len(entries), 0, 0.0
+    for i, (text, needs, post, valu, _) in enumerate(entries):
         if needs:
             e.need(*needs)
         e.raw(text)
@@ -232,10 +266,12 @@ def emit(e, entries, extras=()):
             post()
         for v in valu:
             e.raw(v)
-        upto = (i + 1) * ne // n
-        while xi < upto:
+        cum += gap[i]
+        target = total * (i + 1) / n
+        while xi < len(extras) and (i == n - 1 or cum + cost_x[xi] / 2 <= target):
             for x in extras[xi]:
                 e.raw(x)
+            cum += cost_x[xi]
             xi += 1
 
 
@@ -329,7 +365,7 @@ def single_tile(e, buf, kind, start):
                 k_read(e, buf, 1, s - 4, slot)
         m.append((mfma_s("A", 0, slot, s), (KF + 4 * slot,), None))
         m.append((mfma_s("B", 0, slot, s), None, refill))
-    emit(e, plan(m, []))
+    emit(e, plan(e, m, []))
     e.raw("; S(.,1) | E(.,0)")
     m = []
     for s in range(8):
@@ -341,7 +377,7 @@ def single_tile(e, buf, kind, start):
         for ci, c in enumerate(h1_blocks):
             m.append((mfma_s(c, 1, slot, s), (KF + 4 * slot,) if ci == 0 else None,
                       refill if ci == len(h1_blocks) - 1 else None))
-    emit(e, plan(m, exp_ops(0, mask0), hold=1 if diag else 3))
+    emit(e, plan(e, m, exp_ops(0, mask0), hold=1 if diag else 3))
 
     def first_v_reads():
         for j in range(8):
@@ -358,7 +394,7 @@ def single_tile(e, buf, kind, start):
             v_read(e, buf, 1, j)
         m.append((mfma_o("A", j, P[0]["A"] + 4 * (j // 4)), vneeds(j), None))
         m.append((mfma_o("B", j, P[0]["B"] + 4 * (j // 4)), None, refill))
-    emit(e, plan(m, exp_ops(1, mask1, h1_blocks), hold=3))
+    emit(e, plan(e, m, exp_ops(1, mask1, h1_blocks), hold=3))
     e.raw("s_nop 1")
     e.raw("; O(.,1); the next tile's first K fragments are requested half way")
     m = []
@@ -374,7 +410,7 @@ def single_tile(e, buf, kind, start):
         for ci, c in enumerate(h1_blocks):
             m.append((mfma_o(c, j, P[1][c] + 4 * (j // 4)), vneeds(j) if ci == 0 else None,
                       next_k if ci == len(h1_blocks) - 1 else None))
-    emit(e, plan(m, []))
+    emit(e, plan(e, m, []))
     e.raw(f"v_subrev_u32 v{THR['A']}, 64, v{THR['A']}")     # the next tile's keys are 64 further along
     e.raw(f"v_subrev_u32 v{THR['B']}, 64, v{THR['B']}")
     e.raw("s_add_u32 %[tile], %[tile], 1")
@@ -383,7 +419,7 @@ def single_tile(e, buf, kind, start):
     e.raw("s_branch 20b")
 
 
-def half_step(e, *, s_part, o_part, valu, hold):
+def half_step(e, *, s_part, o_part, valu, hold, span=None):
     """The MFMAs of one pipeline half-step as planned entries.
     s_part: (K buffer, half, k_next(i, slot) called after step i >= 4) -- S(., half) of the tile in that buffer; the
             fragments of steps 0..3 are in flight, those of steps 4..7 are requested as the slots come free
@@ -426,7 +462,7 @@ def half_step(e, *, s_part, o_part, valu, hold):
                     v_next(i)
             m.append((mfma_o("A", i, P[ph]["A"] + 4 * (i // 4)), pair_needs, None))
             m.append((mfma_o("B", i, P[ph]["B"] + 4 * (i // 4)), None, v_refill))
-    return plan(m, valu, hold)
+    return plan(e, m, valu, hold, span)
 
 
 def pipeline(e, b, start, h0_start, dry=False):
@@ -481,7 +517,7 @@ def pipeline(e, b, start, h0_start, dry=False):
     e.raw(f"; ---- pipeline prologue, tile in buffers {b}: S(t,0)")
     emit(e, half_step(e, s_part=(b, 0, lambda i, slot: k_read(e, b, 1, i - 4, slot)), o_part=None, valu=[], hold=0))
     e.raw("; S(t,1) | E(t,0), boundary inside")
-    pro = half_step(e, s_part=(b, 1, k_after_pro), o_part=None, valu=exp_ops(0, NONE), hold=3)
+    pro = half_step(e, s_part=(b, 1, k_after_pro), o_part=None, valu=exp_ops(0, NONE), hold=3, span=12)
     emit(e, pro[:12])                                      # steps 0..5
     at_m = tail_variants(pro[12:], f"5{b}0", f"4{b}4f")
 
@@ -489,7 +525,7 @@ def pipeline(e, b, start, h0_start, dry=False):
     e.raw(f"4{b}1:")
     e.raw(f"; ---- H0, tile in buffers {b}: S(t,1) | E(t,0) | O(t-1,1), boundary inside")
     e.pending = list(h0_start)
-    h0 = half_step(e, s_part=(b, 1, k_after), o_part=(1, v_after), valu=exp_ops(0, NONE), hold=0)
+    h0 = half_step(e, s_part=(b, 1, k_after), o_part=(1, v_after), valu=exp_ops(0, NONE), hold=0, span=28)
     emit(e, h0[:28])                                       # steps 0..5
     at_m2 = tail_variants(h0[28:], f"5{b}1", f"4{b}4f")
     assert dry or at_m == at_m2, (at_m, at_m2)
@@ -527,7 +563,7 @@ def pipeline(e, b, start, h0_start, dry=False):
     for s in range(4):
         k_read(e, o, 0, s, s)
     epi = half_step(e, s_part=None, o_part=(1, None), valu=[], hold=0)
-    emit(e, [(t, None, p_, v) for (t, _, p_, v) in epi])
+    emit(e, [(t, None, p_, v, f) for (t, _, p_, v, f) in epi])
     e.raw("s_add_u32 %[tile], %[tile], 1")
     assert e.pending == start, (e.pending, start)
     e.raw("s_branch 20b")
