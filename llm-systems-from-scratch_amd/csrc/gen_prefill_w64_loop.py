@@ -198,7 +198,7 @@ def exp_ops(h, mask, blocks="AB"):
             ops += pend
             pend = [f"v_cvt_pk_bf16_f32 v{dst + w}, {t0}, {t1}"]
             i += 1
-    ops += ["s_nop 0"] + pend
+    ops += pend          # (the packing of the word before sits between the last exponentials and their packing)
     return ops
 
 
