@@ -419,14 +419,16 @@ def single_tile(e, buf, kind, start):
     e.raw("s_branch 20b")
 
 
-def half_step(e, *, s_part, o_part, valu, hold, span=None):
+def half_step(e, *, s_part, o_part, valu, hold, span=None, a_posts=None):
     """The MFMAs of one pipeline half-step as planned entries.
     s_part: (K buffer, half, k_next(i, slot) called after step i >= 4) -- S(., half) of the tile in that buffer; the
             fragments of steps 0..3 are in flight, those of steps 4..7 are requested as the slots come free
     o_part: (P half, v_next(j) called after fragment j is consumed) -- O += V^T fragments 0..7 (already requested)
             . P(., half)
+    a_posts: {("S", i) or ("O", i): callback} run behind the block-A MFMA of step i
     Order: per step i the two score MFMAs (blocks A, B), then the two (with row sums: four) accumulations of
     fragment i."""
+    a_posts = a_posts or {}
     m = []
     for i in range(8):
         slot = i % 4
@@ -448,7 +450,7 @@ def half_step(e, *, s_part, o_part, valu, hold, span=None):
                     k_read(e, kbuf, kh, i + 4, slot)
                 elif k_next:
                     k_next(i, slot)
-            m.append((mfma_s("A", kh, slot, i), pair_needs, None))
+            m.append((mfma_s("A", kh, slot, i), pair_needs, a_posts.get(("S", i))))
             pair_needs = None
             m.append((mfma_s("B", kh, slot, i), None, k_refill))
         if o_part:
@@ -460,7 +462,7 @@ def half_step(e, *, s_part, o_part, valu, hold, span=None):
             def v_refill(i=i, v_next=v_next):
                 if v_next:
                     v_next(i)
-            m.append((mfma_o("A", i, P[ph]["A"] + 4 * (i // 4)), pair_needs, None))
+            m.append((mfma_o("A", i, P[ph]["A"] + 4 * (i // 4)), pair_needs, a_posts.get(("O", i))))
             m.append((mfma_o("B", i, P[ph]["B"] + 4 * (i // 4)), None, v_refill))
     return plan(e, m, valu, hold, span)
 
@@ -469,39 +471,45 @@ def pipeline(e, b, start, h0_start, dry=False):
     """The software pipeline over unmasked tiles for tiles whose buffers are `b` (code for both parities is
     generated; a tile step ends by jumping to the other parity's H0).  Returns the reads H1 leaves in flight."""
     o = b ^ 1
-    # After the barrier of boundary(t): K[t+1] half 0 fragments 0, 1 and V[t] half 0 fragments 0..5 are requested at
-    # once (their registers are free); slots 2, 3 and fragments 6, 7 follow as steps 6, 7 of H0 consume them.
+    # After the barrier of boundary(t) the first reads of what has landed -- K[t+1] half 0 and V[t] half 0 -- go out
+    # between the last eight MFMAs of H0 (steps 6, 7, whose own fragments are in registers): fragments 0, 1 of both at
+    # once, the others one per MFMA, K slots 2, 3 and V^T fragments 6, 7 as those steps free their registers.  The
+    # order of the reads is the same in the prologue, which has only the score MFMAs to put them behind.
     def k_after(i, slot):
         if i >= 6:
             k_read(e, o, 0, slot, slot)
-
-    def k_after_pro(i, slot):               # the prologue has no O part: fragments 6, 7 follow the K refills
-        if i >= 6:
-            k_read(e, o, 0, slot, slot)
-            v_read(e, b, 0, i)
 
     def v_after(j):
         if j >= 6:
             v_read(e, b, 0, j)
 
+    tail_posts = {("S", 6): lambda: v_read(e, b, 0, 2), ("O", 6): lambda: v_read(e, b, 0, 3),
+                  ("S", 7): lambda: v_read(e, b, 0, 4), ("O", 7): lambda: v_read(e, b, 0, 5)}
+
+    def k_after_pro(i, slot):
+        if i >= 6:
+            k_read(e, o, 0, slot, slot)
+            v_read(e, b, 0, 2 * i - 9)          # 3 behind step 6, 5 behind step 7
+            v_read(e, b, 0, i)
+
+    pro_posts = {("S", 6): tail_posts[("S", 6)], ("S", 7): tail_posts[("S", 7)]}
+
     def first_reads():
         k_read(e, o, 0, 0, 0)
         k_read(e, o, 0, 1, 1)
-        for j in range(6):
-            v_read(e, b, 0, j)
+        v_read(e, b, 0, 0)
+        v_read(e, b, 0, 1)
 
     def tail_variants(entries, tagbase, join_label):
-        """boundary(t) and the rest of the half-step, in three variants by which requests exist."""
+        """boundary(t) and the rest of the half-step, in two variants: with and without the request of K[t+2]
+        (V[t+1] is requested in H1)."""
         wait_and_meet(e)
         first_reads()
         e.raw("s_add_u32 %[t2], %[tile], 2")
         e.raw("s_cmp_lt_u32 %[t2], %[n_tiles]")
-        e.raw(f"s_cbranch_scc1 {tagbase}2f")               # K[t+2] and V[t+1] exist
-        e.raw("s_add_u32 %[t2], %[tile], 1")
-        e.raw("s_cmp_lt_u32 %[t2], %[n_tiles]")
-        e.raw(f"s_cbranch_scc1 {tagbase}1f")               # only V[t+1]
+        e.raw(f"s_cbranch_scc1 {tagbase}1f")
         saved, result = list(e.pending), None
-        for vi, which in ((0, ""), (1, "v"), (2, "kv")):
+        for vi, which in ((0, ""), (1, "k")):
             e.pending = list(saved)
             if vi:
                 e.raw(f"{tagbase}{vi}:")
@@ -517,7 +525,7 @@ def pipeline(e, b, start, h0_start, dry=False):
     e.raw(f"; ---- pipeline prologue, tile in buffers {b}: S(t,0)")
     emit(e, half_step(e, s_part=(b, 0, lambda i, slot: k_read(e, b, 1, i - 4, slot)), o_part=None, valu=[], hold=0))
     e.raw("; S(t,1) | E(t,0), boundary inside")
-    pro = half_step(e, s_part=(b, 1, k_after_pro), o_part=None, valu=exp_ops(0, NONE), hold=3, span=12)
+    pro = half_step(e, s_part=(b, 1, k_after_pro), o_part=None, valu=exp_ops(0, NONE), hold=3, span=12, a_posts=pro_posts)
     emit(e, pro[:12])                                      # steps 0..5
     at_m = tail_variants(pro[12:], f"5{b}0", f"4{b}4f")
 
@@ -525,7 +533,8 @@ def pipeline(e, b, start, h0_start, dry=False):
     e.raw(f"4{b}1:")
     e.raw(f"; ---- H0, tile in buffers {b}: S(t,1) | E(t,0) | O(t-1,1), boundary inside")
     e.pending = list(h0_start)
-    h0 = half_step(e, s_part=(b, 1, k_after), o_part=(1, v_after), valu=exp_ops(0, NONE), hold=0, span=28)
+    h0 = half_step(e, s_part=(b, 1, k_after), o_part=(1, v_after), valu=exp_ops(0, NONE), hold=0, span=28,
+                   a_posts=tail_posts)
     emit(e, h0[:28])                                       # steps 0..5
     at_m2 = tail_variants(h0[28:], f"5{b}1", f"4{b}4f")
     assert dry or at_m == at_m2, (at_m, at_m2)
@@ -536,9 +545,9 @@ def pipeline(e, b, start, h0_start, dry=False):
     e.raw("s_add_u32 %[t2], %[tile], 1")
     e.raw("s_cmp_ge_u32 %[t2], %[n_pipe]")
     e.raw(f"s_cbranch_scc1 4{b}6f")
-    e.raw(f"; ---- H1, tile in buffers {b}: S(t+1,0) | E(t,1) | O(t,0)")
+    e.raw(f"; ---- H1, tile in buffers {b}: S(t+1,0) | E(t,1) | O(t,0); V[t+1] (it exists) is requested on the way")
     emit(e, half_step(e, s_part=(o, 0, lambda i, slot: k_read(e, o, 1, i - 4, slot)),
-                      o_part=(0, lambda j: v_read(e, b, 1, j)), valu=exp_ops(1, NONE), hold=0))
+                      o_part=(0, lambda j: v_read(e, b, 1, j)), valu=exp_ops(1, NONE), hold=0), dma_chunks("v", b))
     leaves = list(e.pending)
     check_sums(e, f"4{b}7f")
     e.raw("s_add_u32 %[tile], %[tile], 1")
@@ -550,6 +559,12 @@ def pipeline(e, b, start, h0_start, dry=False):
     e.raw(f"4{b}6:")
     e.pending = list(at_m2)
     e.raw(f"; ---- H1 tail, tile in buffers {b}: E(t,1) | O(t,0)")
+    e.raw("s_cmp_ge_u32 %[t2], %[n_tiles]")               # (t2 = t + 1) no tile t+1: no V[t+1] to request
+    e.raw(f"s_cbranch_scc1 6{b}9f")
+    for c in dma_chunks("v", b):
+        for x in c:
+            e.raw(x)
+    e.raw(f"6{b}9:")
     emit(e, half_step(e, s_part=None, o_part=(0, lambda j: v_read(e, b, 1, j)), valu=exp_ops(1, NONE), hold=0))
     check_sums(e, f"4{b}9f")
     e.raw(f"s_branch 4{b}5f")
