@@ -1,6 +1,8 @@
 // Producers of the paged KV cache: interleaved-pair RoPE + scatter of new K/V rows into
 // cache blocks, and per-(block, kv head) fp8-e4m3 quantisation of cache blocks.
 // Both are plain streaming kernels (HBM-bound, a few bytes per element).
+#include <algorithm>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -77,13 +79,14 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeCacheParams p) 
 // Requires D % 8 == 0, token strides that are multiples of 8 elements and 16-byte aligned bases.
 // The grid covers the work once (workgroups in dispatch order walk through memory as one window).
 constexpr int kRopeHeads = 4;
-__global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParams p, int n_hu) {
+// (block, n_blocks: this workgroup's index among the workgroups that share the work, and their number)
+__device__ __forceinline__ void rope_and_cache_vec8_body(const RopeCacheParams& p, int n_hu, unsigned block, unsigned n_blocks) {
     const int groups = p.D / 8;
     const int half = p.D / 2;
     const int slots_per_tok = p.head_slots;
     const int64_t total = (int64_t)p.T * n_hu * groups;
-    for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
-         idx += (int64_t)gridDim.x * blockDim.x) {
+    for (int64_t idx = block * (int64_t)blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)n_blocks * blockDim.x) {
         const int c = (int)(idx % groups);
         const int hu = (int)((idx / groups) % n_hu);
         const int t = (int)(idx / ((int64_t)groups * n_hu));
@@ -129,6 +132,10 @@ __global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParam
             if (dst2[j]) __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(dst2[j]));
         }
     }
+}
+
+__global__ __launch_bounds__(256) void rope_and_cache_vec8_kernel(RopeCacheParams p, int n_hu) {
+    rope_and_cache_vec8_body(p, n_hu, blockIdx.x, gridDim.x);
 }
 
 // One wavefront per (block, kv head) slab of 16*D bf16: absmax -> scale = absmax/448 (1 for an
@@ -219,10 +226,10 @@ __device__ __forceinline__ void quantize8(const float (&x)[8], float sc, unsigne
 // win = 16 for a packed prefill (one run per window when sequences start at block boundaries),
 // win = 1 for a decode step (every token is its own run; all of them proceed in parallel).
 template <int D>
-__global__ __launch_bounds__(256) void rope_and_cache_fp8_kernel(RopeCacheFp8Params p, int win, int n_windows) {
+__device__ __forceinline__ void rope_and_cache_fp8_body(const RopeCacheFp8Params& p, int win, int n_windows, unsigned block) {
     constexpr int LPR = D / 8, RPP = 64 / LPR, NP = 16 / RPP;
     const int lane = threadIdx.x & 63;
-    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t w = (int64_t)block * 4 + (threadIdx.x >> 6);
     if (w >= (int64_t)n_windows * 2 * p.Hkv) return;
     const int window = (int)(w / (2 * p.Hkv));
     const int rem = (int)(w % (2 * p.Hkv));
@@ -235,7 +242,11 @@ __global__ __launch_bounds__(256) void rope_and_cache_fp8_kernel(RopeCacheFp8Par
     const int base = window * win;
     const int64_t tok_i = (int64_t)base - 1 + lane;
     int64_t my_slot = -1;
-    if (lane < win + 16 && tok_i >= 0 && tok_i < p.T) my_slot = p.slots[tok_i];
+    int my_pos = 0;                    // (fetched with the slot: a key row's angles then wait for one load, not two)
+    if (lane < win + 16 && tok_i >= 0 && tok_i < p.T) {
+        my_slot = p.slots[tok_i];
+        if (!is_v) my_pos = p.positions[tok_i];
+    }
     if (my_slot >= p.n_slots) my_slot = -1;
     const int64_t prev_slot = __shfl_up(my_slot, 1, 64);
     // a token continues the run of the token before it when both sit in the same block at consecutive offsets
@@ -261,12 +272,14 @@ __global__ __launch_bounds__(256) void rope_and_cache_fp8_kernel(RopeCacheFp8Par
             const int j = pi * RPP + rip;                 // row of the block
 #pragma unroll
             for (int e = 0; e < 8; ++e) val[pi][e] = 0.f;
+            // (every lane takes part in the exchange: a lane outside the run reads some lane's value and drops it)
+            const int pos_j = __shfl(my_pos, (h + j - off0) & 63, 64);
             if (j >= off0 && j < off0 + n) {
                 const int tok = t + j - off0;
                 const __bf16* src = (is_v ? p.v_in + tok * p.v_tok : p.k_in + tok * p.k_tok) + (int64_t)hk * D + 8 * c;
                 u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src));
                 if (!is_v) {
-                    const int pos = min(max(p.positions[tok], 0), p.ctx_len - 1);
+                    const int pos = min(max(pos_j, 0), p.ctx_len - 1);
                     const f32x4 cs = *reinterpret_cast<const f32x4*>(p.freq + (int64_t)pos * half + 4 * c);
                     const f32x4 sn = *reinterpret_cast<const f32x4*>(p.freq + ((int64_t)p.ctx_len + pos) * half + 4 * c);
 #pragma unroll
@@ -323,6 +336,23 @@ __global__ __launch_bounds__(256) void rope_and_cache_fp8_kernel(RopeCacheFp8Par
             const int j = pi * RPP + rip;
             if (j >= off0 && j < off0 + n) quantize8(val[pi], sc, cache + j * D + 8 * c);
         }
+    }
+}
+
+// Queries (rotation only, bf16) and keys/values (rotation, quantisation) of one call in ONE launch: the workgroups
+// of the two kinds are dealt alternately (`ratio` query workgroups, then one key/value workgroup), so that the
+// latency-bound key/value wavefronts -- slot ids, then rows, then scales, each a dependent load -- run in the shadow
+// of the streaming query rows instead of after them.
+template <int D>
+__global__ __launch_bounds__(256) void rope_and_cache_fp8_fused_kernel(RopeCacheParams pq, int n_hu, unsigned q_blocks,
+                                                                      RopeCacheFp8Params p, int win, int n_windows,
+                                                                      unsigned kv_blocks, unsigned ratio) {
+    const unsigned group = blockIdx.x / (ratio + 1), pos = blockIdx.x % (ratio + 1);
+    if (pos < ratio) {
+        const unsigned b = group * ratio + pos;
+        if (b < q_blocks) rope_and_cache_vec8_body(pq, n_hu, b, q_blocks);
+    } else if (group < kv_blocks) {
+        rope_and_cache_fp8_body<D>(p, win, n_windows, group);
     }
 }
 
@@ -436,7 +466,7 @@ extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, cons
         return set_error(MI355_EINVAL, "rope_and_cache_fp8: tensors must be 16-byte aligned with token strides that are multiples of 8");
     if (T == 0) return MI355_OK;
     hipStream_t s = (hipStream_t)stream;
-    // queries (and, when asked for, the packed rotated keys): the bf16 kernel without a cache
+    // queries (and, when asked for, the packed rotated keys): the body of the bf16 kernel, without a cache
     RopeCacheParams pq{};
     pq.q_in = (const __bf16*)q_in;
     pq.k_in = (const __bf16*)k_in;
@@ -458,13 +488,6 @@ extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, cons
     pq.ctx_len = context_length;
     pq.head_slots = k_out ? Hq + Hkv : Hq;
     pq.n_slots = 0;
-    {
-        const int n_hu = (pq.head_slots + kRopeHeads - 1) / kRopeHeads;
-        const int64_t total = (int64_t)T * n_hu * (D / 8);
-        const int64_t blocks = (total + 255) / 256;
-        const unsigned grid = (unsigned)(blocks < 0x7fffffffLL ? blocks : 0x7fffffffLL);
-        hipLaunchKernelGGL(rope_and_cache_vec8_kernel, dim3(grid), dim3(256), 0, s, pq, n_hu);
-    }
     RopeCacheFp8Params p;
     p.k_in = (const __bf16*)k_in;
     p.v_in = (const __bf16*)v_in;
@@ -485,14 +508,25 @@ extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, cons
     // gives every wavefront a window of 16 tokens, which holds one run when sequences start on block boundaries
     const int win = T >= 4096 ? 16 : 1;
     const int n_windows = (T + win - 1) / win;
-    const int64_t wgs = ((int64_t)n_windows * 2 * Hkv + 3) / 4;
+    const int64_t kv_blocks = ((int64_t)n_windows * 2 * Hkv + 3) / 4;
+    const int n_hu = (pq.head_slots + kRopeHeads - 1) / kRopeHeads;
+    const int64_t q_blocks = ((int64_t)T * n_hu * (D / 8) + 255) / 256;
+    // one launch: `ratio` query workgroups, then one key/value workgroup, and so on
+    int64_t ratio = (q_blocks + kv_blocks - 1) / kv_blocks;
+    if (ratio < 1) ratio = 1;
+    const int64_t groups = std::max(kv_blocks, (q_blocks + ratio - 1) / ratio);
+    const int64_t wgs = groups * (ratio + 1);
     if (wgs > 0x7fffffff) return set_error(MI355_EINVAL, "rope_and_cache_fp8: too many tokens for one launch");
+    const dim3 grid((unsigned)wgs), block(256);
     if (D == 128)
-        hipLaunchKernelGGL(rope_and_cache_fp8_kernel<128>, dim3((unsigned)wgs), dim3(256), 0, s, p, win, n_windows);
+        hipLaunchKernelGGL(rope_and_cache_fp8_fused_kernel<128>, grid, block, 0, s, pq, n_hu, (unsigned)q_blocks, p, win,
+                           n_windows, (unsigned)kv_blocks, (unsigned)ratio);
     else if (D == 64)
-        hipLaunchKernelGGL(rope_and_cache_fp8_kernel<64>, dim3((unsigned)wgs), dim3(256), 0, s, p, win, n_windows);
+        hipLaunchKernelGGL(rope_and_cache_fp8_fused_kernel<64>, grid, block, 0, s, pq, n_hu, (unsigned)q_blocks, p, win,
+                           n_windows, (unsigned)kv_blocks, (unsigned)ratio);
     else
-        hipLaunchKernelGGL(rope_and_cache_fp8_kernel<32>, dim3((unsigned)wgs), dim3(256), 0, s, p, win, n_windows);
+        hipLaunchKernelGGL(rope_and_cache_fp8_fused_kernel<32>, grid, block, 0, s, pq, n_hu, (unsigned)q_blocks, p, win,
+                           n_windows, (unsigned)kv_blocks, (unsigned)ratio);
     const int rc = (int)hipGetLastError();
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;
