@@ -388,6 +388,42 @@ def test_prefill_split_keys_varlen_and_paged(ops, splits):
     assert (got.float() - unsplit.float()).abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_prefill_head_dim_128_two_kernels_agree_on_random_shapes(ops, seed):
+    """The 64-query kernel (hand-scheduled, pipelined tile loop) against the 8-wavefront kernel (reached through an
+    explicit boolean mask that says the same thing) and the oracle, on drawn shapes: ragged query and key counts,
+    Sk >= Sq (bottom-right diagonal), GQA, several query tiles per workgroup, and keys whose scores run away in
+    both directions at drawn places -- in unmasked tiles, on the diagonal, in the last partial tile -- so that the
+    loop is left and re-entered at every kind of tile."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    for case in range(5):
+        B = int(torch.randint(1, 3, (1,), generator=g))
+        Hkv = int(torch.randint(1, 3, (1,), generator=g))
+        Hq = Hkv * int(torch.randint(1, 3, (1,), generator=g))
+        Sq = int(torch.randint(1, 900, (1,), generator=g))
+        Sk = Sq + int(torch.randint(0, 700, (1,), generator=g)) * int(torch.randint(0, 2, (1,), generator=g))
+        causal = bool(torch.randint(0, 2, (1,), generator=g))
+        print(f"case: two kernels seed={seed} #{case} B={B} Hq={Hq} Hkv={Hkv} Sq={Sq} Sk={Sk} causal={causal}", flush=True)
+        q = (torch.randn(B, Hq, Sq, 128, generator=g)).to(torch.bfloat16)
+        k = torch.randn(B, Hkv, Sk, 128, generator=g)
+        v = (torch.randn(B, Hkv, Sk, 128, generator=g)).to(torch.bfloat16)
+        for _ in range(int(torch.randint(0, 6, (1,), generator=g))):          # runaway keys
+            j = int(torch.randint(0, Sk, (1,), generator=g))
+            n = int(torch.randint(1, 70, (1,), generator=g))
+            k[:, :, j:j + n] *= float(torch.tensor([6.0, 20.0, -15.0, 45.0])[int(torch.randint(0, 4, (1,), generator=g))])
+        k = k.to(torch.bfloat16)
+        ref = orc.prefill_reference(q, k, v, causal=causal)
+        fast = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=causal, kv_splits=1)
+        keep = torch.ones(Sq, Sk, dtype=torch.bool)
+        if causal:
+            keep = torch.tril(keep, diagonal=Sk - Sq)
+        slow = ops.scaled_dot_product_attention(q.cuda(), k.cuda().repeat_interleave(Hq // Hkv, 1),
+                                                v.cuda().repeat_interleave(Hq // Hkv, 1), keep.cuda())
+        torch.cuda.synchronize()
+        check(fast, ref, what=f"64-query kernel seed {seed} #{case}")
+        check(slow, ref, what=f"8-wavefront kernel seed {seed} #{case}")
+
+
 def _reference_module_tensors(x_proj, freq, num_heads, amp):
     """Q, K, V exactly as CausalMultiHeadSelfAttention.forward hands them to the attention call
     (llm-core/llm_core/model.py:362-378) from the three projection outputs (B, S, H*d): `rearrange` views, then
