@@ -1,4 +1,5 @@
-// Prefill forward for head_dim 128 (no mask or causal), one wavefront per SIMD, 64 queries per wavefront.
+// Prefill forward for head_dim 128 (no mask or causal; optional log-sum-exp output), one wavefront per SIMD, 64
+// queries per wavefront.
 //
 // One workgroup = 4 wavefronts = one tile of 256 queries of one (batch, head); a wavefront owns 64 query rows as two
 // column blocks A and B of 32.  It runs alone on its SIMD with the whole register file: the output accumulators
@@ -131,6 +132,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     struct Job {
         const __bf16 *qb, *kb, *vb;
         __bf16* ob;
+        float* lb;                       // row 0 of this (sequence, head) in the log-sum-exp output, or null
         int sq, sk, q0;
     };
     const int G = gridDim.x, bid = blockIdx.x;
@@ -165,6 +167,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 job_seq.kb = p.k + (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
                 job_seq.vb = p.v + (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
                 job_seq.ob = p.out + (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
+                job_seq.lb = p.lse ? p.lse + q_start + (int64_t)h * p.ls[1] : nullptr;
             } else {
                 job_seq.sq = p.Sq;
                 job_seq.sk = p.Sk;
@@ -172,6 +175,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 job_seq.kb = p.k + (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
                 job_seq.vb = p.v + (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
                 job_seq.ob = p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[1];
+                job_seq.lb = p.lse ? p.lse + (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1] : nullptr;
             }
             job_nq = (job_seq.sq + kWBM - 1) / kWBM;
             job_pair = lid % p.n_pairs;
@@ -555,6 +559,9 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         const auto store_block = [&](auto c_c) {
             constexpr int c = decltype(c_c)::value;
             const float inv = 1.0f / l_row[c];     // l == 0 (no key kept) -> NaN row, like the reference softmax
+            // sum_j exp(scale * s_j) = l * 2^(-nb)  ->  lse = ln2 * (log2 l - nb); no key kept -> -inf
+            if (cur.lb && kg == 0 && qw0 + 32 * c + n < sq)
+                cur.lb[qw0 + 32 * c + n] = l_row[c] > 0.f ? 0.69314718056f * (__log2f(l_row[c]) - nb[c]) : -INFINITY;
             unsigned char* mine = slab + (32 * c + n) * kWORow + 8 * kg;
             const auto store_dt = [&](auto dt_c) {
                 constexpr int dt = decltype(dt_c)::value;

@@ -38,7 +38,7 @@ struct PrefillParams {
     int64_t part_rows;
 };
 
-// The 64-queries-per-wavefront kernel (head_dim 128, no mask or causal, no lse): prefill_fwd_w64.hip.
+// The 64-queries-per-wavefront kernel (head_dim 128, no mask or causal): prefill_fwd_w64.hip.
 int launch_prefill_w64(const PrefillParams& p, hipStream_t stream);
 
 }  // namespace mi355

@@ -5,7 +5,8 @@ Tolerance: the kernels recompute P from bf16 inputs, round P and dS to bf16 for 
 round the results to bf16; against the fp32 oracle on the same bf16 inputs a gradient element is
 accepted within 1e-4 + 2e-2 * max|grad of that tensor| + 2e-2 |ref| (gradients of long sequences sum many
 terms, so the absolute part scales with the tensor), and the relative RMS error must stay below 1.5 %.
-lse: |got - ref| <= 2e-3 + 1e-3 |ref|.
+lse: |got - ref| <= 3e-3 + 1e-3 |ref| (the kernels sum the weights as rounded to bf16 -- exactly what multiplies V --
+so a row whose weights all round the same way is off by up to 2^-9 = 0.002 in its log-sum-exp).
 """
 import pytest
 import torch
@@ -114,17 +115,30 @@ def test_backward_varlen_equals_per_sequence(ops):
     check_grad("dv", vg.grad, dv_ref)
 
 
-def test_forward_lse_matches_oracle(ops):
-    print("case: forward lse", flush=True)
+@pytest.mark.parametrize("D", [64, 128])
+def test_forward_lse_matches_oracle(ops, D):
+    """head_dim 64: the 8-wavefront kernel; 128: the 64-query kernel, whose log-sum-exp comes from its row sums and
+    the exponent reference that went into them -- also after that reference has moved (keys with runaway scores),
+    for ragged packed sequences, and for rows past the end of a partial query tile."""
+    print(f"case: forward lse D={D}", flush=True)
     from mi355_attn import ops as raw
-    B, Hq, Hkv, S, D = 2, 4, 2, 300, 64
+    B, Hq, Hkv, S = 2, 4, 2, 300
     q, k, v = rnd(B, Hq, S, D, seed=70, scale=2.0), rnd(B, Hkv, S, D, seed=71), rnd(B, Hkv, S, D, seed=72)
     out, lse = raw._dense(q.cuda(), k.cuda(), v.cuda(), None, 1, None, want_lse=True)
     torch.cuda.synchronize()
     _, _, _, lse_ref = orc.prefill_backward_reference(q, k, v, torch.zeros(B, Hq, S, D), causal=True)
-    torch.testing.assert_close(lse.cpu(), lse_ref, atol=2e-3, rtol=1e-3)
+    torch.testing.assert_close(lse.cpu(), lse_ref, atol=3e-3, rtol=1e-3)
     # the output is unchanged by asking for lse
-    assert torch.equal(out, ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=True))
+    assert torch.equal(out, ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=True, kv_splits=1))
+    # runaway keys, no mask, more keys than queries
+    Sq, Sk = 200, 1100
+    q, k, v = rnd(1, Hq, Sq, D, seed=73), rnd(1, Hkv, Sk, D, seed=74).float(), rnd(1, Hkv, Sk, D, seed=75)
+    k[:, :, 500:520] *= 25.0
+    k[:, :, 900] *= -40.0
+    k = k.to(torch.bfloat16)
+    out, lse = raw._dense(q.cuda(), k.cuda(), v.cuda(), None, 0, None, want_lse=True)
+    _, _, _, lse_ref = orc.prefill_backward_reference(q, k, v, torch.zeros(1, Hq, Sq, D), causal=False)
+    torch.testing.assert_close(lse.cpu(), lse_ref, atol=3e-3, rtol=1e-3)
 
 
 def test_backward_is_deterministic_and_linear_in_dout(ops):
