@@ -98,7 +98,9 @@ constexpr int kWORow = kWD * 2 + 16; // bytes per row of the query/output stagin
 
 // Direct-to-LDS load of 16 bytes per lane (see dma_to_lds_16 in common.hpp).  This variant writes m0 inside the
 // statement: the assembly loop of this kernel writes m0 too, behind the compiler's back, so nothing here may rely on
-// the compiler's idea of what m0 holds.
+// the compiler's idea of what m0 holds.  (m0 cannot be named in a clobber list -- the compiler treats it as reserved
+// and warns that clobbering it is undefined -- and it needs no naming: the compiler keeps nothing in m0 across
+// statements, it writes m0 directly in front of each of its own instructions that read it.)
 __device__ __forceinline__ void dma_to_lds_16_m0(const void* gbase, uint32_t voff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
