@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             const int r = i * kRowsPerPass + r0;
             q_rows[i] = u32x4{0u, 0u, 0u, 0u};
             if (qw0 + i * kRowsPerPass < jb.sq) {          // (wave-uniform: see row_passes)
-                if (qw0 + r < jb.sq) q_rows[i] = *reinterpret_cast<const u32x4*>(my_rows + (int64_t)(i * kRowsPerPass) * p.qs[2]);
+                if (qw0 + r < jb.sq) q_rows[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(my_rows + (int64_t)(i * kRowsPerPass) * p.qs[2]));
             }
         }
         if (nt > 1) issue_k(jb, 1, 1);
@@ -368,6 +368,9 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         r_ref[0] = r_ref[1] = preset ? 0.f : -INFINITY;
         nb[0] = nb[1] = preset ? -kBias : 0.f;
         bool redo = false;                    // a row sum left the range in which no term can have been lost
+        // The first boundary of a query tile need not wait for the row stores of the query tile before it: they
+        // are younger than every request in flight (first attempt only, and only when their number is the usual 16).
+        bool first_boundary = preset && prev_stores == 16;
 
         // Wait for K[0] and meet the others.  Younger than its request are: on the first attempt this job's query row
         // loads and the previous job's output row stores (each issued once per four rows that exist), and on both
@@ -444,7 +447,8 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         };
         // boundary(tile): see the protocol in the file header
         auto boundary = [&](int tile) {
-            wait_vmcnt<0>();
+            if (first_boundary) wait_vmcnt<16>(); else wait_vmcnt<0>();
+            first_boundary = false;
             __syncthreads();
             if (tile + 1 < n_tiles) issue_v(cur, tile + 1, (tile + 1) & 1);
             if (tile + 2 < n_tiles) issue_k(cur, tile + 2, tile & 1);
@@ -518,12 +522,13 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                   [thr0] "+v"(v_thr0), [thr1] "+v"(v_thr1)
                 : [n_tiles] "s"(__builtin_amdgcn_readfirstlane(n_tiles)), [n_end] "s"(__builtin_amdgcn_readfirstlane(n_loop)),
                   [n_pipe] "s"(__builtin_amdgcn_readfirstlane(min(n_plain, n_loop))), [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)),
-                  [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)),
+                  [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)), [first] "s"(__builtin_amdgcn_readfirstlane((int)first_boundary)),
                   [kstep] "s"(__builtin_amdgcn_readfirstlane(k_step)), [vstep] "s"(__builtin_amdgcn_readfirstlane(v_step)),
                   [ldsdst] "s"(lds_dst), [scale] "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, p.scale_log2))),
                   [klo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)kptr)), [khi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kptr >> 32))),
                   [vlo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)vptr)), [vhi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(vptr >> 32)))
-                : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
+                : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", "s43", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
+            if (tile_s > tile) first_boundary = false;      // (every tile the block ran had its boundary)
             tile = tile_s;
             // status 0: tiles up to n_loop done.  1: tiles up to `tile` done, and the last of them took a row sum to 2.
             if (status != 0) {
@@ -586,7 +591,8 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         store_block(std::integral_constant<int, 1>{});
         break;
         }   // attempts
-        // ---- output rows leave whole, through the slab ----
+        // ---- output rows leave whole, through the slab (written once, never read here: non-temporal, like the
+        // query rows, so that the K/V tiles keep the L2 to themselves) ----
         int64_t out_off = (int64_t)(qw0 + r0) * p.os[2] + c16 * 8;
         asm volatile("" : "+v"(out_off));                  // (as for the query rows: addresses computed here, not earlier)
         __bf16* my_out = cur.ob + out_off;
@@ -595,7 +601,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             const int r = i * kRowsPerPass + r0;
             const u32x4 w = *reinterpret_cast<const u32x4*>(slab + r * kWORow + c16 * 16);
             if (qw0 + i * kRowsPerPass < sq) {             // (wave-uniform: see row_passes)
-                if (qw0 + r < sq) *reinterpret_cast<u32x4*>(my_out + (int64_t)(i * kRowsPerPass) * p.os[2]) = w;
+                if (qw0 + r < sq) __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(my_out + (int64_t)(i * kRowsPerPass) * p.os[2]));
             }
         }
         prev_stores = row_passes(cur);
