@@ -424,6 +424,43 @@ def test_prefill_head_dim_128_two_kernels_agree_on_random_shapes(ops, seed):
         check(slow, ref, what=f"8-wavefront kernel seed {seed} #{case}")
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_prefill_head_dim_128_packed_sequences_of_drawn_lengths(ops, seed):
+    """Packed sequences of drawn lengths (empty ones included) through the persistent 64-query kernel: a workgroup
+    walks from job to job across sequences of different lengths, prefetching the next job's rows and tiles; with
+    a promised maximum that is too small for one sequence; forward-only and with the log-sum-exp output."""
+    g = torch.Generator().manual_seed(2000 + seed)
+    Hq, Hkv, D = 4, 2, 128
+    n_seq = int(torch.randint(2, 9, (1,), generator=g))
+    lens = [int(x) for x in torch.randint(0, 700, (n_seq,), generator=g)]
+    lens[int(torch.randint(0, n_seq, (1,), generator=g))] = 1
+    if sum(lens) == 0:
+        lens[0] = 5
+    print(f"case: packed drawn lengths seed={seed} lens={lens}", flush=True)
+    T = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q, k, v = rnd(T, Hq, D, seed=3000 + seed), rnd(T, Hkv, D, seed=3100 + seed), rnd(T, Hkv, D, seed=3200 + seed)
+    ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True)
+    got = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens),
+                                        causal=True, kv_splits=1)
+    check(got, ref, what="packed drawn lengths")
+    short = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(1, max(lens) // 3),
+                                          max(1, max(lens) // 3), causal=True, kv_splits=1)
+    check(short, ref, what="packed drawn lengths, promised maximum too small")
+    from mi355_attn import ops as raw
+    out2, lse = raw._varlen(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens), True, None, want_lse=True)
+    assert torch.equal(out2, got)
+    scores = []
+    for b, n in enumerate(lens):
+        if n == 0:
+            continue
+        a, e = int(cu[b]), int(cu[b + 1])
+        s_ = torch.einsum("qhd,khd->hqk", q[a:e].float(), k[a:e].float().repeat_interleave(Hq // Hkv, 1)) / math.sqrt(D)
+        s_ = s_.masked_fill(~torch.tril(torch.ones(n, n, dtype=torch.bool)), float("-inf"))
+        scores.append(torch.logsumexp(s_, -1))
+    torch.testing.assert_close(lse.cpu(), torch.cat(scores, 1), atol=3e-3, rtol=1e-3)
+
+
 def _reference_module_tensors(x_proj, freq, num_heads, amp):
     """Q, K, V exactly as CausalMultiHeadSelfAttention.forward hands them to the attention call
     (llm-core/llm_core/model.py:362-378) from the three projection outputs (B, S, H*d): `rearrange` views, then
