@@ -57,7 +57,8 @@ Register map (physical, fixed; the block loads them itself from its operands, se
   a[0:63] O^T of block A (d-tile dt = a[16dt:16dt+15]), a[64:127] block B, a[128:131] / a[132:135] row sums:
   these live in the AGPRs for a whole query tile and are touched only by the assembly snippets below (the kernel
   is compiled with its builtin MFMAs in VGPR form, so the compiler has no use for AGPRs of its own)
-  a[136:167] Q^T fragments of block A (step s = a[136+4s:139+4s]), a[168:199] block B: loaded by entry()
+  a[136:167] Q^T fragments of block A (step s = a[136+4s:139+4s]), a[168:199] block B: loaded from LDS by the
+  W64_QFRAGS statement before the block first runs for a query tile; they stay across re-entries
   a[200:215] K fragments (4 in flight), a[216:247] V^T fragments (8: 2 slices x 4 d-tiles): LDS reads land in
   AGPRs directly and the MFMAs take them as A operands, which leaves the vector registers to the compiler
   s[36:37] / s[38:39] global address of the wavefront's first DMA row of K[t+2] / V[t+1] (advanced per tile),
@@ -82,14 +83,13 @@ N_FIXED_VGPRS = 130
 # Scratch registers are the block's vector operands themselves: each is read once by entry() and is free from then on
 # (the operands are declared in/out), so the block needs no register beyond v[0:129] and its operands.
 ETMP = ["%[nb0]", "%[nb1]", "%[suma]", "%[k0]", "%[vlo0]", "%[vhi0]", "%[rowk]", "%[rowv]"]   # exponentials on their way to packing
-TMP = "%[qaddr]"                    # scratch
+TMP = "v0"                          # scratch of entry() (the score registers hold nothing yet)
 OREG = {"A": 0, "B": 64}
 LREG = {"A": 128, "B": 132}
 QREG = {"A": 136, "B": 168}
 N_ACC = 136                         # a[0:135]: what ordinary code reaches through the snippets
 N_AGPRS = 248
 KPTR, VPTR, FLAG, KSTEP16, VSTEP16, FIRST = 36, 38, 42, 40, 41, 43
-Q_SLAB_ROW = 272                    # bytes per row of the query staging slab (256 + 16 of padding)
 K_TILE = 16384                      # bytes of one K (or V) tile in LDS: 64 rows x 256 bytes
 ROW = 256
 NONE = {"A": False, "B": False}
@@ -603,12 +603,8 @@ def pipeline(e, b, start, h0_start, dry=False):
 
 
 def entry(e):
-    """Loads the fixed registers from the block's operands: the Q^T fragments from the staging slab, nb, the row-sum
-    operand, LDS read addresses (the address of step s / d-tile dt is the one of step 0 / d-tile 0 with s << 5 /
+    """Loads the fixed registers from the block's operands: nb, the row-sum operand, LDS read addresses (the address of step s / d-tile dt is the one of step 0 / d-tile 0 with s << 5 /
     dt << 6 XORed in: the swizzle XORs exactly those bits), DMA lane offsets and pointers, mask thresholds."""
-    for c in "AB":
-        for s_ in range(8):
-            e.lines.append(f"ds_read_b128 a{rng(QREG[c] + 4 * s_, 4)}, %[qaddr] offset:{(c == 'B') * 32 * Q_SLAB_ROW + 32 * s_}")
     e.raw(f"v_mov_b32 v{NB['A']}, %[nb0]")
     e.raw(f"v_mov_b32 v{NB['B']}, %[nb1]")
     e.raw(f"v_mov_b32 v{NEGINF}, 0xff800000")
@@ -621,7 +617,6 @@ def entry(e):
     for dt in range(4):
         e.raw(f"v_xor_b32 v{VOFF + dt}, {hex(dt << 6)}, %[vlo0]")
         e.raw(f"v_xor_b32 v{VOFF + 4 + dt}, {hex(dt << 6)}, %[vhi0]")
-    e.raw("s_waitcnt lgkmcnt(0)")                      # the Q^T fragments are in; %[qaddr] is scratch from here on
     for j in range(4):                                 # load j of a tile: swizzled chunk, row part, and j * four rows
         e.raw(f"v_xor_b32 {TMP}, {hex(j << 4)}, %[c0s]")
         e.raw(f"v_add_u32 v{DMAOFF + j}, {TMP}, %[rowk]")
@@ -723,7 +718,23 @@ def snippets():
     # cannot see that an MFMA reads it here.)
     out["W64_ZERO"] = (["s_nop 3"] + [f"v_mfma_f32_32x32x16_bf16 a{rng(16 * i, 16)}, %0, %0, 0" for i in range(8)] +
                        [f"v_mfma_f32_16x16x32_bf16 a{rng(LREG[c], 4)}, %0, %0, 0" for c in "AB"])
+    # Q^T fragments from the wavefront's query rows in LDS (64 rows of 256 bytes, swizzled like a K tile) into their
+    # AGPRs.  Operands: %0 scratch (early-clobber output), %1 LDS address of the lane's piece of step 0 in block A
+    # (the one of step s is that with s << 5 XORed in; block B sits 32 rows further).
+    lines = []
+    for s_ in range(8):
+        lines.append(f"v_xor_b32 %0, {hex(s_ << 5)}, %1")
+        lines += [f"ds_read_b128 a{rng(QREG[c] + 4 * s_, 4)}, %0 offset:{(c == 'B') * 32 * ROW}" for c in "AB"]
+        if s_ == 5:
+            lines.append("s_waitcnt lgkmcnt(4)")           # (the counter of LDS operations in flight holds 15)
+    lines.append("s_waitcnt lgkmcnt(0)")
+    out["W64_QFRAGS"] = lines
     for c in range(2):
+        # scores of one 32-key half in ordinary code: %0 = sum over steps of K fragment %(1+s) . Q^T fragment s
+        q = (QREG["A"], QREG["B"])[c]
+        out[f"W64_QK_{c}"] = (["s_nop 3"] +
+                              [f"v_mfma_f32_32x32x16_bf16 %0, %{1 + s_}, a{rng(q + 4 * s_, 4)}, {'%0' if s_ else '0'}"
+                               for s_ in range(8)] + ["s_nop 15"])
         for dt in range(4):
             a = acc_of(c, dt)
             # operands: %0 V^T fragment (4 registers), %1 P^T fragment (4 registers), both ready when the statement

@@ -627,7 +627,7 @@ static int prefill_common(const void* q, const void* k, const void* v, void* out
         return MI355_OK;
     }
     // head_dim 128 without an explicit mask: the kernel with 64 queries per wavefront and a hand-scheduled tile loop
-    if (D == 128 && mask_mode != MI355_MASK_BOOL) rc = launch_prefill_w64(p, s);
+    if (D == 128 && mask_mode != MI355_MASK_BOOL && prefill_w64_takes(p)) rc = launch_prefill_w64(p, s);
     else rc = D == 128 ? launch_prefill<128>(p, s) : (D == 64 ? launch_prefill<64>(p, s) : launch_prefill<32>(p, s));
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;

@@ -63,6 +63,16 @@ __device__ __forceinline__ void acc_sum(bf16x8 sum_a, bf16x8 pt) {  // row sums 
     if constexpr (C == 0) asm volatile(W64_SUM_0 : : "v"(sum_a), "v"(pt) : W64_CLOBBER_ACC);
     else asm volatile(W64_SUM_1 : : "v"(sum_a), "v"(pt) : W64_CLOBBER_ACC);
 }
+// scores of one 32-key half against column block C: sum over the eight steps of K fragment . Q^T fragment
+template <int C>
+__device__ __forceinline__ f32x16 qk_scores(const u32x4 (&kf)[8]) {
+    f32x16 s;
+    if constexpr (C == 0)
+        asm volatile(W64_QK_0 : "=&v"(s) : "v"(kf[0]), "v"(kf[1]), "v"(kf[2]), "v"(kf[3]), "v"(kf[4]), "v"(kf[5]), "v"(kf[6]), "v"(kf[7]) : W64_CLOBBER_ACC);
+    else
+        asm volatile(W64_QK_1 : "=&v"(s) : "v"(kf[0]), "v"(kf[1]), "v"(kf[2]), "v"(kf[3]), "v"(kf[4]), "v"(kf[5]), "v"(kf[6]), "v"(kf[7]) : W64_CLOBBER_ACC);
+    return s;
+}
 template <int C>
 __device__ __forceinline__ void acc_scale(float alpha, float a_lo, float a_hi) {   // O^T(C, .) *= alpha, row sums likewise
     float scratch;
@@ -94,7 +104,6 @@ constexpr int kWBN = 64;             // keys per LDS tile
 constexpr int kWD = 128;
 constexpr int kWRow = kWD * 2;       // bytes per LDS row
 constexpr int kWTile = kWBN * kWRow; // bytes per K (or V) tile
-constexpr int kWORow = kWD * 2 + 16; // bytes per row of the query/output staging slab
 
 // Direct-to-LDS load of 16 bytes per lane (see dma_to_lds_16 in common.hpp).  This variant writes m0 inside the
 // statement: the assembly loop of this kernel writes m0 too, behind the compiler's back, so nothing here may rely on
@@ -108,6 +117,21 @@ __device__ __forceinline__ void dma_to_lds_16_m0(const void* gbase, uint32_t vof
                  : "memory");
 }
 
+// cu_q[b], cu_q[b+1], cu_k[b], cu_k[b+1] through the scalar cache (the arrays do not change while the kernel runs;
+// the compiler, seeing stores all around, would fetch them one after the other with vector loads)
+__device__ __forceinline__ void load_bounds(const int32_t* cu_q, const int32_t* cu_k, int b, int& q_lo, int& q_hi, int& k_lo, int& k_hi) {
+    typedef int i32x2 __attribute__((ext_vector_type(2)));
+    i32x2 qb, kb;
+    asm volatile("s_load_dwordx2 %0, %2, 0x0\n\ts_load_dwordx2 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(qb), "=&s"(kb)
+                 : "s"(cu_q + b), "s"(cu_k + b)
+                 : "memory");
+    q_lo = qb[0];
+    q_hi = qb[1];
+    k_lo = kb[0];
+    k_hi = kb[1];
+}
+
 template <bool CAUSAL>
 __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int n_logical) {
     constexpr int D = kWD, NS = D / 16, NDT = D / 32, CPR = D / 8;
@@ -117,7 +141,8 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
 
     // K buffers 0,1 then V buffers 0,1 (the assembly loop addresses all four relative to one base)
     __shared__ __attribute__((aligned(1024))) unsigned char kv_lds[4 * kWTile];
-    __shared__ __attribute__((aligned(16))) unsigned char o_lds[kWWaves * 64 * kWORow];
+    // the four wavefronts' 64 query rows each, laid out like a K tile
+    __shared__ __attribute__((aligned(1024))) unsigned char q_lds[kWWaves * 64 * kWRow];
     unsigned char* const k_lds = kv_lds;
     unsigned char* const v_lds = kv_lds + 2 * kWTile;
 
@@ -137,53 +162,77 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         float* lb;                       // row 0 of this (sequence, head) in the log-sum-exp output, or null
         int sq, sk, q0;
     };
+    // head and row strides fit 32 bits (the host checks), so an address takes two scalar multiplications
+    const int qs2 = (int)p.qs[2], ks2 = (int)p.ks[2], vs2 = (int)p.vs[2], os2 = (int)p.os[2];
+    const int n_pairs = p.n_pairs, Hq = p.Hq;
+    // the ids of this workgroup: id, id + id_step, ... below id_end
     const int G = gridDim.x, bid = blockIdx.x;
     const bool by_xcd = (n_logical % 8 == 0) && (G % 8 == 0);
+    const int id_step = by_xcd ? G / 8 : G;
+    const int id_end = by_xcd ? (bid % 8 + 1) * (n_logical / 8) : n_logical;
+    int id = by_xcd ? (bid % 8) * (n_logical / 8) + bid / 8 : bid;
+    // (pair, head, batch) of id and of id_step: an id advances digit by digit, with no division per job
+    int id_pair = id % n_pairs, id_h = (id / n_pairs) % Hq, id_b = id / (n_pairs * Hq);
+    const int st_pair = id_step % n_pairs, st_h = (id_step / n_pairs) % Hq, st_b = id_step / (n_pairs * Hq);
+    const int group = Hq / p.Hkv, group_shift = (group & (group - 1)) == 0 ? __builtin_ctz(group) : -1;
     int job_k = -1, job_nq = 0, job_pair = 0, job_half = 1;      // position: "after the last query tile of id number job_k"
-    Job job_seq{};                                               // sequence-level fields of the current id
-    auto next_job = [&](Job& j) -> bool {
+    // next_job(j, prev): the job after `prev` (whatever `prev` holds before the first).
+    // What only a new id needs -- tensor addresses, batch strides, the bounds arrays -- is read from the kernel
+    // arguments (first argument, offset 0 of the segment) where it is needed, through an offset the compiler cannot
+    // trace: two scalar loads per id instead of three dozen scalar registers held, and spilled, for the whole kernel.
+    typedef const __attribute__((address_space(4))) PrefillParams* ParamsPtr;
+    auto args = [&]() -> ParamsPtr {
+        size_t off = 0;
+        asm volatile("" : "+s"(off));
+        return (ParamsPtr)((const __attribute__((address_space(4))) char*)__builtin_amdgcn_kernarg_segment_ptr() + off);
+    };
+    auto next_job = [&](Job& j, const Job& prev) -> bool {
+        j = prev;                             // the sequence-level fields stay while the id stays
         if (job_half == 0 && job_pair != job_nq - 1 - job_pair) {           // second query tile of the pair
             job_half = 1;
-            j = job_seq;
             j.q0 = job_pair * kWBM;
             return true;
         }
-        job_pair += p.n_pairs;                // a further pair of the same sequence: only if it is longer than Sq_max promised
+        job_pair += n_pairs;                  // a further pair of the same sequence: only if it is longer than Sq_max promised
         while (!(job_k >= 0 && 2 * job_pair < job_nq)) {
+            if (job_k >= 0) {
+                id += id_step;
+                id_pair += st_pair;
+                int carry = id_pair >= n_pairs;
+                id_pair -= carry ? n_pairs : 0;
+                id_h += st_h + carry;
+                carry = id_h >= Hq;
+                id_h -= carry ? Hq : 0;
+                id_b += st_b + carry;
+            }
             ++job_k;
-            int lid;
-            if (by_xcd) {
-                const int per = n_logical / 8, slot = bid / 8 + job_k * (G / 8);
-                if (slot >= per) return false;
-                lid = (bid % 8) * per + slot;
+            if (id >= id_end) return false;
+            const int h = id_h, b = id_b, hk = group_shift >= 0 ? h >> group_shift : h / group;
+            const ParamsPtr a = args();
+            const int qs1 = (int)a->qs[1], ks1 = (int)a->ks[1], vs1 = (int)a->vs[1], os1 = (int)a->os[1], ls1 = (int)a->ls[1];
+            if (a->cu_q) {
+                int q_start, q_end, k_start, k_end;
+                load_bounds(a->cu_q, a->cu_k, b, q_start, q_end, k_start, k_end);
+                j.sq = q_end - q_start;
+                j.sk = k_end - k_start;
+                j.qb = a->q + ((int64_t)q_start * qs2 + (int64_t)h * qs1);
+                j.kb = a->k + ((int64_t)k_start * ks2 + (int64_t)hk * ks1);
+                j.vb = a->v + ((int64_t)k_start * vs2 + (int64_t)hk * vs1);
+                j.ob = a->out + ((int64_t)q_start * os2 + (int64_t)h * os1);
+                j.lb = a->lse ? a->lse + (q_start + (int64_t)h * ls1) : nullptr;
             } else {
-                lid = bid + job_k * G;
-                if (lid >= n_logical) return false;
+                j.sq = a->Sq;
+                j.sk = a->Sk;
+                j.qb = a->q + ((int64_t)b * a->qs[0] + (int64_t)h * qs1);
+                j.kb = a->k + ((int64_t)b * a->ks[0] + (int64_t)hk * ks1);
+                j.vb = a->v + ((int64_t)b * a->vs[0] + (int64_t)hk * vs1);
+                j.ob = a->out + ((int64_t)b * a->os[0] + (int64_t)h * os1);
+                j.lb = a->lse ? a->lse + ((int64_t)b * a->ls[0] + (int64_t)h * ls1) : nullptr;
             }
-            const int h = (lid / p.n_pairs) % p.Hq, b = lid / (p.n_pairs * p.Hq), hk = h / (p.Hq / p.Hkv);
-            if (p.cu_q) {
-                const int q_start = p.cu_q[b], k_start = p.cu_k[b];
-                job_seq.sq = p.cu_q[b + 1] - q_start;
-                job_seq.sk = p.cu_k[b + 1] - k_start;
-                job_seq.qb = p.q + (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
-                job_seq.kb = p.k + (int64_t)k_start * p.ks[2] + (int64_t)hk * p.ks[1];
-                job_seq.vb = p.v + (int64_t)k_start * p.vs[2] + (int64_t)hk * p.vs[1];
-                job_seq.ob = p.out + (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
-                job_seq.lb = p.lse ? p.lse + q_start + (int64_t)h * p.ls[1] : nullptr;
-            } else {
-                job_seq.sq = p.Sq;
-                job_seq.sk = p.Sk;
-                job_seq.qb = p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[1];
-                job_seq.kb = p.k + (int64_t)b * p.ks[0] + (int64_t)hk * p.ks[1];
-                job_seq.vb = p.v + (int64_t)b * p.vs[0] + (int64_t)hk * p.vs[1];
-                job_seq.ob = p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[1];
-                job_seq.lb = p.lse ? p.lse + (int64_t)b * p.ls[0] + (int64_t)h * p.ls[1] : nullptr;
-            }
-            job_nq = (job_seq.sq + kWBM - 1) / kWBM;
-            job_pair = lid % p.n_pairs;
+            job_nq = (j.sq + kWBM - 1) / kWBM;
+            job_pair = id_pair;
         }
         job_half = 0;
-        j = job_seq;
         j.q0 = (job_nq - 1 - job_pair) * kWBM;
         return true;
     };
@@ -193,17 +242,17 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const int ld_q = lane >> 4;
     const int ld_c0 = (lane & 15) ^ (ld_q << 2);
     // byte offset of the lane's 16 bytes from the wavefront's first row of step j: row part + ((ld_c0 ^ j) << 4)
-    const uint32_t dma_row_k = (uint32_t)(ld_q * (int)p.ks[2] * 2), dma_row_v = (uint32_t)(ld_q * (int)p.vs[2] * 2);
+    const uint32_t dma_row_k = (uint32_t)(ld_q * ks2 * 2), dma_row_v = (uint32_t)(ld_q * vs2 * 2);
     const uint32_t lds_dst = __builtin_amdgcn_readfirstlane(lds_address(kv_lds + wave * 4096));
-    const uint32_t k_step = (uint32_t)(4 * p.ks[2] * 2), v_step = (uint32_t)(4 * p.vs[2] * 2);   // 4 rows, in bytes
+    const uint32_t k_step = (uint32_t)(4 * ks2 * 2), v_step = (uint32_t)(4 * vs2 * 2);   // 4 rows, in bytes
     // K (which == 0) or V (which == 1) rows of tile `tile` into that tensor's LDS buffer `buf`
     auto issue_rows = [&](const Job& jb, int which, int tile, int buf) {
         const __bf16* src = which ? jb.vb : jb.kb;
-        const int64_t stride = which ? p.vs[2] : p.ks[2];
+        const int stride = which ? vs2 : ks2;
         const uint32_t step = which ? v_step : k_step, dma_row = which ? dma_row_v : dma_row_k;
         const uint32_t dst = lds_dst + (2 * which + buf) * kWTile;
         if (tile * kWBN + kWBN <= jb.sk) {
-            const unsigned char* base = reinterpret_cast<const unsigned char*>(src + ((int64_t)tile * kWBN + 16 * wave) * stride);
+            const unsigned char* base = reinterpret_cast<const unsigned char*>(src + (int64_t)(tile * kWBN + 16 * wave) * stride);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 dma_to_lds_16_m0(base + (size_t)j * step, dma_row + ((ld_c0 ^ j) << 4), dst + j * 1024);
@@ -213,7 +262,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             // the top of the job it occupied two dozen registers that then lived in scratch memory.)
             int last = jb.sk - 1 - tile * kWBN;
             asm volatile("" : "+s"(last));
-            const unsigned char* t0 = reinterpret_cast<const unsigned char*>(src + (int64_t)tile * kWBN * stride);
+            const unsigned char* t0 = reinterpret_cast<const unsigned char*>(src + (int64_t)(tile * kWBN) * stride);
             const uint32_t row_bytes = (uint32_t)stride * 2u;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -264,42 +313,63 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     }
     const bf16x8 sum_a = as_bf16x8(u32x4{sum_word, sum_word, sum_word, sum_word});
 
-    // The staging slab of the wavefront: its 64 query rows during a job (the assembly loop loads its fragments from
-    // here whenever it starts, ordinary code reads them as it needs them), the output rows at the end of the job.
-    unsigned char* const slab = o_lds + wave * (64 * kWORow);
-    const uint32_t q_addr = lds_address(slab + n * kWORow + 8 * kg * 2);
-    auto qfrag = [&](int c, int s) { return as_bf16x8(lds_load_at<u32x4>(q_addr + c * 32 * kWORow + 32 * s)); };
-    constexpr int kRowsPerPass = 64 / CPR;           // the slab is filled and emptied 4 whole rows at a time, 16 passes
-    const int c16 = lane % CPR, r0 = lane / CPR;
-
-    // What a job needs before it can start is requested as early as possible -- for the first job right here, for
-    // every other one while the job before it normalises and stores its output: K[0] (direct-to-LDS), the wavefront's
-    // query rows (into registers; rows past the end of the sequence are zero), then K[1] and V[0].
-    u32x4 q_rows[64 / kRowsPerPass];
-    auto prefetch = [&](const Job& jb) {
-        const int nt = tiles_of(jb);
-        if (nt > 0) issue_k(jb, 0, 0);
+    // ---- query rows: the wavefront's 64 rows go to its own part of q_lds with sixteen direct-to-LDS loads of four
+    // rows each, swizzled like a K tile (load i covers rows 4i + lane/16, and swz of that row is ((lane/16) << 2) |
+    // (i & 3)); a row past the end of the sequence re-reads the last row (finite; nothing of it is ever stored) ----
+    const uint32_t q_dst = __builtin_amdgcn_readfirstlane(lds_address(q_lds + wave * (64 * kWRow)));
+    // (loads 4 * part .. 4 * part + 3: rows 16 * part .. 16 * part + 15)
+    auto issue_q = [&](const Job& jb, int part) {
         const int qw0 = jb.q0 + 64 * wave;
-        // (the row addresses are derived from a value the compiler cannot trace, so that it computes them here and
-        // not at the top of the job, where sixteen 64-bit addresses would have to wait in registers)
-        // (an offset, not the pointer, goes through the empty statement: a pointer would come back without its
-        // address space and the loads would become flat ones, which also count as LDS operations)
-        int64_t my_off = (int64_t)(qw0 + r0) * p.qs[2] + c16 * 8;
-        asm volatile("" : "+v"(my_off));
-        const __bf16* my_rows = jb.qb + my_off;
+        const uint32_t row_bytes = (uint32_t)qs2 * 2u;
+        if (qw0 + 64 <= jb.sq) {
+            const unsigned char* base = reinterpret_cast<const unsigned char*>(jb.qb + (int64_t)(qw0 + 16 * part) * qs2);
 #pragma unroll
-        for (int i = 0; i < 64 / kRowsPerPass; ++i) {
-            const int r = i * kRowsPerPass + r0;
-            q_rows[i] = u32x4{0u, 0u, 0u, 0u};
-            if (qw0 + i * kRowsPerPass < jb.sq) {          // (wave-uniform: see row_passes)
-                if (qw0 + r < jb.sq) q_rows[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(my_rows + (int64_t)(i * kRowsPerPass) * p.qs[2]));
+            for (int j = 0; j < 4; ++j)
+                dma_to_lds_16_m0(base + (size_t)(4 * j) * row_bytes, (uint32_t)ld_q * row_bytes + ((ld_c0 ^ j) << 4), q_dst + (4 * part + j) * 1024);
+        } else {
+            // (the empty statement keeps the arithmetic of this rare path inside the branch)
+            int last = jb.sq - 1;
+            asm volatile("" : "+s"(last));
+            const int first = min(qw0, last);              // (a wavefront wholly past the end reads the last row 64 times)
+            const unsigned char* base = reinterpret_cast<const unsigned char*>(jb.qb + (int64_t)first * qs2);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t row = (uint32_t)(min(qw0 + 16 * part + 4 * j + ld_q, last) - first);
+                dma_to_lds_16_m0(base, row * row_bytes + (uint32_t)((ld_c0 ^ j) << 4), q_dst + (4 * part + j) * 1024);
             }
         }
-        if (nt > 1) issue_k(jb, 1, 1);
-        if (nt > 0) issue_v(jb, 0, 0);
     };
-    // number of row instructions (loads of query rows, stores of output rows: four rows each) a job issues: a pass
-    // whose four rows all lie past the end of the sequence is jumped over, so the count is known here
+    // Q^T fragment of step s in block c: row 32c + n, chunk (2s + kg) ^ swz(n), as for K
+    const uint32_t q_rd0 = q_dst + n * kWRow + ((kg ^ swz<D>(n)) << 4);
+
+    // ---- output rows leave whole, 32 at a time, through LDS: through the wavefront's own shares of the second K and
+    // V buffers (the 16 rows each that its own direct-to-LDS loads fill), which are idle between the last tile of a
+    // job and the requests of K[1] / V[1] of the next.  Rows of 256 bytes, chunk c of row r at c ^ swz(r). ----
+    constexpr int kRowsPerPass = 64 / CPR;           // a store instruction takes 4 whole rows
+    const int c16 = lane % CPR, r0 = lane / CPR;
+    unsigned char* const stage_w = kv_lds + ((n < 16) ? 1 : 3) * kWTile + wave * 4096 + (n & 15) * kWRow + 8 * kg;   // the lane's row n
+    const int stage_wx = swz<D>(n);
+    unsigned char* const stage_r = kv_lds + kWTile + wave * 4096 + r0 * kWRow;        // row r0 of pass 0
+
+    // What a job needs before it can start is requested as early as possible -- for the first job right away, for
+    // every other one while the job before it normalises and stores its output: K[0], the query rows, V[0], and K[1]
+    // once the output rows have left its buffer.  Six groups of four requests and a seventh: in the epilogue of a job
+    // they go out one group at a time between pieces of vector work, so that the wavefront does not sit behind a
+    // full request queue (the four wavefronts all do this at the same time).
+    auto prefetch_group = [&](const Job& jb, int group) {
+        if (group == 0) {
+            if (tiles_of(jb) > 0) issue_k(jb, 0, 0);
+        } else if (group <= 4) {
+            issue_q(jb, group - 1);
+        } else if (group == 5) {
+            if (tiles_of(jb) > 0) issue_v(jb, 0, 0);
+        } else {
+            if (tiles_of(jb) > 1) issue_k(jb, 1, 1);
+        }
+    };
+    // number of output row stores a job issues at its end (four whole rows each): a pass whose four rows all lie
+    // past the end of the sequence is jumped over, so the count is known here.  (The one or two stores of a
+    // log-sum-exp output are not counted: a count that is too low only makes a wait take a little more than it must.)
     auto row_passes = [&](const Job& jb) {
         return min(max((jb.sq - (jb.q0 + 64 * wave) + kRowsPerPass - 1) / kRowsPerPass, 0), 64 / kRowsPerPass);
     };
@@ -322,9 +392,12 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     };
 
     Job cur{}, nxt{};
-    bool have = next_job(cur);
-    if (have) prefetch(cur);
-    int prev_stores = 0;                                   // output row stores of the job before `cur`
+    bool have = next_job(cur, cur);
+    if (have) {
+#pragma unroll
+        for (int group = 0; group < 7; ++group) prefetch_group(cur, group);
+    }
+    int prev_stores = 0;       // output row stores of the job before `cur` that are younger than the requests for `cur`
     while (have) {
         const int sq = cur.sq, sk = cur.sk, q0 = cur.q0;
         const int coff = sk - sq;                          // bottom-right aligned causal diagonal
@@ -343,74 +416,44 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         // the assembly loop requests tile+2 with whole-tile loads: it may run tile t only if tile t+2 is a whole tile
         // (or does not exist), so it stops three tiles before a partial last tile
         const int n_asm = n_tiles > sk / kWBN ? max(0, n_tiles - 3) : n_tiles;
-        const int young_rows = row_passes(cur) + prev_stores;
+        // the job after this one (scalar work, done while the first tile is still landing)
+        const bool have_next = next_job(nxt, cur);
 
-        // query rows: registers -> slab (the previous job has read its output rows back from the slab by now: LDS
-        // operations of a wavefront execute in order)
-#pragma unroll
-        for (int i = 0; i < 64 / kRowsPerPass; ++i)
-            *reinterpret_cast<u32x4*>(slab + (i * kRowsPerPass + r0) * kWORow + c16 * 16) = q_rows[i];
-
-        // Two attempts at most: the first with the references preset to 0, the second -- only if some row's sum came
-        // out suspiciously small or large -- entirely in ordinary code with references taken from the data.
-        bool have_next = false;
-        for (int attempt = 0; attempt < 2; ++attempt) {
-        const bool preset = attempt == 0;
-        const int young_dma = (n_tiles > 1 ? 4 : 0) + (n_tiles > 0 ? 4 : 0);      // requests of K[1] and V[0]
-        if (!preset) {                        // start over: the buffers are free (everybody passed the vote below)
-            if (n_tiles > 0) issue_k(cur, 0, 0);
-            if (n_tiles > 1) issue_k(cur, 1, 1);
-            if (n_tiles > 0) issue_v(cur, 0, 0);
-        }
-        asm volatile(W64_ZERO : : "v"(as_bf16x8(u32x4{0u, 0u, 0u, 0u})) : W64_CLOBBER_ACC);      // O^T and the row sums
         // per column block: r_ref exponent reference in the log2 domain (-inf: none yet), nb = -r_ref - kBias
-        float r_ref[2], nb[2];
-        r_ref[0] = r_ref[1] = preset ? 0.f : -INFINITY;
-        nb[0] = nb[1] = preset ? -kBias : 0.f;
+        float r_ref[2], nb[2], l_row[2];
         bool redo = false;                    // a row sum left the range in which no term can have been lost
-        // The first boundary of a query tile need not wait for the row stores of the query tile before it: they
-        // are younger than every request in flight (first attempt only, and only when their number is the usual 16).
-        bool first_boundary = preset && prev_stores == 16;
+        const int young_dma = (n_tiles > 1 ? 4 : 0) + (n_tiles > 0 ? 4 : 0);      // requests of V[0] and K[1]
 
-        // Wait for K[0] and meet the others.  Younger than its request are: on the first attempt this job's query row
-        // loads and the previous job's output row stores (each issued once per four rows that exist), and on both
-        // the requests of K[1] and V[0].
-        wait_all_but(young_dma + (preset ? young_rows : 0));
-        __syncthreads();
-
-        // Scores of one 32-key half of a tile for one column block, in ordinary code (reads K[tile]).
+        // Ordinary code for single tiles.  Everything it derives from the job goes through `fresh`, a copy of the few
+        // values it needs that the compiler cannot trace back: what could be computed once per job would otherwise
+        // be computed at the top of every job and wait in registers (spilled ones, mostly) for a tile that rarely comes.
+        struct Fresh {
+            int sk, qw0, coff, n_tiles;
+        };
+        // Scores of one 32-key half of a tile for one column block (reads K[tile]).
         auto scores = [&](auto c_c, int tile, int t) {
             constexpr int c = decltype(c_c)::value;
             const int buf = tile & 1;
-            f32x16 s_acc;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) s_acc[j] = 0.f;
             // (all fragment reads first, then the MFMAs: one LDS latency instead of eight)
             u32x4 kf[NS];
-            bf16x8 qf[NS];
 #pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                kf[s] = lds_load_at<u32x4>(rd_k(s) + buf * kWTile + t * 32 * kWRow);
-                qf[s] = qfrag(c, s);
-            }
-#pragma unroll
-            for (int s = 0; s < NS; ++s) s_acc = mfma32(as_bf16x8(kf[s]), qf[s], s_acc);
-            return s_acc;
+            for (int s = 0; s < NS; ++s) kf[s] = lds_load_at<u32x4>(rd_k(s) + buf * kWTile + t * 32 * kWRow);
+            return qk_scores<c>(kf);
         };
         // The rest of that half: mask, reference move, weights, accumulation (reads V[tile]).
-        auto finish = [&](auto c_c, int tile, int t, bool masked, f32x16 s_acc) {
+        auto finish = [&](const Fresh& fr, auto c_c, int tile, int t, bool masked, f32x16 s_acc) {
             constexpr int c = decltype(c_c)::value;
             const int buf = tile & 1;
             const int k0 = tile * kWBN + 32 * t;
-            const int qi = qw0 + 32 * c + n;
+            const int qi = fr.qw0 + 32 * c + n;
             float mx = -INFINITY;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 float x = fmaf(s_acc[i], p.scale_log2, nb[c]);
                 if (masked) {
                     const int key = k0 + 8 * (i >> 2) + 4 * kg + (i & 3);
-                    bool keep = key < sk;
-                    if (CAUSAL) keep = keep & (key <= qi + coff);
+                    bool keep = key < fr.sk;
+                    if (CAUSAL) keep = keep & (key <= qi + fr.coff);
                     x = keep ? x : -INFINITY;
                 }
                 s_acc[i] = x;
@@ -446,17 +489,22 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             }
         };
         // boundary(tile): see the protocol in the file header
-        auto boundary = [&](int tile) {
-            if (first_boundary) wait_vmcnt<16>(); else wait_vmcnt<0>();
-            first_boundary = false;
+        auto boundary = [&](const Fresh& fr, int tile) {
+            wait_vmcnt<0>();
             __syncthreads();
-            if (tile + 1 < n_tiles) issue_v(cur, tile + 1, (tile + 1) & 1);
-            if (tile + 2 < n_tiles) issue_k(cur, tile + 2, tile & 1);
+            Job jc = cur;
+            asm volatile("" : "+s"(jc.kb), "+s"(jc.vb));
+            jc.sk = fr.sk;
+            if (tile + 1 < fr.n_tiles) issue_v(jc, tile + 1, (tile + 1) & 1);
+            if (tile + 2 < fr.n_tiles) issue_k(jc, tile + 2, tile & 1);
         };
         // a whole tile in ordinary code: scores from K[tile], boundary, everything else from V[tile]
         // (a tile past n_mask has nothing for this wavefront: it only takes part in the boundary)
         auto step_cxx = [&](int tile) {
-            const bool visible = tile < n_mask, masked = tile >= n_plain;
+            Fresh fr{sk, qw0, coff, n_tiles};
+            int first_masked = n_plain, first_hidden = n_mask;
+            asm volatile("" : "+s"(fr.sk), "+s"(fr.qw0), "+s"(fr.coff), "+s"(fr.n_tiles), "+s"(first_masked), "+s"(first_hidden), "+s"(tile));
+            const bool visible = tile < first_hidden, masked = tile >= first_masked;
             constexpr std::integral_constant<int, 0> A{};
             constexpr std::integral_constant<int, 1> B{};
             f32x16 sa0{}, sb0{}, sa1{}, sb1{};
@@ -466,12 +514,12 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 sa1 = scores(A, tile, 1);
                 sb1 = scores(B, tile, 1);
             }
-            boundary(tile);
+            boundary(fr, tile);
             if (visible) {
-                finish(A, tile, 0, masked, sa0);
-                finish(B, tile, 0, masked, sb0);
-                finish(A, tile, 1, masked, sa1);
-                finish(B, tile, 1, masked, sb1);
+                finish(fr, A, tile, 0, masked, sa0);
+                finish(fr, B, tile, 0, masked, sb0);
+                finish(fr, A, tile, 1, masked, sa1);
+                finish(fr, B, tile, 1, masked, sb1);
             }
         };
         // The assembly loop saw a row sum reach 2: every row's reference moves up by the exponent of its sum (the sum,
@@ -492,6 +540,32 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             nb[c] -= (float)k;
         };
 
+        // Two attempts at most: the first with the references preset to 0 and the hand-scheduled loop wherever it can
+        // run; the second -- only if some row's sum came out suspiciously small or large -- entirely in ordinary code
+        // with references taken from the data.
+        for (int attempt = 0; attempt < 2; ++attempt) {
+        const bool preset = attempt == 0;
+        // (What this loop would let the compiler compute once, before it -- the addresses of the tiles requested
+        // again -- it would compute at the top of every job and park in spilled registers; the copy below, which it
+        // cannot trace, keeps that arithmetic where it is used.)
+        if (!preset) {                        // start over: the buffers are free (everybody passed the vote below)
+            Job jc = cur;
+            asm volatile("" : "+s"(jc.kb), "+s"(jc.vb), "+s"(jc.sk));
+            if (n_tiles > 0) issue_k(jc, 0, 0);
+            if (n_tiles > 1) issue_k(jc, 1, 1);
+            if (n_tiles > 0) issue_v(jc, 0, 0);
+        }
+        asm volatile(W64_ZERO : : "v"(as_bf16x8(u32x4{0u, 0u, 0u, 0u})) : W64_CLOBBER_ACC);      // O^T and the row sums
+        r_ref[0] = r_ref[1] = preset ? 0.f : -INFINITY;
+        nb[0] = nb[1] = preset ? -kBias : 0.f;
+        // Wait for K[0] and the query rows.  Younger than the last request of those are the requests of V[0] and K[1]
+        // and, the first time, the last output row stores of the job before this one.
+        wait_all_but(young_dma + (preset ? prev_stores : 0));
+        if (preset) {                         // the query rows go to their registers
+            uint32_t scratch;
+            asm volatile(W64_QFRAGS : "=&v"(scratch) : "v"(q_rd0) : "memory", W64_CLOBBER_ACC);
+        }
+        __syncthreads();                      // everybody's share of K[0] is in
         int tile = 0;
         const int n_loop = preset ? n_asm : 0;
         while (tile < n_tiles) {
@@ -501,8 +575,8 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 continue;
             }
             // ---- the hand-scheduled loop over tiles [tile, n_loop); leaves after a tile that took a row sum to 2 ----
-            const uint64_t kptr = (uint64_t)(uintptr_t)(cur.kb + ((int64_t)(tile + 2) * kWBN + 16 * wave) * p.ks[2]);
-            const uint64_t vptr = (uint64_t)(uintptr_t)(cur.vb + ((int64_t)(tile + 1) * kWBN + 16 * wave) * p.vs[2]);
+            const uint64_t kptr = (uint64_t)(uintptr_t)(cur.kb + (int64_t)((tile + 2) * kWBN + 16 * wave) * ks2);
+            const uint64_t vptr = (uint64_t)(uintptr_t)(cur.vb + (int64_t)((tile + 1) * kWBN + 16 * wave) * vs2);
             // mask thresholds for the first masked tile the loop will meet: a key at index j of that tile is kept by
             // query i of the wavefront iff j <= i + (qw0 + coff - k0) and j < sk - k0 (the lane part 4*kg of a key's
             // index is folded in)
@@ -512,23 +586,22 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             float v_nb0 = nb[0], v_nb1 = nb[1];
             int v_thr0 = min(n + diag, sk - 1 - k0m) - 4 * kg, v_thr1 = min(n + 32 + diag, sk - 1 - k0m) - 4 * kg;
             uint32_t v_sum = sum_word, v_k0 = rd_k0, v_vlo = rd_vlo0, v_vhi = rd_vhi0;
-            uint32_t v_rowk = dma_row_k, v_rowv = dma_row_v, v_c0s = (uint32_t)(ld_c0 << 4), v_q = q_addr;
+            uint32_t v_rowk = dma_row_k, v_rowv = dma_row_v, v_c0s = (uint32_t)(ld_c0 << 4);
             int status;
             int tile_s = __builtin_amdgcn_readfirstlane(tile);
             asm volatile(W64_LOOP
                 : [tile] "+&s"(tile_s), [t2] "=&s"(status),
                   [nb0] "+v"(v_nb0), [nb1] "+v"(v_nb1), [suma] "+v"(v_sum), [k0] "+v"(v_k0), [vlo0] "+v"(v_vlo),
-                  [vhi0] "+v"(v_vhi), [rowk] "+v"(v_rowk), [rowv] "+v"(v_rowv), [c0s] "+v"(v_c0s), [qaddr] "+v"(v_q),
+                  [vhi0] "+v"(v_vhi), [rowk] "+v"(v_rowk), [rowv] "+v"(v_rowv), [c0s] "+v"(v_c0s),
                   [thr0] "+v"(v_thr0), [thr1] "+v"(v_thr1)
                 : [n_tiles] "s"(__builtin_amdgcn_readfirstlane(n_tiles)), [n_end] "s"(__builtin_amdgcn_readfirstlane(n_loop)),
                   [n_pipe] "s"(__builtin_amdgcn_readfirstlane(min(n_plain, n_loop))), [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)),
-                  [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)), [first] "s"(__builtin_amdgcn_readfirstlane((int)first_boundary)),
+                  [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)), [first] "s"(0),
                   [kstep] "s"(__builtin_amdgcn_readfirstlane(k_step)), [vstep] "s"(__builtin_amdgcn_readfirstlane(v_step)),
                   [ldsdst] "s"(lds_dst), [scale] "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, p.scale_log2))),
                   [klo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)kptr)), [khi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kptr >> 32))),
                   [vlo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)vptr)), [vhi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(vptr >> 32)))
                 : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", "s43", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
-            if (tile_s > tile) first_boundary = false;      // (every tile the block ran had its boundary)
             tile = tile_s;
             // status 0: tiles up to n_loop done.  1: tiles up to `tile` done, and the last of them took a row sum to 2.
             if (status != 0) {
@@ -536,10 +609,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 move_references(std::integral_constant<int, 1>{});
             }
         }
-
-        // ---- row sums; the workgroup meets (everybody is done with the K/V buffers) and, on the first attempt,
-        // votes on doing the query tile again ----
-        float l_row[2];
+        // row sums
         const auto read_sums = [&](auto c_c) {
             constexpr int c = decltype(c_c)::value;
             float s_lo, s_hi;
@@ -549,28 +619,39 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         };
         read_sums(std::integral_constant<int, 0>{});
         read_sums(std::integral_constant<int, 1>{});
-        if (preset) {
-            // (rows past the end of the sequence count too: their sums are sk * 2^-32, far above the lower limit)
-            const bool bad = redo || !(l_row[0] >= kUnderflow) || !(l_row[1] >= kUnderflow) || !(l_row[0] <= kOverflow) ||
-                             !(l_row[1] <= kOverflow);
-            if (__syncthreads_or(bad ? 1 : 0)) continue;
-        } else {
+        // ---- the workgroup meets (everybody is done with the K/V buffers) and, the first time, votes: if some row's
+        // sum came out suspiciously small or large, the query tile is done again (rows past the end of the sequence
+        // count too: they repeat the last row) ----
+        if (!preset) {
             __syncthreads();
+            break;
         }
+        const bool bad = redo || !(l_row[0] >= kUnderflow) || !(l_row[1] >= kUnderflow) || !(l_row[0] <= kOverflow) ||
+                         !(l_row[1] <= kOverflow);
+        if (!__syncthreads_or(bad ? 1 : 0)) break;
+        redo = false;
+        }   // attempts
 
-        // the next job's first tiles and query rows are on their way while this one finishes
-        have_next = next_job(nxt);
-        if (have_next) prefetch(nxt);
-
-        // ---- normalise: lane owns query qw0 + 32c + n, d = 32dt + 8(i/4) + 4kg + i%4 ----
+        // ---- normalise: lane owns query qw0 + 32c + n, d = 32dt + 8(i/4) + 4kg + i%4; the rows of a block leave
+        // whole (written once, never read here: non-temporal, so that the K/V tiles keep the L2 to themselves).  The
+        // next job's first requests go out in between. ----
+        __bf16* const wave_out = cur.ob + (int64_t)qw0 * os2;                              // (wave-uniform)
+        const uint32_t lane_out = (uint32_t)(r0 * os2 + c16 * 8) * 2u;                     // bytes from there
+        auto out_row = [&](int r) {           // the lane's 16 bytes of the wavefront's row r + r0
+            return reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(wave_out + (int64_t)r * os2) + lane_out);
+        };
+        auto staged_row = [&](int i) {
+            // row 4i + r0 of the block: in the K share for i < 4, in the V share after; swz of it is (r0 << 2) | (i & 3)
+            return *reinterpret_cast<const u32x4*>(stage_r + (i / 4) * (2 * kWTile) + (i & 3) * (kRowsPerPass * kWRow) +
+                                                   ((c16 ^ ((r0 << 2) | (i & 3))) << 4));
+        };
         const auto store_block = [&](auto c_c) {
             constexpr int c = decltype(c_c)::value;
             const float inv = 1.0f / l_row[c];     // l == 0 (no key kept) -> NaN row, like the reference softmax
             // sum_j exp(scale * s_j) = l * 2^(-nb)  ->  lse = ln2 * (log2 l - nb); no key kept -> -inf
             if (cur.lb && kg == 0 && qw0 + 32 * c + n < sq)
                 cur.lb[qw0 + 32 * c + n] = l_row[c] > 0.f ? 0.69314718056f * (__log2f(l_row[c]) - nb[c]) : -INFINITY;
-            unsigned char* mine = slab + (32 * c + n) * kWORow + 8 * kg;
-            const auto store_dt = [&](auto dt_c) {
+            const auto stage_dt = [&](auto dt_c) {
                 constexpr int dt = decltype(dt_c)::value;
                 float x[16];
                 acc_read<c, dt>(x);
@@ -579,35 +660,49 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                     u32x2 w;
                     w[0] = pack_bf16(x[4 * g + 0] * inv, x[4 * g + 1] * inv);
                     w[1] = pack_bf16(x[4 * g + 2] * inv, x[4 * g + 3] * inv);
-                    *reinterpret_cast<u32x2*>(mine + (32 * dt + 8 * g) * 2) = w;
+                    *reinterpret_cast<u32x2*>(stage_w + (((4 * dt + g) ^ stage_wx) << 4)) = w;
                 }
+                if (have_next && 4 * c + dt < 6) prefetch_group(nxt, 4 * c + dt);
             };
-            store_dt(std::integral_constant<int, 0>{});
-            store_dt(std::integral_constant<int, 1>{});
-            store_dt(std::integral_constant<int, 2>{});
-            store_dt(std::integral_constant<int, 3>{});
+            stage_dt(std::integral_constant<int, 0>{});
+            stage_dt(std::integral_constant<int, 1>{});
+            stage_dt(std::integral_constant<int, 2>{});
+            stage_dt(std::integral_constant<int, 3>{});
+            if (qw0 + 64 <= sq) {                  // all rows exist: reads first, then the stores
+                u32x4 w[32 / kRowsPerPass];
+#pragma unroll
+                for (int i = 0; i < 32 / kRowsPerPass; ++i) w[i] = staged_row(i);
+#pragma unroll
+                for (int i = 0; i < 32 / kRowsPerPass; ++i) __builtin_nontemporal_store(w[i], out_row(32 * c + i * kRowsPerPass));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 32 / kRowsPerPass; ++i) {
+                    const u32x4 w = staged_row(i);
+                    const int r = 32 * c + i * kRowsPerPass;
+                    if (qw0 + r < sq) {                    // (wave-uniform: see row_passes)
+                        if (qw0 + r + r0 < sq) __builtin_nontemporal_store(w, out_row(r));
+                    }
+                }
+            }
         };
         store_block(std::integral_constant<int, 0>{});
         store_block(std::integral_constant<int, 1>{});
-        break;
-        }   // attempts
-        // ---- output rows leave whole, through the slab (written once, never read here: non-temporal, like the
-        // query rows, so that the K/V tiles keep the L2 to themselves) ----
-        int64_t out_off = (int64_t)(qw0 + r0) * p.os[2] + c16 * 8;
-        asm volatile("" : "+v"(out_off));                  // (as for the query rows: addresses computed here, not earlier)
-        __bf16* my_out = cur.ob + out_off;
-#pragma unroll
-        for (int i = 0; i < 64 / kRowsPerPass; ++i) {
-            const int r = i * kRowsPerPass + r0;
-            const u32x4 w = *reinterpret_cast<const u32x4*>(slab + r * kWORow + c16 * 16);
-            if (qw0 + i * kRowsPerPass < sq) {             // (wave-uniform: see row_passes)
-                if (qw0 + r < sq) __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(my_out + (int64_t)(i * kRowsPerPass) * p.os[2]));
-            }
-        }
-        prev_stores = row_passes(cur);
+        // (the stores above took their data from the staged rows, so every read of them has returned)
+        if (have_next) prefetch_group(nxt, 6);
+        // (the rows of block A leave before the last query rows of the next job are requested; those of block B after)
+        prev_stores = max(row_passes(cur) - 32 / kRowsPerPass, 0);
         cur = nxt;
         have = have_next;
     }
+}
+
+// The kernel multiplies head and row strides as 32-bit numbers (batch strides stay 64-bit).
+bool prefill_w64_takes(const PrefillParams& p) {
+    const int64_t strides[] = {p.qs[1], p.qs[2], p.ks[1], p.ks[2], p.vs[1], p.vs[2], p.os[1], p.os[2], p.lse ? p.ls[1] : 0};
+    for (int64_t v : strides)
+        if (v < 0 || v > 0x7fffffffLL) return false;
+    // a row offset inside a tile of 64 rows, in bytes, is a 32-bit number as well
+    return p.qs[2] < (1 << 23) && p.ks[2] < (1 << 23) && p.vs[2] < (1 << 23) && p.os[2] < (1 << 23);
 }
 
 int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {

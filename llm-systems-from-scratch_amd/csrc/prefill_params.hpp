@@ -39,6 +39,8 @@ struct PrefillParams {
 };
 
 // The 64-queries-per-wavefront kernel (head_dim 128, no mask or causal): prefill_fwd_w64.hip.
+// prefill_w64_takes: whether its 32-bit address arithmetic covers the strides of p.
+bool prefill_w64_takes(const PrefillParams& p);
 int launch_prefill_w64(const PrefillParams& p, hipStream_t stream);
 
 }  // namespace mi355
