@@ -62,7 +62,7 @@ Register map (physical, fixed; the block loads them itself from its operands, se
   a[200:215] K fragments (4 in flight), a[216:247] V^T fragments (8: 2 slices x 4 d-tiles): LDS reads land in
   AGPRs directly and the MFMAs take them as A operands, which leaves the vector registers to the compiler
   s[36:37] / s[38:39] global address of the wavefront's first DMA row of K[t+2] / V[t+1] (advanced per tile),
-  s40 / s41 bytes from one tile to the next in K / V, s43 "the next boundary is the query tile's first", s42 "a row sum reached 2"; every other scalar is a named operand
+  s40 / s41 bytes from one tile to the next in K / V, s42 "a row sum reached 2"; every other scalar is a named operand
 """
 import os
 
@@ -89,7 +89,7 @@ LREG = {"A": 128, "B": 132}
 QREG = {"A": 136, "B": 168}
 N_ACC = 136                         # a[0:135]: what ordinary code reaches through the snippets
 N_AGPRS = 248
-KPTR, VPTR, FLAG, KSTEP16, VSTEP16, FIRST = 36, 38, 42, 40, 41, 43
+KPTR, VPTR, FLAG, KSTEP16, VSTEP16 = 36, 38, 42, 40, 41
 K_TILE = 16384                      # bytes of one K (or V) tile in LDS: 64 rows x 256 bytes
 ROW = 256
 NONE = {"A": False, "B": False}
@@ -309,29 +309,12 @@ def dma_chunks(which, buf):
     return chunks
 
 
-_first_labels = [0]
-
-
-def wait_and_meet(e, maybe_first=False):
+def wait_and_meet(e):
     """First half of a boundary: all LDS reads of this wavefront have returned, its shares of K[t+1] and V[t] have
-    landed, and every wavefront of the workgroup is here.  maybe_first: this may be the first boundary of a query
-    tile, when the sixteen row stores of the query tile before it -- younger than every request in flight -- need
-    not be waited for (s43 says so; it is cleared here).  They take longer than the first tile step."""
+    landed, and every wavefront of the workgroup is here."""
     e.raw("; boundary")
     e.drain()
-    if maybe_first:
-        _first_labels[0] += 1
-        a, b = f"7{_first_labels[0]:03d}0", f"7{_first_labels[0]:03d}1"
-        e.raw(f"s_cmp_eq_u32 s{FIRST}, 0")
-        e.raw(f"s_cbranch_scc1 {a}f")
-        e.raw("s_waitcnt vmcnt(16)")
-        e.raw(f"s_mov_b32 s{FIRST}, 0")
-        e.raw(f"s_branch {b}f")
-        e.raw(f"{a}:")
-        e.raw("s_waitcnt vmcnt(0)")
-        e.raw(f"{b}:")
-    else:
-        e.raw("s_waitcnt vmcnt(0)")
+    e.raw("s_waitcnt vmcnt(0)")
     if "nobarrier" not in ABL:
         e.raw("s_barrier")
 
@@ -339,7 +322,7 @@ def wait_and_meet(e, maybe_first=False):
 def boundary_plain(e, buf, tag, after):
     """A whole boundary with nothing to interleave: the requests are jumped over when their tiles do not exist.
     `after` emits what follows the barrier and precedes the requests (LDS reads of the data that has just landed)."""
-    wait_and_meet(e, maybe_first=True)
+    wait_and_meet(e)
     after()
     e.raw("s_add_u32 %[t2], %[tile], 1")
     e.raw("s_cmp_ge_u32 %[t2], %[n_tiles]")
@@ -517,10 +500,10 @@ def pipeline(e, b, start, h0_start, dry=False):
         v_read(e, b, 0, 0)
         v_read(e, b, 0, 1)
 
-    def tail_variants(entries, tagbase, join_label, maybe_first=False):
+    def tail_variants(entries, tagbase, join_label):
         """boundary(t) and the rest of the half-step, in two variants: with and without the request of K[t+2]
         (V[t+1] is requested in H1)."""
-        wait_and_meet(e, maybe_first)
+        wait_and_meet(e)
         first_reads()
         e.raw("s_add_u32 %[t2], %[tile], 2")
         e.raw("s_cmp_lt_u32 %[t2], %[n_tiles]")
@@ -544,7 +527,7 @@ def pipeline(e, b, start, h0_start, dry=False):
     e.raw("; S(t,1) | E(t,0), boundary inside")
     pro = half_step(e, s_part=(b, 1, k_after_pro), o_part=None, valu=exp_ops(0, NONE), hold=3, span=12, a_posts=pro_posts)
     emit(e, pro[:12])                                      # steps 0..5
-    at_m = tail_variants(pro[12:], f"5{b}0", f"4{b}4f", maybe_first=True)
+    at_m = tail_variants(pro[12:], f"5{b}0", f"4{b}4f")
 
     # ---------------- H0(t): S(t,1) | E(t,0) | O(t-1,1) ----------------
     e.raw(f"4{b}1:")
@@ -633,7 +616,6 @@ def entry(e):
     e.raw(f"s_mov_b32 s{VPTR}, %[vlo]")
     e.raw(f"s_mov_b32 s{VPTR + 1}, %[vhi]")
     e.raw(f"s_mov_b32 s{FLAG}, 0")
-    e.raw(f"s_mov_b32 s{FIRST}, %[first]")
 
 
 def generate():

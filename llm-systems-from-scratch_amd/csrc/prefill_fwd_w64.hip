@@ -596,12 +596,12 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                   [thr0] "+v"(v_thr0), [thr1] "+v"(v_thr1)
                 : [n_tiles] "s"(__builtin_amdgcn_readfirstlane(n_tiles)), [n_end] "s"(__builtin_amdgcn_readfirstlane(n_loop)),
                   [n_pipe] "s"(__builtin_amdgcn_readfirstlane(min(n_plain, n_loop))), [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)),
-                  [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)), [first] "s"(0),
+                  [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)),
                   [kstep] "s"(__builtin_amdgcn_readfirstlane(k_step)), [vstep] "s"(__builtin_amdgcn_readfirstlane(v_step)),
                   [ldsdst] "s"(lds_dst), [scale] "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, p.scale_log2))),
                   [klo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)kptr)), [khi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kptr >> 32))),
                   [vlo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)vptr)), [vhi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(vptr >> 32)))
-                : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", "s43", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
+                : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
             tile = tile_s;
             // status 0: tiles up to n_loop done.  1: tiles up to `tile` done, and the last of them took a row sum to 2.
             if (status != 0) {
