@@ -28,6 +28,15 @@
 // diagonal and the tiles above it.  Ragged ends and the recomputation go through step_cxx below, ordinary HIP code
 // on the same state.
 //
+// Between query tiles: a workgroup is persistent and works through (batch, head, query tile) jobs.  The 64 query rows
+// of a wavefront reach its own part of LDS by direct-to-LDS loads (laid out like a K tile) and go from there into
+// AGPRs once per job; the output rows are normalised 32 at a time and leave whole through the wavefront's own shares
+// of the second K and V buffers, which nobody needs between the last tile of a job and the first boundary of the
+// next.  The next job is worked out at the top of the current one, and its first requests (K[0], query rows, V[0],
+// then K[1]) go out between the pieces of output work.  No ordinary vector load sits in the job loop, so the only
+// waits on memory are the ones written here (the compiler would add s_waitcnt vmcnt(0), which also waits for every
+// request in flight, in front of the first use of a loaded register).
+//
 // Hand-over protocol between the two (and between tiles), one "boundary" per tile t and wavefront: K[t] and V[t]
 // live in LDS buffers t % 2.  When tile t starts, K[t] has landed and the workgroup has met since; K[t+1] and V[t]
 // are in flight.  At boundary(t) the wavefront has read what it needs of K[t] and V[t-1]; it waits for its own
