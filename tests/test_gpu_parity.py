@@ -461,6 +461,23 @@ def test_prefill_head_dim_128_packed_sequences_of_drawn_lengths(ops, seed):
     torch.testing.assert_close(lse.cpu(), torch.cat(scores, 1), atol=3e-3, rtol=1e-3)
 
 
+def test_prefill_head_dim_128_rows_too_far_apart_for_the_64_query_kernel(ops):
+    """The 64-query kernel multiplies row strides as 32-bit byte offsets inside a tile; a query tensor whose rows lie
+    2^23 elements apart (a view into a 1 GiB buffer) must be sent to the other kernel, not read from wrapped
+    addresses.  Same inputs, contiguous, give the comparison."""
+    Sq, D = 64, 128
+    print("case: head_dim 128, query row stride 2^23 elements", flush=True)
+    q, k, v = rnd(1, 1, Sq, D, seed=71), rnd(1, 1, 300, D, seed=72), rnd(1, 1, 300, D, seed=73)
+    big = torch.zeros(Sq * (1 << 23), dtype=torch.bfloat16, device="cuda")
+    q_far = big.as_strided((1, 1, Sq, D), (0, 0, 1 << 23, 1))
+    q_far.copy_(q.cuda())
+    ref = orc.prefill_reference(q, k, v, causal=True)
+    got = ops.flash_attn_prefill(q_far, k.cuda(), v.cuda(), causal=True, kv_splits=1)
+    check(got, ref, what="rows 2^23 elements apart")
+    del big, q_far
+    torch.cuda.empty_cache()
+
+
 def _reference_module_tensors(x_proj, freq, num_heads, amp):
     """Q, K, V exactly as CausalMultiHeadSelfAttention.forward hands them to the attention call
     (llm-core/llm_core/model.py:362-378) from the three projection outputs (B, S, H*d): `rearrange` views, then
