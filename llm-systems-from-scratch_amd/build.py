@@ -6,8 +6,10 @@ Python package so the built library travels with the source tree)
 from __future__ import annotations
 
 import os
+import re
 import subprocess
 import sys
+import tempfile
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -44,6 +46,39 @@ def library_path() -> str:
     return os.path.join(OUT_DIR, LIB_NAME)
 
 
+def check_w64_registers() -> str:
+    """prefill_fwd_w64.hip keeps values in a[0:N_AGPRS-1] across its assembly statements, behind the compiler's back:
+    the statements name those registers as clobbered, so the compiler holds nothing of its own in them ACROSS a
+    statement, but nothing in the language keeps it from using one BETWEEN two statements (as a spill slot, say).
+    This compiles the file to assembly and fails the build if any instruction outside the statements touches one."""
+    n_agprs = 0
+    with open(os.path.join(CSRC, "prefill_w64_asm.inc")) as f:
+        for line in f:
+            if line.startswith("#define W64_CLOBBER_ACC"):
+                n_agprs = line.count('"a')
+    if n_agprs == 0:
+        raise RuntimeError("prefill_w64_asm.inc: no W64_CLOBBER_ACC")
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, "w64.s")
+        _run([HIPCC, *FLAGS, *EXTRA_FLAGS["prefill_fwd_w64.hip"], "-S", "--cuda-device-only",
+              os.path.join(CSRC, "prefill_fwd_w64.hip"), "-o", asm])
+        inside, bad = False, []
+        with open(asm) as f:
+            for no, line in enumerate(f, 1):
+                if "#ASMSTART" in line:
+                    inside = True
+                elif "#ASMEND" in line:
+                    inside = False
+                elif not inside and not line.lstrip().startswith((";", ".")):
+                    for m in re.finditer(r"\ba\[(\d+):\d+\]|\ba(\d+)\b", line.split(";")[0]):
+                        if int(m.group(1) or m.group(2)) < n_agprs:
+                            bad.append("%d: %s" % (no, line.strip()))
+        if bad:
+            raise RuntimeError("prefill_fwd_w64.hip: compiler-generated code touches AGPRs below a%d, which the "
+                               "assembly statements own:\n%s" % (n_agprs, "\n".join(bad[:20])))
+    return "prefill_fwd_w64.hip: no compiler-generated instruction touches a[0:%d]" % (n_agprs - 1)
+
+
 def build_library(verbose: bool = True) -> str:
     # the hand-scheduled assembly of prefill_fwd_w64.hip is generated text: regenerate it so that it cannot go stale
     _run([sys.executable, os.path.join(CSRC, "gen_prefill_w64_loop.py")])
@@ -57,7 +92,11 @@ def build_library(verbose: bool = True) -> str:
         return obj, log
 
     with ThreadPoolExecutor(max_workers=4) as ex:
+        check = ex.submit(check_w64_registers)
         results = list(ex.map(compile_one, srcs))
+        note = check.result()
+    if verbose:
+        print(note)
     for _, log in results:
         if verbose and log.strip():
             print(log)
