@@ -732,6 +732,9 @@ extern "C" int mi355_prefill_suggest_kv_splits(int B, int Hq, int D, int Sq_max,
             return 1;
     }
     const int nq = (Sq_max + kBM - 1) / kBM, n_pairs = (nq + 1) / 2;
+    // (the unsplit head_dim 128 kernel gives every query tile a workgroup of its own when there are enough compute
+    // units for that; the split kernel always works on pairs)
+    const bool single_tiles = D == 128 && (int64_t)nq * Hq * B <= n_cu;
     const double jobs = (double)n_pairs * Hq * B;
     // K/V tiles and query tiles of the heaviest workgroup (a pair of query tiles; causal: bottom-right diagonal)
     const double halves = nq >= 2 ? 2.0 : 1.0;
@@ -743,7 +746,11 @@ extern "C" int mi355_prefill_suggest_kv_splits(int B, int Hq, int D, int Sq_max,
     }
     const double tiles = keys / kBN;
     const auto rounds = [&](double wgs) { return (double)(int64_t)((wgs + n_cu - 1) / n_cu); };
-    const double plain = rounds(jobs) * (tiles * 1.5 + 5.0 * halves);
+    double plain = rounds(jobs) * (tiles * 1.5 + 5.0 * halves);
+    if (single_tiles) {
+        const double heaviest = causal ? (double)(Sk_max > Sq_max ? Sk_max - Sq_max : 0) + Sq_max : (double)Sk_max;
+        plain = (heaviest < Sk_max ? heaviest : (double)Sk_max) / kBN * 1.5 + 5.0;
+    }
     double best = plain * 0.85;                       // a split must win clearly
     int best_n = 1;
     static const int kCandidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};

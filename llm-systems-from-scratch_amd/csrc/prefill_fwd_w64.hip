@@ -142,7 +142,7 @@ __device__ __forceinline__ void load_bounds(const int32_t* cu_q, const int32_t* 
 }
 
 template <bool CAUSAL>
-__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int n_logical) {
+__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int n_logical, int tiles_per_id) {
     constexpr int D = kWD, NS = D / 16, NDT = D / 32, CPR = D / 8;
     constexpr float kBias = 32.0f;             // the largest weight sits at 2^-kBias when a reference is set
     constexpr float kUnderflow = 0x1p-92f;     // a row sum below this may have lost terms (see the file header)
@@ -164,7 +164,9 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     // ---- jobs: a workgroup works through query tiles, one "job" each.  Logical id = (batch, head, tile pair); a
     // pair is the query tiles (nq-1-i, i) of a sequence, so that causal work is the same for every id.  The ids are
     // dealt so that the workgroups resident on one XCD (workgroup ids are dealt round-robin to the 8 XCDs) walk
-    // through one contiguous range of ids together and stream the same K/V through that XCD's L2. ----
+    // through one contiguous range of ids together and stream the same K/V through that XCD's L2.
+    // (tiles_per_id == 1: an id is a single query tile nq-1-i, and p.n_pairs counts tiles.  The launch code chooses
+    // that when every query tile can have a compute unit of its own.) ----
     struct Job {
         const __bf16 *qb, *kb, *vb;
         __bf16* ob;
@@ -197,13 +199,13 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     };
     auto next_job = [&](Job& j, const Job& prev) -> bool {
         j = prev;                             // the sequence-level fields stay while the id stays
-        if (job_half == 0 && job_pair != job_nq - 1 - job_pair) {           // second query tile of the pair
+        if (tiles_per_id == 2 && job_half == 0 && job_pair != job_nq - 1 - job_pair) {      // second query tile of the pair
             job_half = 1;
             j.q0 = job_pair * kWBM;
             return true;
         }
         job_pair += n_pairs;                  // a further pair of the same sequence: only if it is longer than Sq_max promised
-        while (!(job_k >= 0 && 2 * job_pair < job_nq)) {
+        while (!(job_k >= 0 && tiles_per_id * job_pair < job_nq)) {
             if (job_k >= 0) {
                 id += id_step;
                 id_pair += st_pair;
@@ -720,15 +722,23 @@ int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
     hipError_t e = hipGetDevice(&dev);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return (int)e;
-    const int n_logical = p.n_pairs * p.Hq * p.B;
+    // Ids are pairs of query tiles (equal causal work per id) unless every single tile can have a compute unit of
+    // its own: then pairing would only leave half of those idle.
+    PrefillParams q = p;
+    int tiles_per_id = 2;
+    if ((int64_t)p.n_qtiles * p.Hq * p.B <= n_cu) {
+        tiles_per_id = 1;
+        q.n_pairs = p.n_qtiles;
+    }
+    const int n_logical = q.n_pairs * q.Hq * q.B;
     if (n_logical <= 0) return 0;
     int grid = n_logical < n_cu ? n_logical : n_cu;
     if (n_logical % 8 == 0 && grid >= 8) grid -= grid % 8;          // whole number of workgroups per XCD
     dim3 block(kWWaves * 64);
     if (p.mask_mode == MI355_MASK_CAUSAL)
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), dim3((unsigned)grid), block, 0, stream, p, n_logical);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), dim3((unsigned)grid), block, 0, stream, q, n_logical, tiles_per_id);
     else
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), dim3((unsigned)grid), block, 0, stream, p, n_logical);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), dim3((unsigned)grid), block, 0, stream, q, n_logical, tiles_per_id);
     return (int)hipGetLastError();
 }
 

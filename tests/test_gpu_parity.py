@@ -461,6 +461,29 @@ def test_prefill_head_dim_128_packed_sequences_of_drawn_lengths(ops, seed):
     torch.testing.assert_close(lse.cpu(), torch.cat(scores, 1), atol=3e-3, rtol=1e-3)
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_prefill_head_dim_128_paired_query_tiles_on_ragged_sequences(ops, seed):
+    """Enough (sequence, head, query tile) triples that the persistent kernel deals PAIRS of query tiles to its
+    workgroups (with fewer triples than compute units it deals single tiles, which is what the small shapes of the
+    other tests get): ragged packed sequences, 32 query heads on 8 kv heads, causal and not, one promised maximum that
+    is too small."""
+    g = torch.Generator().manual_seed(4000 + seed)
+    Hq, Hkv, D = 32, 8, 128
+    lens = [int(x) for x in torch.randint(520, 1000, (3,), generator=g)]        # 3 or 4 query tiles each: > 256 triples
+    lens[seed % 3] = 1 + int(torch.randint(0, 255, (1,), generator=g))
+    print(f"case: paired query tiles seed={seed} lens={lens}", flush=True)
+    T = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q, k, v = rnd(T, Hq, D, seed=4100 + seed), rnd(T, Hkv, D, seed=4200 + seed), rnd(T, Hkv, D, seed=4300 + seed)
+    for causal in (True, False):
+        ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=causal)
+        got = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens),
+                                            causal=causal, kv_splits=1)
+        check(got, ref, what=f"paired query tiles, causal={causal}")
+    short = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), 600, 600, causal=True, kv_splits=1)
+    check(short, orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True), what="paired query tiles, promised maximum too small")
+
+
 def test_prefill_head_dim_128_rows_too_far_apart_for_the_64_query_kernel(ops):
     """The 64-query kernel multiplies row strides as 32-bit byte offsets inside a tile; a query tensor whose rows lie
     2^23 elements apart (a view into a 1 GiB buffer) must be sent to the other kernel, not read from wrapped
