@@ -459,7 +459,7 @@ def bench_prefill_few_sequences(args):
                                    "head_dim 128, dense layout" % (Sq, Sk)},
             "roofline": {"bound": "mfma",
                          "kernel": "prefill_fwd_w64_kernel<causal>" if n_split == 1 else
-                                   "prefill_fwd_kernel<128, causal> (keys split %d ways) + prefill_merge_kernel" % n_split,
+                                   "prefill_fwd_w64_kernel<causal> (keys split %d ways) + prefill_merge_kernel" % n_split,
                          "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms, "traffic": None},
         }

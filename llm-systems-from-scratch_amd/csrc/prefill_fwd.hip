@@ -621,7 +621,8 @@ static int prefill_common(const void* q, const void* k, const void* v, void* out
     hipStream_t s = (hipStream_t)stream;
     int rc;
     if (p.n_split > 1) {
-        rc = D == 128 ? launch_prefill<128>(p, s) : (D == 64 ? launch_prefill<64>(p, s) : launch_prefill<32>(p, s));
+        if (D == 128 && mask_mode != MI355_MASK_BOOL && prefill_w64_takes(p)) rc = launch_prefill_w64(p, s);
+        else rc = D == 128 ? launch_prefill<128>(p, s) : (D == 64 ? launch_prefill<64>(p, s) : launch_prefill<32>(p, s));
         if (rc == 0) rc = launch_merge(p, D, s);
         if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
         return MI355_OK;
@@ -720,7 +721,8 @@ extern "C" size_t mi355_prefill_splitkv_workspace_bytes(int64_t total_q_rows, in
 // Cost model behind mi355_prefill_suggest_kv_splits, in microseconds, from timings on an MI355X (32 and 8 query
 // heads, head_dim 128, 64..2048 query rows over 1.5K..32K keys): a workgroup spends about 1.5 us per K/V tile of 64
 // keys (1.6 us in the split kernel) and 5 us per query tile outside the tile loop; the partial rows cost their bytes
-// twice (written, then read by the merge) at about 2.5 TB/s, plus 8 us for the second launch.
+// twice (written, then read by the merge) at about 2.5 TB/s, plus 8 us for the second launch.  Head_dim 128 runs on
+// the persistent 64-query kernel, split or not, and has figures of its own (below).
 extern "C" int mi355_prefill_suggest_kv_splits(int B, int Hq, int D, int Sq_max, int Sk_max, int64_t total_q_rows,
                                                int causal, int n_compute_units) {
     if (B <= 0 || Hq <= 0 || D <= 0 || Sq_max <= 0 || Sk_max <= 0 || total_q_rows <= 0) return 1;
@@ -732,32 +734,51 @@ extern "C" int mi355_prefill_suggest_kv_splits(int B, int Hq, int D, int Sq_max,
             return 1;
     }
     const int nq = (Sq_max + kBM - 1) / kBM, n_pairs = (nq + 1) / 2;
-    // (the unsplit head_dim 128 kernel gives every query tile a workgroup of its own when there are enough compute
-    // units for that; the split kernel always works on pairs)
-    const bool single_tiles = D == 128 && (int64_t)nq * Hq * B <= n_cu;
-    const double jobs = (double)n_pairs * Hq * B;
-    // K/V tiles and query tiles of the heaviest workgroup (a pair of query tiles; causal: bottom-right diagonal)
-    const double halves = nq >= 2 ? 2.0 : 1.0;
-    double keys = halves * Sk_max;
+    const double over = causal && Sk_max > Sq_max ? Sk_max - Sq_max : 0;            // keys every query sees (causal)
+    // K/V tiles of the heaviest single query tile and of the heaviest pair (causal: bottom-right diagonal)
+    double keys_single = Sk_max, keys_pair = (nq >= 2 ? 2.0 : 1.0) * Sk_max;
     if (causal) {
-        const int over = Sk_max > Sq_max ? Sk_max - Sq_max : 0;         // keys every query sees
-        keys = nq >= 2 ? 2.0 * over + Sq_max + kBM : (double)over + (Sq_max < kBM ? Sq_max : kBM);
-        if (keys > halves * Sk_max) keys = halves * Sk_max;
+        keys_single = over + Sq_max;
+        keys_pair = nq >= 2 ? 2.0 * over + Sq_max + kBM : over + (Sq_max < kBM ? Sq_max : kBM);
+        if (keys_single > Sk_max) keys_single = Sk_max;
+        if (keys_pair > (nq >= 2 ? 2.0 : 1.0) * Sk_max) keys_pair = (nq >= 2 ? 2.0 : 1.0) * Sk_max;
     }
-    const double tiles = keys / kBN;
+    const double halves = nq >= 2 ? 2.0 : 1.0;
     const auto rounds = [&](double wgs) { return (double)(int64_t)((wgs + n_cu - 1) / n_cu); };
-    double plain = rounds(jobs) * (tiles * 1.5 + 5.0 * halves);
-    if (single_tiles) {
-        const double heaviest = causal ? (double)(Sk_max > Sq_max ? Sk_max - Sq_max : 0) + Sq_max : (double)Sk_max;
-        plain = (heaviest < Sk_max ? heaviest : (double)Sk_max) / kBN * 1.5 + 5.0;
-    }
-    double best = plain * 0.85;                       // a split must win clearly
+    const auto partials = [&](int n) { return 8.0 + 2.0 * ((double)total_q_rows * Hq * (D + 1) * 4.0 * n) / 2.5e6; };
+    double plain;
     int best_n = 1;
     static const int kCandidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
+    if (D == 128) {
+        // The persistent 64-query kernel serves both: a workgroup per query tile and share while there are compute units
+        // for all of them, per pair of query tiles otherwise; 1.45 us per K/V tile on a busy GPU, 1.25 us when at most
+        // three quarters of the compute units have a workgroup (the clock is higher then), 5 us per query tile around
+        // the tile loop.
+        const auto time_of = [&](int n) {
+            const double singles = (double)nq * Hq * B * n;
+            if (singles <= n_cu) return keys_single / n / kBN * (singles >= 0.75 * n_cu ? 1.45 : 1.25) + 5.0;
+            const double wgs = (double)n_pairs * Hq * B * n;
+            return rounds(wgs) * (keys_pair / n / kBN * (wgs >= 0.75 * n_cu ? 1.45 : 1.25) + 5.0 * halves);
+        };
+        plain = time_of(1);
+        double best = plain * 0.85;                   // a split must win clearly
+        for (int n : kCandidates) {
+            if (keys_single / kBN / n < 2.0) break;   // at least two tiles per share and query tile
+            const double t = time_of(n) + partials(n);
+            if (t < best) {
+                best = t;
+                best_n = n;
+            }
+        }
+        return best_n;
+    }
+    const double jobs = (double)n_pairs * Hq * B;
+    const double tiles = keys_pair / kBN;
+    plain = rounds(jobs) * (tiles * 1.5 + 5.0 * halves);
+    double best = plain * 0.85;                       // a split must win clearly
     for (int n : kCandidates) {
         if (tiles / n < 2.0 * halves) break;          // at least two tiles per share and query tile
-        const double bytes = (double)total_q_rows * Hq * (D + 1) * 4.0 * n;
-        const double t = rounds(jobs * n) * (tiles / n * 1.6 + 5.0 * halves) + 8.0 + 2.0 * bytes / 2.5e6;
+        const double t = rounds(jobs * n) * (tiles / n * 1.6 + 5.0 * halves) + partials(n);
         if (t < best) {
             best = t;
             best_n = n;

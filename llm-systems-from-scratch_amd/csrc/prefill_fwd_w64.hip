@@ -172,7 +172,12 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         __bf16* ob;
         float* lb;                       // row 0 of this (sequence, head) in the log-sum-exp output, or null
         int sq, sk, q0;
+        int split;                       // which share of the query tile's K/V tiles (0 when the keys are not split)
     };
+    // Split keys (p.n_split > 1): an id is (batch, head, tile pair, share); a job works on its share of the K/V tiles and
+    // writes, instead of output rows, a normalised fp32 partial row and its log-sum-exp per query, which a second
+    // kernel merges.  `ob` and `lb` of such a job point at row 0 of its (share, head, sequence) in the two partial buffers.
+    const int n_split = p.n_split > 1 ? p.n_split : 1;
     // head and row strides fit 32 bits (the host checks), so an address takes two scalar multiplications
     const int qs2 = (int)p.qs[2], ks2 = (int)p.ks[2], vs2 = (int)p.vs[2], os2 = (int)p.os[2];
     const int n_pairs = p.n_pairs, Hq = p.Hq;
@@ -183,8 +188,10 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const int id_end = by_xcd ? (bid % 8 + 1) * (n_logical / 8) : n_logical;
     int id = by_xcd ? (bid % 8) * (n_logical / 8) + bid / 8 : bid;
     // (pair, head, batch) of id and of id_step: an id advances digit by digit, with no division per job
-    int id_pair = id % n_pairs, id_h = (id / n_pairs) % Hq, id_b = id / (n_pairs * Hq);
-    const int st_pair = id_step % n_pairs, st_h = (id_step / n_pairs) % Hq, st_b = id_step / (n_pairs * Hq);
+    int id_split = id % n_split, id_pair = (id / n_split) % n_pairs, id_h = (id / (n_split * n_pairs)) % Hq,
+        id_b = id / (n_split * n_pairs * Hq);
+    const int st_split = id_step % n_split, st_pair = (id_step / n_split) % n_pairs,
+              st_h = (id_step / (n_split * n_pairs)) % Hq, st_b = id_step / (n_split * n_pairs * Hq);
     const int group = Hq / p.Hkv, group_shift = (group & (group - 1)) == 0 ? __builtin_ctz(group) : -1;
     int job_k = -1, job_nq = 0, job_pair = 0, job_half = 1;      // position: "after the last query tile of id number job_k"
     // next_job(j, prev): the job after `prev` (whatever `prev` holds before the first).
@@ -208,8 +215,11 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         while (!(job_k >= 0 && tiles_per_id * job_pair < job_nq)) {
             if (job_k >= 0) {
                 id += id_step;
-                id_pair += st_pair;
-                int carry = id_pair >= n_pairs;
+                id_split += st_split;
+                int carry = id_split >= n_split;
+                id_split -= carry ? n_split : 0;
+                id_pair += st_pair + carry;
+                carry = id_pair >= n_pairs;
                 id_pair -= carry ? n_pairs : 0;
                 id_h += st_h + carry;
                 carry = id_h >= Hq;
@@ -231,6 +241,11 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 j.vb = a->v + ((int64_t)k_start * vs2 + (int64_t)hk * vs1);
                 j.ob = a->out + ((int64_t)q_start * os2 + (int64_t)h * os1);
                 j.lb = a->lse ? a->lse + (q_start + (int64_t)h * ls1) : nullptr;
+                if (n_split > 1) {
+                    const int64_t prow = ((int64_t)id_split * Hq + h) * a->part_rows + q_start;
+                    j.ob = reinterpret_cast<__bf16*>(a->part_o + prow * kWD);
+                    j.lb = a->part_lse + prow;
+                }
             } else {
                 j.sq = a->Sq;
                 j.sk = a->Sk;
@@ -239,7 +254,13 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 j.vb = a->v + ((int64_t)b * a->vs[0] + (int64_t)hk * vs1);
                 j.ob = a->out + ((int64_t)b * a->os[0] + (int64_t)h * os1);
                 j.lb = a->lse ? a->lse + ((int64_t)b * a->ls[0] + (int64_t)h * ls1) : nullptr;
+                if (n_split > 1) {
+                    const int64_t prow = ((int64_t)id_split * Hq + h) * a->part_rows + (int64_t)b * a->Sq;
+                    j.ob = reinterpret_cast<__bf16*>(a->part_o + prow * kWD);
+                    j.lb = a->part_lse + prow;
+                }
             }
+            j.split = id_split;
             job_nq = (j.sq + kWBM - 1) / kWBM;
             job_pair = id_pair;
         }
@@ -289,6 +310,18 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         int kv_end = jb.sk;
         if (CAUSAL) kv_end = max(0, min(jb.sk, min(jb.sq, jb.q0 + kWBM) + (jb.sk - jb.sq)));
         return (kv_end + kWBN - 1) / kWBN;
+    };
+
+    // first and one-past-last tile of a job's share
+    auto share_of = [&](const Job& jb, int& t0, int& t1) {
+        const int nt = tiles_of(jb);
+        t0 = 0;
+        t1 = nt;
+        if (n_split > 1) {
+            const int per = (nt + n_split - 1) / n_split;
+            t0 = min(nt, jb.split * per);
+            t1 = min(nt, t0 + per);
+        }
     };
 
     // ---- per-lane LDS read addresses for buffer 0 (absolute: the assembly loop uses them as they are) ----
@@ -355,7 +388,9 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
 
     // ---- output rows leave whole, 32 at a time, through LDS: through the wavefront's own shares of the second K and
     // V buffers (the 16 rows each that its own direct-to-LDS loads fill), which are idle between the last tile of a
-    // job and the requests of K[1] / V[1] of the next.  Rows of 256 bytes, chunk c of row r at c ^ swz(r). ----
+    // job and the requests of K[1] / V[1] of the next.  Rows of 256 bytes, chunk c of row r at c ^ swz(r).
+    // (Jobs on split keys, whose first tile may live in either buffer, write fp32 partial rows straight from their
+    // registers instead.) ----
     constexpr int kRowsPerPass = 64 / CPR;           // a store instruction takes 4 whole rows
     const int c16 = lane % CPR, r0 = lane / CPR;
     unsigned char* const stage_w = kv_lds + ((n < 16) ? 1 : 3) * kWTile + wave * 4096 + (n & 15) * kWRow + 8 * kg;   // the lane's row n
@@ -368,14 +403,16 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     // they go out one group at a time between pieces of vector work, so that the wavefront does not sit behind a
     // full request queue (the four wavefronts all do this at the same time).
     auto prefetch_group = [&](const Job& jb, int group) {
+        int t0, t1;
+        share_of(jb, t0, t1);
         if (group == 0) {
-            if (tiles_of(jb) > 0) issue_k(jb, 0, 0);
+            if (t1 > t0) issue_k(jb, t0, t0 & 1);
         } else if (group <= 4) {
             issue_q(jb, group - 1);
         } else if (group == 5) {
-            if (tiles_of(jb) > 0) issue_v(jb, 0, 0);
+            if (t1 > t0) issue_v(jb, t0, t0 & 1);
         } else {
-            if (tiles_of(jb) > 1) issue_k(jb, 1, 1);
+            if (t1 > t0 + 1) issue_k(jb, t0 + 1, (t0 + 1) & 1);
         }
     };
     // number of output row stores a job issues at its end (four whole rows each): a pass whose four rows all lie
@@ -413,7 +450,9 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         const int sq = cur.sq, sk = cur.sk, q0 = cur.q0;
         const int coff = sk - sq;                          // bottom-right aligned causal diagonal
         const int qw0 = q0 + 64 * wave;                    // first query of this wavefront
-        const int n_tiles = tiles_of(cur);
+        // the job's tiles are [t_first, n_tiles): all of the query tile's, or its share of them
+        int t_first, n_tiles;
+        share_of(cur, t_first, n_tiles);
         // tile kinds of this wavefront: [0, n_plain) every key visible to each of its queries, [n_plain, n_mask) some,
         // [n_mask, n_tiles) none (the wavefront then only takes part in the hand-over)
         int n_plain = sk / kWBN, n_mask = n_tiles;
@@ -427,13 +466,14 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         // the assembly loop requests tile+2 with whole-tile loads: it may run tile t only if tile t+2 is a whole tile
         // (or does not exist), so it stops three tiles before a partial last tile
         const int n_asm = n_tiles > sk / kWBN ? max(0, n_tiles - 3) : n_tiles;
+        const int share_tiles = n_tiles - t_first;
         // the job after this one (scalar work, done while the first tile is still landing)
         const bool have_next = next_job(nxt, cur);
 
         // per column block: r_ref exponent reference in the log2 domain (-inf: none yet), nb = -r_ref - kBias
         float r_ref[2], nb[2], l_row[2];
         bool redo = false;                    // a row sum left the range in which no term can have been lost
-        const int young_dma = (n_tiles > 1 ? 4 : 0) + (n_tiles > 0 ? 4 : 0);      // requests of V[0] and K[1]
+        const int young_dma = (share_tiles > 1 ? 4 : 0) + (share_tiles > 0 ? 4 : 0);      // requests of the first V and the second K tile
 
         // Ordinary code for single tiles.  Everything it derives from the job goes through `fresh`, a copy of the few
         // values it needs that the compiler cannot trace back: what could be computed once per job would otherwise
@@ -562,9 +602,9 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         if (!preset) {                        // start over: the buffers are free (everybody passed the vote below)
             Job jc = cur;
             asm volatile("" : "+s"(jc.kb), "+s"(jc.vb), "+s"(jc.sk));
-            if (n_tiles > 0) issue_k(jc, 0, 0);
-            if (n_tiles > 1) issue_k(jc, 1, 1);
-            if (n_tiles > 0) issue_v(jc, 0, 0);
+            if (share_tiles > 0) issue_k(jc, t_first, t_first & 1);
+            if (share_tiles > 1) issue_k(jc, t_first + 1, (t_first + 1) & 1);
+            if (share_tiles > 0) issue_v(jc, t_first, t_first & 1);
         }
         asm volatile(W64_ZERO : : "v"(as_bf16x8(u32x4{0u, 0u, 0u, 0u})) : W64_CLOBBER_ACC);      // O^T and the row sums
         r_ref[0] = r_ref[1] = preset ? 0.f : -INFINITY;
@@ -577,7 +617,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             asm volatile(W64_QFRAGS : "=&v"(scratch) : "v"(q_rd0) : "memory", W64_CLOBBER_ACC);
         }
         __syncthreads();                      // everybody's share of K[0] is in
-        int tile = 0;
+        int tile = t_first;
         const int n_loop = preset ? n_asm : 0;
         while (tile < n_tiles) {
             if (tile >= n_loop) {
@@ -637,8 +677,13 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             __syncthreads();
             break;
         }
-        const bool bad = redo || !(l_row[0] >= kUnderflow) || !(l_row[1] >= kUnderflow) || !(l_row[0] <= kOverflow) ||
-                         !(l_row[1] <= kOverflow);
+        // (a query that sees none of the job's keys -- causal with fewer keys than queries, or a share of split keys
+        // that lies past its diagonal -- has a sum of zero by right)
+        const int k_first = t_first * kWBN;
+        const bool sees0 = k_first < sk && (!CAUSAL || k_first <= qw0 + n + coff);
+        const bool sees1 = k_first < sk && (!CAUSAL || k_first <= qw0 + 32 + n + coff);
+        const bool bad = redo || (sees0 && !(l_row[0] >= kUnderflow)) || (sees1 && !(l_row[1] >= kUnderflow)) ||
+                         !(l_row[0] <= kOverflow) || !(l_row[1] <= kOverflow);
         if (!__syncthreads_or(bad ? 1 : 0)) break;
         redo = false;
         }   // attempts
@@ -646,6 +691,43 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         // ---- normalise: lane owns query qw0 + 32c + n, d = 32dt + 8(i/4) + 4kg + i%4; the rows of a block leave
         // whole (written once, never read here: non-temporal, so that the K/V tiles keep the L2 to themselves).  The
         // next job's first requests go out in between. ----
+        if (n_split > 1) {
+            // partial result of this share of the keys: normalised fp32 rows and their log-sum-exp (-inf and zeros when
+            // the share kept no key for the row), straight from the registers; the merge kernel weighs them
+            float* const part = reinterpret_cast<float*>(cur.ob);
+            const auto partial_block = [&](auto c_c) {
+                constexpr int c = decltype(c_c)::value;
+                const int qi = qw0 + 32 * c + n;
+                const bool q_ok = qi < sq;
+                const float inv_p = l_row[c] > 0.f ? 1.0f / l_row[c] : 0.f;
+                if (q_ok && kg == 0)
+                    cur.lb[qi] = l_row[c] > 0.f ? 0.69314718056f * (__log2f(l_row[c]) - nb[c]) : -INFINITY;
+                float* const po = part + (int64_t)qi * D + 4 * kg;
+                const auto store_dt = [&](auto dt_c) {
+                    constexpr int dt = decltype(dt_c)::value;
+                    float x[16];
+                    acc_read<c, dt>(x);
+                    if (q_ok) {
+#pragma unroll
+                        for (int g = 0; g < 4; ++g)
+                            *reinterpret_cast<f32x4*>(po + 32 * dt + 8 * g) =
+                                f32x4{x[4 * g] * inv_p, x[4 * g + 1] * inv_p, x[4 * g + 2] * inv_p, x[4 * g + 3] * inv_p};
+                    }
+                    if (have_next && 4 * c + dt < 6) prefetch_group(nxt, 4 * c + dt);
+                };
+                store_dt(std::integral_constant<int, 0>{});
+                store_dt(std::integral_constant<int, 1>{});
+                store_dt(std::integral_constant<int, 2>{});
+                store_dt(std::integral_constant<int, 3>{});
+            };
+            partial_block(std::integral_constant<int, 0>{});
+            partial_block(std::integral_constant<int, 1>{});
+            if (have_next) prefetch_group(nxt, 6);
+            prev_stores = 0;                   // (the stores above are not counted: the next wait takes a few of them along)
+            cur = nxt;
+            have = have_next;
+            continue;
+        }
         __bf16* const wave_out = cur.ob + (int64_t)qw0 * os2;                              // (wave-uniform)
         const uint32_t lane_out = (uint32_t)(r0 * os2 + c16 * 8) * 2u;                     // bytes from there
         auto out_row = [&](int r) {           // the lane's 16 bytes of the wavefront's row r + r0
@@ -726,11 +808,13 @@ int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
     // its own: then pairing would only leave half of those idle.
     PrefillParams q = p;
     int tiles_per_id = 2;
-    if ((int64_t)p.n_qtiles * p.Hq * p.B <= n_cu) {
+    const int n_split = p.n_split > 1 ? p.n_split : 1;
+    if ((int64_t)p.n_qtiles * p.Hq * p.B * n_split <= n_cu) {
         tiles_per_id = 1;
         q.n_pairs = p.n_qtiles;
     }
-    const int n_logical = q.n_pairs * q.Hq * q.B;
+    if ((int64_t)q.n_pairs * q.Hq * q.B * n_split > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+    const int n_logical = q.n_pairs * q.Hq * q.B * n_split;
     if (n_logical <= 0) return 0;
     int grid = n_logical < n_cu ? n_logical : n_cu;
     if (n_logical % 8 == 0 && grid >= 8) grid -= grid % 8;          // whole number of workgroups per XCD
