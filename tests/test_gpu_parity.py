@@ -419,9 +419,12 @@ def test_prefill_head_dim_128_two_kernels_agree_on_random_shapes(ops, seed):
             keep = torch.tril(keep, diagonal=Sk - Sq)
         slow = ops.scaled_dot_product_attention(q.cuda(), k.cuda().repeat_interleave(Hq // Hkv, 1),
                                                 v.cuda().repeat_interleave(Hq // Hkv, 1), keep.cuda())
+        n_shares = 2 + (seed + case) % 3              # shares that start at odd and even tiles, some of them empty
+        shared = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=causal, kv_splits=n_shares)
         torch.cuda.synchronize()
         check(fast, ref, what=f"64-query kernel seed {seed} #{case}")
         check(slow, ref, what=f"8-wavefront kernel seed {seed} #{case}")
+        check(shared, ref, what=f"64-query kernel, keys split {n_shares} ways, seed {seed} #{case}")
 
 
 @pytest.mark.parametrize("seed", [0, 1, 2])
@@ -480,8 +483,12 @@ def test_prefill_head_dim_128_paired_query_tiles_on_ragged_sequences(ops, seed):
         got = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens),
                                             causal=causal, kv_splits=1)
         check(got, ref, what=f"paired query tiles, causal={causal}")
+    ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True)
     short = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), 600, 600, causal=True, kv_splits=1)
-    check(short, orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True), what="paired query tiles, promised maximum too small")
+    check(short, ref, what="paired query tiles, promised maximum too small")
+    shared = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens),
+                                           causal=True, kv_splits=3)
+    check(shared, ref, what="paired query tiles, keys split 3 ways")
 
 
 def test_prefill_head_dim_128_rows_too_far_apart_for_the_64_query_kernel(ops):
