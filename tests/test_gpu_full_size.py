@@ -134,6 +134,42 @@ def test_decode_full_size(ops, cfg):
     assert torch.equal(out, out2)
 
 
+def test_prefill_full_size_is_the_same_on_every_launch(ops):
+    """The persistent prefill kernel keeps its own books on what is in flight (query rows, K/V tiles and output rows
+    pass through the same LDS, requests of the next query tile are issued while the current one is stored): a wait
+    that is one request short shows up as a result that changes from launch to launch.  configs[2] at full size, and
+    ragged packed sequences with the log-sum-exp output, twenty launches each, bit for bit."""
+    from mi355_attn import workloads
+    from mi355_attn import ops as raw
+    print("case: prefill configs[2] full size, repeated launches", flush=True)
+    case = workloads.prefill_config(2, seed=1)
+    S = case.seqlen
+    first = ops.flash_attn_varlen_prefill(case.q, case.k, case.v, case.cu_seqlens, case.cu_seqlens, S, S, causal=True)
+    for i in range(20):
+        again = ops.flash_attn_varlen_prefill(case.q, case.k, case.v, case.cu_seqlens, case.cu_seqlens, S, S, causal=True)
+        assert torch.equal(first, again), f"launch {i + 1} differs from the first"
+    del first, again
+    print("case: ragged packed sequences with lse, repeated launches", flush=True)
+    g = torch.Generator().manual_seed(77)
+    lens = [int(x) for x in torch.randint(1, 3000, (24,), generator=g)]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32).cuda()
+    T = sum(lens)
+    gd = torch.Generator(device="cuda").manual_seed(78)
+    q = (torch.randn(T, 32, 128, generator=gd, device="cuda") * 0.5).to(torch.bfloat16)
+    k = (torch.randn(T, 8, 128, generator=gd, device="cuda") * 0.5).to(torch.bfloat16)
+    v = (torch.randn(T, 8, 128, generator=gd, device="cuda") * 0.5).to(torch.bfloat16)
+    out0, lse0 = raw._varlen(q, k, v, cu, cu, max(lens), max(lens), True, None, want_lse=True)
+    for i in range(20):
+        out1, lse1 = raw._varlen(q, k, v, cu, cu, max(lens), max(lens), True, None, want_lse=True)
+        assert torch.equal(out0, out1) and torch.equal(lse0, lse1), f"launch {i + 1} differs from the first"
+    for splits in (2, 5):
+        sp0 = ops.flash_attn_varlen_prefill(q, k, v, cu, cu, max(lens), max(lens), causal=True, kv_splits=splits)
+        for i in range(10):
+            sp1 = ops.flash_attn_varlen_prefill(q, k, v, cu, cu, max(lens), max(lens), causal=True, kv_splits=splits)
+            assert torch.equal(sp0, sp1), f"keys split {splits} ways: launch {i + 1} differs from the first"
+        assert (sp0.float() - out0.float()).abs().max().item() <= 2e-2
+
+
 def test_prefill_and_backward_full_size(ops):
     from mi355_attn import workloads
     print("case: prefill configs[2] full size", flush=True)
