@@ -430,9 +430,9 @@ def bench_prefill(cfg, args):
 
 
 def bench_prefill_few_sequences(args):
-    """Prefill of ONE sequence (what a per-request prefill of `generate` produces): whole long prompts, where the
-    launch of one workgroup per pair of query tiles still fills the GPU, and a chunk of a prompt over a long cached
-    context, where it does not and the keys are split over workgroups (mi355_prefill_fwd_splitkv)."""
+    """Prefill of ONE sequence (what a per-request prefill of `generate` produces): whole long prompts, whose query
+    tiles alone fill the GPU, and a chunk of a prompt over a long cached context, where they do not and the keys
+    are split over workgroups (mi355_prefill_fwd_splitkv).  Then one packed batch of very different lengths."""
     import torch
     import mi355_attn
 
@@ -468,6 +468,27 @@ def bench_prefill_few_sequences(args):
             res["unsplit_device_ms"] = one_ms
             res["speedup_over_unsplit"] = one_ms / dev_ms
         out[name] = res
+    # A packed batch of sequences of very different lengths (what a serving step's batched prefill looks like): the
+    # kernel deals its (sequence, head, query tile) jobs by cost, so the rate should stay near that of equal lengths.
+    import math
+    import random
+    rng = random.Random(args.seed + 11)
+    lens = [int(round(math.exp(rng.uniform(math.log(256), math.log(8192))))) for _ in range(16)]
+    T, longest = sum(lens), max(lens)
+    cu = torch.tensor([0] + [sum(lens[:i + 1]) for i in range(len(lens))], dtype=torch.int32, device="cuda")
+    q, k, v = rnd(T, Hq, D), rnd(T, Hkv, D), rnd(T, Hkv, D)
+    flops = sum(4.0 * Hq * D * n * n / 2.0 for n in lens)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.flash_attn_varlen_prefill(q, k, v, cu, cu, longest, longest, causal=True, kv_splits=1),
+                            steps, warmup, BURN_IN)
+    out["ragged_batch_16"] = {
+        "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
+        "algorithmic_flops": flops, "kv_splits": 1,
+        "config": {"workload": "causal prefill forward of 16 packed sequences, lengths log-uniform in [256, 8192] "
+                               "(%d tokens, longest %d), 32 q / 8 kv heads, head_dim 128" % (T, longest)},
+        "roofline": {"bound": "mfma", "kernel": "prefill_fwd_w64_kernel<causal>",
+                     "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms, "traffic": None},
+    }
     return out
 
 

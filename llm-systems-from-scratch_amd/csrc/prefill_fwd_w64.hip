@@ -113,6 +113,7 @@ constexpr int kWBN = 64;             // keys per LDS tile
 constexpr int kWD = 128;
 constexpr int kWRow = kWD * 2;       // bytes per LDS row
 constexpr int kWTile = kWBN * kWRow; // bytes per K (or V) tile
+constexpr int kWMaxSeqs = 4096;      // sequences of a packed batch
 
 // Direct-to-LDS load of 16 bytes per lane (see dma_to_lds_16 in common.hpp).  This variant writes m0 inside the
 // statement: the assembly loop of this kernel writes m0 too, behind the compiler's back, so nothing here may rely on
@@ -142,7 +143,7 @@ __device__ __forceinline__ void load_bounds(const int32_t* cu_q, const int32_t* 
 }
 
 template <bool CAUSAL>
-__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int n_logical, int tiles_per_id) {
+__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int tiles_per_unit) {
     constexpr int D = kWD, NS = D / 16, NDT = D / 32, CPR = D / 8;
     constexpr float kBias = 32.0f;             // the largest weight sits at 2^-kBias when a reference is set
     constexpr float kUnderflow = 0x1p-92f;     // a row sum below this may have lost terms (see the file header)
@@ -152,6 +153,8 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     __shared__ __attribute__((aligned(1024))) unsigned char kv_lds[4 * kWTile];
     // the four wavefronts' 64 query rows each, laid out like a K tile
     __shared__ __attribute__((aligned(1024))) unsigned char q_lds[kWWaves * 64 * kWRow];
+    // the number of query tiles of every sequence of a packed batch (see the jobs below)
+    __shared__ int nq_lds[kWMaxSeqs];
     unsigned char* const k_lds = kv_lds;
     unsigned char* const v_lds = kv_lds + 2 * kWTile;
 
@@ -161,12 +164,20 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const int n = lane & 31;          // query column inside a block / key row of K / d row of V^T
     const int kg = lane >> 5;
 
-    // ---- jobs: a workgroup works through query tiles, one "job" each.  Logical id = (batch, head, tile pair); a
-    // pair is the query tiles (nq-1-i, i) of a sequence, so that causal work is the same for every id.  The ids are
-    // dealt so that the workgroups resident on one XCD (workgroup ids are dealt round-robin to the 8 XCDs) walk
-    // through one contiguous range of ids together and stream the same K/V through that XCD's L2.
-    // (tiles_per_id == 1: an id is a single query tile nq-1-i, and p.n_pairs counts tiles.  The launch code chooses
-    // that when every query tile can have a compute unit of its own.) ----
+    // ---- jobs: a workgroup works through query tiles, one "job" each.  The unit that is dealt to workgroups is a
+    // PAIR of query tiles (n-1-i, i) of one (sequence, head [, share of the keys]), n the number of query tiles of
+    // the sequence: under a causal mask every pair of a sequence then costs the same.  (tiles_per_unit == 1: single
+    // tiles.  The launch code chooses that when every tile can have a compute unit of its own.)
+    // All units of the launch form one list: sequences by their number of query tiles, the longest class first (so
+    // the list is sorted by cost); inside a class by sequence, inside a sequence by share of the keys, K/V head,
+    // pair, query head of that K/V head.  The list is dealt in rounds of one unit per workgroup, every other round in
+    // reverse order: each workgroup gets the same number of units from every part of the list, whatever the lengths
+    // of the sequences are.  Nothing of this lives in memory: a workgroup walks down the classes and counts the
+    // sequences of a class (their numbers of query tiles sit in LDS, 64 per instruction), and finds the sequence of
+    // its unit by the same count.
+    // The 32 workgroups of an XCD (workgroup ids are dealt round-robin to the 8 XCDs) take 32 neighbours of the list:
+    // pairs and query heads of one K/V head, as far as the numbers allow, which stream the same K/V tiles through
+    // that XCD's L2 at the same time. ----
     struct Job {
         const __bf16 *qb, *kb, *vb;
         __bf16* ob;
@@ -174,30 +185,77 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         int sq, sk, q0;
         int split;                       // which share of the query tile's K/V tiles (0 when the keys are not split)
     };
-    // Split keys (p.n_split > 1): an id is (batch, head, tile pair, share); a job works on its share of the K/V tiles and
-    // writes, instead of output rows, a normalised fp32 partial row and its log-sum-exp per query, which a second
-    // kernel merges.  `ob` and `lb` of such a job point at row 0 of its (share, head, sequence) in the two partial buffers.
+    // Split keys (p.n_split > 1): a job works on its share of the K/V tiles and writes, instead of output rows, a
+    // normalised fp32 partial row and its log-sum-exp per query, which a second kernel merges.  `ob` and `lb` of such
+    // a job point at row 0 of its (share, head, sequence) in the two partial buffers.
     const int n_split = p.n_split > 1 ? p.n_split : 1;
     // head and row strides fit 32 bits (the host checks), so an address takes two scalar multiplications
     const int qs2 = (int)p.qs[2], ks2 = (int)p.ks[2], vs2 = (int)p.vs[2], os2 = (int)p.os[2];
-    const int n_pairs = p.n_pairs, Hq = p.Hq;
-    // the ids of this workgroup: id, id + id_step, ... below id_end
+    const int Hq = p.Hq, Hkv = p.Hkv, inner = Hq * n_split;
+    const int group = Hq / Hkv, group_shift = (group & (group - 1)) == 0 ? __builtin_ctz(group) : -1;
+    const bool packed = p.cu_q != nullptr;
+    const int n_seq_chunks = (p.B + 63) / 64;
+    // numbers of query tiles per sequence (packed layout; zero past the last sequence) and the first class
+    int cls;
+    if (packed) {
+        for (int b = tid; b < 64 * n_seq_chunks; b += kWWaves * 64)
+            nq_lds[b] = b < p.B ? (p.cu_q[b + 1] - p.cu_q[b] + kWBM - 1) / kWBM : 0;
+        __syncthreads();
+    }
+    // the largest number of query tiles below `limit` that a sequence has (0: none)
+    auto class_below = [&](int limit) -> int {
+        if (!packed) return 0;
+        int most = 0;
+        for (int m = 0; m < n_seq_chunks; ++m) {
+            const int v = nq_lds[64 * m + lane];
+            most = max(most, v < limit ? v : 0);
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) most = max(most, __shfl_xor(most, d, 64));
+        return __builtin_amdgcn_readfirstlane(most);
+    };
+    // number of sequences with exactly `tiles` query tiles, and the `rank`-th of them
+    auto seqs_of = [&](int tiles) -> int {
+        if (!packed) return p.B;
+        int c = 0;
+        for (int m = 0; m < n_seq_chunks; ++m)
+            c += __builtin_popcountll(__builtin_amdgcn_ballot_w64(nq_lds[64 * m + lane] == tiles));
+        return __builtin_amdgcn_readfirstlane(c);
+    };
+    auto seq_of = [&](int tiles, int rank) -> int {
+        if (!packed) return rank;
+        for (int m = 0; m < n_seq_chunks; ++m) {
+            const uint64_t mask = __builtin_amdgcn_ballot_w64(nq_lds[64 * m + lane] == tiles);
+            const int c = __builtin_popcountll(mask);
+            if (rank < c) {                   // position of set bit number `rank`: halving by counts
+                int pos = 0;
+#pragma unroll
+                for (int w = 32; w >= 1; w >>= 1) {
+                    const int below = __builtin_popcountll((mask >> pos) & ((1ull << w) - 1));
+                    const bool skip = rank >= below;
+                    rank -= skip ? below : 0;
+                    pos += skip ? w : 0;
+                }
+                return 64 * m + pos;
+            }
+            rank -= c;
+        }
+        return 0;
+    };
+    auto units_of = [&](int tiles) { return tiles_per_unit == 2 ? (tiles + 1) / 2 : tiles; };
+    cls = packed ? class_below(0x7fffffff) : (p.Sq + kWBM - 1) / kWBM;
+    // place of this workgroup in a round: neighbours of the list go to the workgroups of one XCD
     const int G = gridDim.x, bid = blockIdx.x;
-    const bool by_xcd = (n_logical % 8 == 0) && (G % 8 == 0);
-    const int id_step = by_xcd ? G / 8 : G;
-    const int id_end = by_xcd ? (bid % 8 + 1) * (n_logical / 8) : n_logical;
-    int id = by_xcd ? (bid % 8) * (n_logical / 8) + bid / 8 : bid;
-    // (pair, head, batch) of id and of id_step: an id advances digit by digit, with no division per job
-    int id_split = id % n_split, id_pair = (id / n_split) % n_pairs, id_h = (id / (n_split * n_pairs)) % Hq,
-        id_b = id / (n_split * n_pairs * Hq);
-    const int st_split = id_step % n_split, st_pair = (id_step / n_split) % n_pairs,
-              st_h = (id_step / (n_split * n_pairs)) % Hq, st_b = id_step / (n_split * n_pairs * Hq);
-    const int group = Hq / p.Hkv, group_shift = (group & (group - 1)) == 0 ? __builtin_ctz(group) : -1;
-    int job_k = -1, job_nq = 0, job_pair = 0, job_half = 1;      // position: "after the last query tile of id number job_k"
+    const int place = G % 8 == 0 ? (G / 8) * (bid % 8) + bid / 8 : bid;
+    int round = 0;
+    int64_t cls_first = 0;                    // position in the list of the first unit of the class
+    int per_seq = units_of(cls) * inner;      // units of one sequence of the class
+    int cls_units = cls > 0 ? seqs_of(cls) * per_seq : 0;
+    int job_tiles = 0, job_unit = 0, job_half = 1;      // the current job: tiles of its sequence, its unit, which tile of the pair
     // next_job(j, prev): the job after `prev` (whatever `prev` holds before the first).
-    // What only a new id needs -- tensor addresses, batch strides, the bounds arrays -- is read from the kernel
+    // What only a new unit needs -- tensor addresses, batch strides, the bounds arrays -- is read from the kernel
     // arguments (first argument, offset 0 of the segment) where it is needed, through an offset the compiler cannot
-    // trace: two scalar loads per id instead of three dozen scalar registers held, and spilled, for the whole kernel.
+    // trace: two scalar loads per unit instead of three dozen scalar registers held, and spilled, for the whole kernel.
     typedef const __attribute__((address_space(4))) PrefillParams* ParamsPtr;
     auto args = [&]() -> ParamsPtr {
         size_t off = 0;
@@ -205,67 +263,67 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         return (ParamsPtr)((const __attribute__((address_space(4))) char*)__builtin_amdgcn_kernarg_segment_ptr() + off);
     };
     auto next_job = [&](Job& j, const Job& prev) -> bool {
-        j = prev;                             // the sequence-level fields stay while the id stays
-        if (tiles_per_id == 2 && job_half == 0 && job_pair != job_nq - 1 - job_pair) {      // second query tile of the pair
+        j = prev;                             // the sequence-level fields stay while the unit stays
+        if (tiles_per_unit == 2 && job_half == 0 && job_unit != job_tiles - 1 - job_unit) {      // second query tile of the pair
             job_half = 1;
-            j.q0 = job_pair * kWBM;
+            j.q0 = job_unit * kWBM;
             return true;
         }
-        job_pair += n_pairs;                  // a further pair of the same sequence: only if it is longer than Sq_max promised
-        while (!(job_k >= 0 && tiles_per_id * job_pair < job_nq)) {
-            if (job_k >= 0) {
-                id += id_step;
-                id_split += st_split;
-                int carry = id_split >= n_split;
-                id_split -= carry ? n_split : 0;
-                id_pair += st_pair + carry;
-                carry = id_pair >= n_pairs;
-                id_pair -= carry ? n_pairs : 0;
-                id_h += st_h + carry;
-                carry = id_h >= Hq;
-                id_h -= carry ? Hq : 0;
-                id_b += st_b + carry;
-            }
-            ++job_k;
-            if (id >= id_end) return false;
-            const int h = id_h, b = id_b, hk = group_shift >= 0 ? h >> group_shift : h / group;
-            const ParamsPtr a = args();
-            const int qs1 = (int)a->qs[1], ks1 = (int)a->ks[1], vs1 = (int)a->vs[1], os1 = (int)a->os[1], ls1 = (int)a->ls[1];
-            if (a->cu_q) {
-                int q_start, q_end, k_start, k_end;
-                load_bounds(a->cu_q, a->cu_k, b, q_start, q_end, k_start, k_end);
-                j.sq = q_end - q_start;
-                j.sk = k_end - k_start;
-                j.qb = a->q + ((int64_t)q_start * qs2 + (int64_t)h * qs1);
-                j.kb = a->k + ((int64_t)k_start * ks2 + (int64_t)hk * ks1);
-                j.vb = a->v + ((int64_t)k_start * vs2 + (int64_t)hk * vs1);
-                j.ob = a->out + ((int64_t)q_start * os2 + (int64_t)h * os1);
-                j.lb = a->lse ? a->lse + (q_start + (int64_t)h * ls1) : nullptr;
-                if (n_split > 1) {
-                    const int64_t prow = ((int64_t)id_split * Hq + h) * a->part_rows + q_start;
-                    j.ob = reinterpret_cast<__bf16*>(a->part_o + prow * kWD);
-                    j.lb = a->part_lse + prow;
-                }
-            } else {
-                j.sq = a->Sq;
-                j.sk = a->Sk;
-                j.qb = a->q + ((int64_t)b * a->qs[0] + (int64_t)h * qs1);
-                j.kb = a->k + ((int64_t)b * a->ks[0] + (int64_t)hk * ks1);
-                j.vb = a->v + ((int64_t)b * a->vs[0] + (int64_t)hk * vs1);
-                j.ob = a->out + ((int64_t)b * a->os[0] + (int64_t)h * os1);
-                j.lb = a->lse ? a->lse + ((int64_t)b * a->ls[0] + (int64_t)h * ls1) : nullptr;
-                if (n_split > 1) {
-                    const int64_t prow = ((int64_t)id_split * Hq + h) * a->part_rows + (int64_t)b * a->Sq;
-                    j.ob = reinterpret_cast<__bf16*>(a->part_o + prow * kWD);
-                    j.lb = a->part_lse + prow;
-                }
-            }
-            j.split = id_split;
-            job_nq = (j.sq + kWBM - 1) / kWBM;
-            job_pair = id_pair;
+        const int64_t at = (int64_t)round * G + ((round & 1) ? G - 1 - place : place);
+        ++round;
+        while (cls > 0 && at >= cls_first + cls_units) {
+            cls_first += cls_units;
+            cls = class_below(cls);
+            per_seq = units_of(cls) * inner;
+            cls_units = cls > 0 ? seqs_of(cls) * per_seq : 0;
         }
+        if (cls <= 0) return false;
+        // (the compiler divides on the vector unit)
+        const int local = (int)(at - cls_first);
+        const int seq_rank = __builtin_amdgcn_readfirstlane(local / per_seq), rest = local - seq_rank * per_seq;
+        const int units = units_of(cls);
+        const int g = group_shift >= 0 ? rest & (group - 1) : rest % group;
+        const int above = group_shift >= 0 ? rest >> group_shift : __builtin_amdgcn_readfirstlane(rest / group);      // (share, K/V head, unit)
+        const int head_share = __builtin_amdgcn_readfirstlane(above / units), unit = above - head_share * units;
+        const int share = n_split > 1 ? __builtin_amdgcn_readfirstlane(head_share / Hkv) : 0, hk = head_share - share * Hkv;
+        const int h = hk * group + g;
+        const int b = __builtin_amdgcn_readfirstlane(seq_of(cls, seq_rank));
+        const ParamsPtr a = args();
+        const int qs1 = (int)a->qs[1], ks1 = (int)a->ks[1], vs1 = (int)a->vs[1], os1 = (int)a->os[1], ls1 = (int)a->ls[1];
+        if (a->cu_q) {
+            int q_start, q_end, k_start, k_end;
+            load_bounds(a->cu_q, a->cu_k, b, q_start, q_end, k_start, k_end);
+            j.sq = q_end - q_start;
+            j.sk = k_end - k_start;
+            j.qb = a->q + ((int64_t)q_start * qs2 + (int64_t)h * qs1);
+            j.kb = a->k + ((int64_t)k_start * ks2 + (int64_t)hk * ks1);
+            j.vb = a->v + ((int64_t)k_start * vs2 + (int64_t)hk * vs1);
+            j.ob = a->out + ((int64_t)q_start * os2 + (int64_t)h * os1);
+            j.lb = a->lse ? a->lse + (q_start + (int64_t)h * ls1) : nullptr;
+            if (n_split > 1) {
+                const int64_t prow = ((int64_t)share * Hq + h) * a->part_rows + q_start;
+                j.ob = reinterpret_cast<__bf16*>(a->part_o + prow * kWD);
+                j.lb = a->part_lse + prow;
+            }
+        } else {
+            j.sq = a->Sq;
+            j.sk = a->Sk;
+            j.qb = a->q + ((int64_t)b * a->qs[0] + (int64_t)h * qs1);
+            j.kb = a->k + ((int64_t)b * a->ks[0] + (int64_t)hk * ks1);
+            j.vb = a->v + ((int64_t)b * a->vs[0] + (int64_t)hk * vs1);
+            j.ob = a->out + ((int64_t)b * a->os[0] + (int64_t)h * os1);
+            j.lb = a->lse ? a->lse + ((int64_t)b * a->ls[0] + (int64_t)h * ls1) : nullptr;
+            if (n_split > 1) {
+                const int64_t prow = ((int64_t)share * Hq + h) * a->part_rows + (int64_t)b * a->Sq;
+                j.ob = reinterpret_cast<__bf16*>(a->part_o + prow * kWD);
+                j.lb = a->part_lse + prow;
+            }
+        }
+        j.split = share;
+        job_tiles = cls;
+        job_unit = unit;
         job_half = 0;
-        j.q0 = (job_nq - 1 - job_pair) * kWBM;
+        j.q0 = (cls - 1 - unit) * kWBM;
         return true;
     };
 
@@ -789,40 +847,40 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     }
 }
 
-// The kernel multiplies head and row strides as 32-bit numbers (batch strides stay 64-bit).
+// The kernel multiplies head and row strides as 32-bit numbers (batch strides stay 64-bit), and keeps one number per
+// sequence of a packed batch in LDS.
 bool prefill_w64_takes(const PrefillParams& p) {
     const int64_t strides[] = {p.qs[1], p.qs[2], p.ks[1], p.ks[2], p.vs[1], p.vs[2], p.os[1], p.os[2], p.lse ? p.ls[1] : 0};
     for (int64_t v : strides)
         if (v < 0 || v > 0x7fffffffLL) return false;
+    if (p.cu_q && p.B > kWMaxSeqs) return false;
     // a row offset inside a tile of 64 rows, in bytes, is a 32-bit number as well
     return p.qs[2] < (1 << 23) && p.ks[2] < (1 << 23) && p.vs[2] < (1 << 23) && p.os[2] < (1 << 23);
 }
 
 int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
-    // One resident workgroup per compute unit, each working through its share of the (batch, head, tile pair) ids.
+    // One resident workgroup per compute unit (fewer when there are fewer jobs), each working through its share of
+    // the (sequence, head, query tiles [, share of the keys]) units.  The kernel finds them from the sequence
+    // lengths themselves; Sq_max only bounds their number here.
     int dev = 0, n_cu = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return (int)e;
-    // Ids are pairs of query tiles (equal causal work per id) unless every single tile can have a compute unit of
-    // its own: then pairing would only leave half of those idle.
-    PrefillParams q = p;
-    int tiles_per_id = 2;
     const int n_split = p.n_split > 1 ? p.n_split : 1;
-    if ((int64_t)p.n_qtiles * p.Hq * p.B * n_split <= n_cu) {
-        tiles_per_id = 1;
-        q.n_pairs = p.n_qtiles;
-    }
-    if ((int64_t)q.n_pairs * q.Hq * q.B * n_split > 0x7fffffffLL) return (int)hipErrorInvalidValue;
-    const int n_logical = q.n_pairs * q.Hq * q.B * n_split;
-    if (n_logical <= 0) return 0;
-    int grid = n_logical < n_cu ? n_logical : n_cu;
-    if (n_logical % 8 == 0 && grid >= 8) grid -= grid % 8;          // whole number of workgroups per XCD
+    // Units are pairs of query tiles (equal causal work per unit of a sequence) unless every single tile can have a
+    // compute unit of its own: then pairing would only leave half of those idle.
+    const int64_t most_tiles = (int64_t)p.n_qtiles * p.Hq * p.B * n_split;
+    const int tiles_per_unit = most_tiles <= n_cu ? 1 : 2;
+    const int64_t most_units = tiles_per_unit == 1 ? most_tiles : (int64_t)((p.n_qtiles + 1) / 2) * p.Hq * p.B * n_split;
+    if (most_units <= 0) return 0;
+    if (most_units > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+    int grid = most_units < n_cu ? (int)most_units : n_cu;
+    if (grid >= 8) grid -= grid % 8;          // whole number of workgroups per XCD
     dim3 block(kWWaves * 64);
     if (p.mask_mode == MI355_MASK_CAUSAL)
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), dim3((unsigned)grid), block, 0, stream, q, n_logical, tiles_per_id);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit);
     else
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), dim3((unsigned)grid), block, 0, stream, q, n_logical, tiles_per_id);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit);
     return (int)hipGetLastError();
 }
 

@@ -465,16 +465,15 @@ def test_prefill_head_dim_128_packed_sequences_of_drawn_lengths(ops, seed):
 
 
 @pytest.mark.parametrize("seed", [0, 1])
-def test_prefill_head_dim_128_paired_query_tiles_on_ragged_sequences(ops, seed):
-    """Enough (sequence, head, query tile) triples that the persistent kernel deals PAIRS of query tiles to its
-    workgroups (with fewer triples than compute units it deals single tiles, which is what the small shapes of the
-    other tests get): ragged packed sequences, 32 query heads on 8 kv heads, causal and not, one promised maximum that
-    is too small."""
+def test_prefill_head_dim_128_more_jobs_than_compute_units_on_ragged_sequences(ops, seed):
+    """More (sequence, head, query tile) jobs than compute units, so that the persistent kernel deals several rounds
+    of its job list, forwards and backwards (the small shapes of the other tests fit in one round): ragged packed
+    sequences, 32 query heads on 8 kv heads, causal and not, one promised maximum that is too small."""
     g = torch.Generator().manual_seed(4000 + seed)
     Hq, Hkv, D = 32, 8, 128
     lens = [int(x) for x in torch.randint(520, 1000, (3,), generator=g)]        # 3 or 4 query tiles each: > 256 triples
     lens[seed % 3] = 1 + int(torch.randint(0, 255, (1,), generator=g))
-    print(f"case: paired query tiles seed={seed} lens={lens}", flush=True)
+    print(f"case: several rounds of jobs seed={seed} lens={lens}", flush=True)
     T = sum(lens)
     cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
     q, k, v = rnd(T, Hq, D, seed=4100 + seed), rnd(T, Hkv, D, seed=4200 + seed), rnd(T, Hkv, D, seed=4300 + seed)
@@ -482,13 +481,58 @@ def test_prefill_head_dim_128_paired_query_tiles_on_ragged_sequences(ops, seed):
         ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=causal)
         got = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens),
                                             causal=causal, kv_splits=1)
-        check(got, ref, what=f"paired query tiles, causal={causal}")
+        check(got, ref, what=f"several rounds of jobs, causal={causal}")
     ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True)
     short = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), 600, 600, causal=True, kv_splits=1)
-    check(short, ref, what="paired query tiles, promised maximum too small")
+    check(short, ref, what="several rounds of jobs, promised maximum too small")
     shared = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens),
                                            causal=True, kv_splits=3)
-    check(shared, ref, what="paired query tiles, keys split 3 ways")
+    check(shared, ref, what="several rounds of jobs, keys split 3 ways")
+
+
+@pytest.mark.parametrize("n_seq", [70, 150])
+def test_prefill_head_dim_128_many_packed_sequences_of_very_different_lengths(ops, n_seq):
+    """The persistent kernel orders its jobs by query tile index and finds the sequences that reach an index by
+    counting over all sequences, 64 at a time: more than 64 sequences, most of them short or empty and a few long
+    ones at drawn places, so that every level of the job list has its own set of sequences; causal and not, keys
+    whole and split."""
+    g = torch.Generator().manual_seed(5000 + n_seq)
+    Hq, Hkv, D = 4, 2, 128
+    lens = [int(x) for x in torch.randint(0, 40, (n_seq,), generator=g)]
+    for _ in range(6):
+        lens[int(torch.randint(0, n_seq, (1,), generator=g))] = int(torch.randint(200, 1300, (1,), generator=g))
+    lens[n_seq - 1] = 700                     # the last sequence reaches the third level
+    print(f"case: many packed sequences n_seq={n_seq} longest={max(lens)} total={sum(lens)}", flush=True)
+    T = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q, k, v = rnd(T, Hq, D, seed=5100 + n_seq), rnd(T, Hkv, D, seed=5200 + n_seq), rnd(T, Hkv, D, seed=5300 + n_seq)
+    for causal in (True, False):
+        ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=causal)
+        for splits in (1, 2):
+            got = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), max(lens), max(lens),
+                                                causal=causal, kv_splits=splits)
+            check(got, ref, what=f"{n_seq} packed sequences, causal={causal}, keys split {splits} ways")
+
+
+def test_prefill_head_dim_128_more_packed_sequences_than_the_64_query_kernel_keeps_counts_for(ops):
+    """The 64-query kernel keeps one number per sequence in LDS, 4096 at most; a packed batch of more sequences goes
+    to the other kernel.  4100 sequences of one to three tokens."""
+    n_seq, Hq, Hkv, D = 4100, 2, 1, 128
+    g = torch.Generator().manual_seed(5500)
+    lens = [int(x) for x in torch.randint(1, 4, (n_seq,), generator=g)]
+    print(f"case: {n_seq} packed sequences total={sum(lens)}", flush=True)
+    T = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q, k, v = rnd(T, Hq, D, seed=5501), rnd(T, Hkv, D, seed=5502), rnd(T, Hkv, D, seed=5503)
+    ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True)
+    got = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu.cuda(), cu.cuda(), 3, 3, causal=True, kv_splits=1)
+    check(got, ref, what="4100 packed sequences")
+    # the same tokens as 4096 sequences (the last one takes what is left): the 64-query kernel at its limit
+    cu2 = torch.cat([cu[:4096], cu[-1:]])
+    ref2 = orc.varlen_prefill_reference(q, k, v, cu2, cu2, causal=True)
+    longest = int((cu2[1:] - cu2[:-1]).max())
+    got2 = ops.flash_attn_varlen_prefill(q.cuda(), k.cuda(), v.cuda(), cu2.cuda(), cu2.cuda(), longest, longest, causal=True, kv_splits=1)
+    check(got2, ref2, what="4096 packed sequences")
 
 
 def test_prefill_head_dim_128_rows_too_far_apart_for_the_64_query_kernel(ops):
