@@ -134,6 +134,19 @@ __device__ __forceinline__ void dma_to_lds_16(const void* gbase, uint32_t voff, 
                  : "v"(voff), "s"(gbase), "{m0}"(lds_addr)
                  : "memory");
 }
+// Logical id of workgroup `bid` of a one-dimensional grid whose ids come in chunks of `chunk` that read the same
+// tensor rows (e.g. the query tiles and query heads of one K/V head).  Workgroup ids are dealt round-robin to the 8
+// XCDs, each with an L2 of its own; the XCDs take whole chunks in turn, so the workgroups of a chunk are resident on
+// one XCD at about the same time, and what one sequence brings is spread over all XCDs however long it is.
+// (Ids past the last whole round of eight chunks stay as they are.)
+__device__ __forceinline__ int xcd_chunked_id(int bid, int n_wg, int chunk) {
+    const int whole = n_wg / (8 * chunk) * (8 * chunk);
+    const int xcd = bid % 8, k = bid / 8, turn = k / chunk;
+    const int id = (turn * 8 + xcd) * chunk + (k - turn * chunk);
+    // (the compiler divides on the vector unit; the result is the same in every lane)
+    return __builtin_amdgcn_readfirstlane(bid >= whole ? bid : id);
+}
+
 __device__ __forceinline__ uint32_t lds_address(const void* lds_ptr) {
     return (uint32_t)(uintptr_t)(const MI355_LDS void*)lds_ptr;
 }

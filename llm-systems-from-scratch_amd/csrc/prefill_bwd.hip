@@ -111,12 +111,10 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
     // Workgroup ids are dealt round-robin to the 8 XCDs (private L2s) and, in order, to their shader
     // engines: workgroups must carry EQUAL work (a periodic heavy/light pattern starves the engines that
     // always draw the light ones), and the workgroups that stream the same K/V should share an XCD.  So a
-    // workgroup takes the query-tile PAIR (nq-1-i, i), and the id is remapped so that every XCD works
-    // through a contiguous range of (pair, query head, batch).
-    const int n_wg = gridDim.x;
-    int lid = blockIdx.x;
-    if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
+    // workgroup takes the query-tile PAIR (nq-1-i, i), and the pairs and query heads of one kv head -- a chunk
+    // of the logical order (pair, query head, batch) -- run on one XCD.
     const int n_pairs = (p.n_qtiles + 1) / 2;
+    const int lid = xcd_chunked_id(blockIdx.x, gridDim.x, n_pairs * (p.Hq / p.Hkv));
     const int pair = lid % n_pairs;
     const int h = (lid / n_pairs) % p.Hq;
     const int b = lid / (n_pairs * p.Hq);
@@ -343,10 +341,9 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
     __shared__ __attribute__((aligned(16))) float lse_lds2[2 * kBwRows];
     __shared__ __attribute__((aligned(16))) float delta_lds2[2 * kBwRows];
 
-    const int n_wg = gridDim.x;
-    int lid = blockIdx.x;
-    if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
+    // (the key-tile pairs of one (batch, kv head), which stream the same Q and dO tiles, run on one XCD)
     const int n_pairs = (p.n_ktiles + 1) / 2;
+    const int lid = xcd_chunked_id(blockIdx.x, gridDim.x, n_pairs);
     const int pair = lid % n_pairs;
     const int hk = (lid / n_pairs) % p.Hkv;
     const int b = lid / (n_pairs * p.Hkv);

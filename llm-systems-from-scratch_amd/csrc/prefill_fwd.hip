@@ -58,13 +58,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     constexpr int kORow = D * 2 + 16;
     __shared__ __attribute__((aligned(16))) unsigned char o_lds[kPfWaves * 32 * kORow];
 
-    // Workgroup ids are dealt round-robin to the 8 XCDs, each with a private L2.  The id is
-    // remapped so that every XCD works through a contiguous range of the logical order
-    // (pair fastest, then the query heads of one kv head, then kv head, then batch): the
-    // workgroups that stream the same K/V are then resident on the same XCD at the same time.
-    const int n_wg = gridDim.x;
-    int lid = blockIdx.x;
-    if (n_wg % 8 == 0) lid = (lid % 8) * (n_wg / 8) + lid / 8;
+    // Logical order: pair fastest, then the query heads of one kv head, then kv head, then batch.  The workgroups
+    // that stream the same K/V -- the pairs and query heads of one kv head -- form a chunk of that order and run on
+    // one XCD.
+    const int lid = xcd_chunked_id(blockIdx.x, gridDim.x, p.n_pairs * (p.Hq / p.Hkv));
     const int split = blockIdx.y;                    // share of the keys this workgroup serves (gridDim.y = n_split)
     const int pair0 = lid % p.n_pairs;
     const int h = (lid / p.n_pairs) % p.Hq;
