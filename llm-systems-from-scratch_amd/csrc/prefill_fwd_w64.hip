@@ -164,20 +164,24 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const int n = lane & 31;          // query column inside a block / key row of K / d row of V^T
     const int kg = lane >> 5;
 
-    // ---- jobs: a workgroup works through query tiles, one "job" each.  The unit that is dealt to workgroups is a
-    // PAIR of query tiles (n-1-i, i) of one (sequence, head [, share of the keys]), n the number of query tiles of
-    // the sequence: under a causal mask every pair of a sequence then costs the same.  (tiles_per_unit == 1: single
-    // tiles.  The launch code chooses that when every tile can have a compute unit of its own.)
-    // All units of the launch form one list: sequences by their number of query tiles, the longest class first (so
-    // the list is sorted by cost); inside a class by sequence, inside a sequence by share of the keys, K/V head,
-    // pair, query head of that K/V head.  The list is dealt in rounds of one unit per workgroup, every other round in
-    // reverse order: each workgroup gets the same number of units from every part of the list, whatever the lengths
-    // of the sequences are.  Nothing of this lives in memory: a workgroup walks down the classes and counts the
-    // sequences of a class (their numbers of query tiles sit in LDS, 64 per instruction), and finds the sequence of
-    // its unit by the same count.
-    // The 32 workgroups of an XCD (workgroup ids are dealt round-robin to the 8 XCDs) take 32 neighbours of the list:
-    // pairs and query heads of one K/V head, as far as the numbers allow, which stream the same K/V tiles through
-    // that XCD's L2 at the same time. ----
+    // ---- jobs: a workgroup works through query tiles, one "job" each.  What is dealt to workgroups are UNITS of one
+    // (sequence, head [, share of the keys]), all units of the launch forming one list sorted by cost, in one of two
+    // ways that the launch code chooses between:
+    //   pairs (tiles_per_unit == 2): a unit is the PAIR of query tiles (n-1-i, i), n the number of query tiles of the
+    //     sequence: under a causal mask every pair of a sequence costs the same.  The list: sequences by their number
+    //     of query tiles, the longest class first; inside a class by sequence; inside a sequence by share of the keys,
+    //     K/V head, pair, query head of that K/V head.  Neighbours in the list read the same K/V.
+    //   single tiles (tiles_per_unit == 1): the list goes by tile index from the highest down -- "class c" is then
+    //     every sequence with at least c query tiles, and its unit the tile c-1 -- inside a class by sequence, share,
+    //     K/V head, query head.  Finer units: this is for launches of few rounds, where a round of pairs more or
+    //     less for some workgroups would be felt.
+    // The list is dealt in rounds of one unit per workgroup, every other round in reverse order: each workgroup gets
+    // the same number of units from every part of the list, whatever the lengths of the sequences are.  Nothing of
+    // this lives in memory: a workgroup walks down the classes and counts the sequences of a class (their numbers of
+    // query tiles sit in LDS, 64 per instruction), and finds the sequence of its unit by the same count.
+    // In pairs mode the 32 workgroups of an XCD (workgroup ids are dealt round-robin to the 8 XCDs) take 32 neighbours
+    // of the list: the pairs and query heads of one K/V head, as far as the numbers allow, which stream the same K/V
+    // tiles through that XCD's L2 at the same time. ----
     struct Job {
         const __bf16 *qb, *kb, *vb;
         __bf16* ob;
@@ -202,32 +206,37 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             nq_lds[b] = b < p.B ? (p.cu_q[b + 1] - p.cu_q[b] + kWBM - 1) / kWBM : 0;
         __syncthreads();
     }
-    // the largest number of query tiles below `limit` that a sequence has (0: none)
-    auto class_below = [&](int limit) -> int {
+    const bool pairs = tiles_per_unit == 2;
+    // the class after class `c` (0: none): the largest number of query tiles below c that a sequence has, or c - 1
+    auto class_below = [&](int c) -> int {
+        if (!pairs) return c - 1;
         if (!packed) return 0;
         int most = 0;
         for (int m = 0; m < n_seq_chunks; ++m) {
             const int v = nq_lds[64 * m + lane];
-            most = max(most, v < limit ? v : 0);
+            most = max(most, v < c ? v : 0);
         }
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) most = max(most, __shfl_xor(most, d, 64));
         return __builtin_amdgcn_readfirstlane(most);
     };
-    // number of sequences with exactly `tiles` query tiles, and the `rank`-th of them
-    auto seqs_of = [&](int tiles) -> int {
-        if (!packed) return p.B;
-        int c = 0;
-        for (int m = 0; m < n_seq_chunks; ++m)
-            c += __builtin_popcountll(__builtin_amdgcn_ballot_w64(nq_lds[64 * m + lane] == tiles));
-        return __builtin_amdgcn_readfirstlane(c);
+    // the sequences of class c, 64 at a time as a bit mask; their number; the `rank`-th of them
+    auto members = [&](int c, int m) -> uint64_t {
+        const int v = nq_lds[64 * m + lane];
+        return __builtin_amdgcn_ballot_w64(pairs ? v == c : v >= c);
     };
-    auto seq_of = [&](int tiles, int rank) -> int {
+    auto seqs_of = [&](int c) -> int {
+        if (!packed) return p.B;
+        int count = 0;
+        for (int m = 0; m < n_seq_chunks; ++m) count += __builtin_popcountll(members(c, m));
+        return __builtin_amdgcn_readfirstlane(count);
+    };
+    auto seq_of = [&](int c, int rank) -> int {
         if (!packed) return rank;
         for (int m = 0; m < n_seq_chunks; ++m) {
-            const uint64_t mask = __builtin_amdgcn_ballot_w64(nq_lds[64 * m + lane] == tiles);
-            const int c = __builtin_popcountll(mask);
-            if (rank < c) {                   // position of set bit number `rank`: halving by counts
+            const uint64_t mask = members(c, m);
+            const int count = __builtin_popcountll(mask);
+            if (rank < count) {               // position of set bit number `rank`: halving by counts
                 int pos = 0;
 #pragma unroll
                 for (int w = 32; w >= 1; w >>= 1) {
@@ -238,15 +247,31 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 }
                 return 64 * m + pos;
             }
-            rank -= c;
+            rank -= count;
         }
         return 0;
     };
-    auto units_of = [&](int tiles) { return tiles_per_unit == 2 ? (tiles + 1) / 2 : tiles; };
-    cls = packed ? class_below(0x7fffffff) : (p.Sq + kWBM - 1) / kWBM;
-    // place of this workgroup in a round: neighbours of the list go to the workgroups of one XCD
+    auto units_of = [&](int c) { return pairs ? (c + 1) / 2 : 1; };      // units of one (sequence, head, share) in class c
+    if (packed) {                             // the first class: the largest number of query tiles
+        int most = 0;
+        for (int m = 0; m < n_seq_chunks; ++m) most = max(most, nq_lds[64 * m + lane]);
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) most = max(most, __shfl_xor(most, d, 64));
+        cls = __builtin_amdgcn_readfirstlane(most);
+    } else {
+        cls = (p.Sq + kWBM - 1) / kWBM;
+    }
+    // place of this workgroup in a round: neighbours of the list go to the workgroups of one XCD -- in pairs mode
+    // as many as the XCD has workgroups; in single-tile mode, where neighbours cost the same, only the query heads
+    // of one K/V head, so that the dearest units of the launch are spread over all XCDs
     const int G = gridDim.x, bid = blockIdx.x;
-    const int place = G % 8 == 0 ? (G / 8) * (bid % 8) + bid / 8 : bid;
+    int place = bid;
+    if (G % 8 == 0) {
+        const int xcd = bid % 8, local = bid / 8;
+        const int chunk = min(group & -group, 32);
+        if (pairs) place = (G / 8) * xcd + local;
+        else if ((G / 8) % chunk == 0) place = chunk * ((local / chunk) * 8 + xcd) + local % chunk;
+    }
     int round = 0;
     int64_t cls_first = 0;                    // position in the list of the first unit of the class
     int per_seq = units_of(cls) * inner;      // units of one sequence of the class
@@ -264,7 +289,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     };
     auto next_job = [&](Job& j, const Job& prev) -> bool {
         j = prev;                             // the sequence-level fields stay while the unit stays
-        if (tiles_per_unit == 2 && job_half == 0 && job_unit != job_tiles - 1 - job_unit) {      // second query tile of the pair
+        if (pairs && job_half == 0 && job_unit != job_tiles - 1 - job_unit) {      // second query tile of the pair
             job_half = 1;
             j.q0 = job_unit * kWBM;
             return true;
@@ -867,11 +892,16 @@ int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
     if (e == hipSuccess) e = hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return (int)e;
     const int n_split = p.n_split > 1 ? p.n_split : 1;
-    // Units are pairs of query tiles (equal causal work per unit of a sequence) unless every single tile can have a
-    // compute unit of its own: then pairing would only leave half of those idle.
+    // Units are pairs of query tiles (equal causal work per unit of a sequence, neighbours that share K/V) unless
+    // pairs would leave compute units idle: when every single tile can have a compute unit of its own, or when the
+    // pairs make few rounds and the last of them is far from full (judged for sequences of Sq_max rows; then single
+    // tiles, dealt by cost, fill the gap better than half as many pairs).
     const int64_t most_tiles = (int64_t)p.n_qtiles * p.Hq * p.B * n_split;
-    const int tiles_per_unit = most_tiles <= n_cu ? 1 : 2;
-    const int64_t most_units = tiles_per_unit == 1 ? most_tiles : (int64_t)((p.n_qtiles + 1) / 2) * p.Hq * p.B * n_split;
+    const int64_t most_pairs = (int64_t)((p.n_qtiles + 1) / 2) * p.Hq * p.B * n_split;
+    const int64_t rounds = (most_pairs + n_cu - 1) / n_cu;
+    const bool singles = most_tiles <= n_cu || (rounds < 8 && most_pairs * 100 < rounds * n_cu * 97);
+    const int tiles_per_unit = singles ? 1 : 2;
+    const int64_t most_units = singles ? most_tiles : most_pairs;
     if (most_units <= 0) return 0;
     if (most_units > 0x7fffffffLL) return (int)hipErrorInvalidValue;
     int grid = most_units < n_cu ? (int)most_units : n_cu;

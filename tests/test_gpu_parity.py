@@ -467,8 +467,9 @@ def test_prefill_head_dim_128_packed_sequences_of_drawn_lengths(ops, seed):
 @pytest.mark.parametrize("seed", [0, 1])
 def test_prefill_head_dim_128_more_jobs_than_compute_units_on_ragged_sequences(ops, seed):
     """More (sequence, head, query tile) jobs than compute units, so that the persistent kernel deals several rounds
-    of its job list, forwards and backwards (the small shapes of the other tests fit in one round): ragged packed
-    sequences, 32 query heads on 8 kv heads, causal and not, one promised maximum that is too small."""
+    of its job list, forwards and backwards (the small shapes of the other tests fit in one round; here the list is
+    made of single tiles by tile index): ragged packed sequences, 32 query heads on 8 kv heads, causal and not, one
+    promised maximum that is too small."""
     g = torch.Generator().manual_seed(4000 + seed)
     Hq, Hkv, D = 32, 8, 128
     lens = [int(x) for x in torch.randint(520, 1000, (3,), generator=g)]        # 3 or 4 query tiles each: > 256 triples
@@ -494,8 +495,9 @@ def test_prefill_head_dim_128_more_jobs_than_compute_units_on_ragged_sequences(o
 def test_prefill_head_dim_128_many_packed_sequences_of_very_different_lengths(ops, n_seq):
     """The persistent kernel orders its jobs by query tile index and finds the sequences that reach an index by
     counting over all sequences, 64 at a time: more than 64 sequences, most of them short or empty and a few long
-    ones at drawn places, so that every level of the job list has its own set of sequences; causal and not, keys
-    whole and split."""
+    ones at drawn places, so that every class of the job list has its own set of sequences; causal and not, keys
+    whole and split.  With 150 sequences the list is made of tile pairs (eight rounds and more on 256 compute units),
+    with 70 of single tiles by tile index (four rounds, the last far from full)."""
     g = torch.Generator().manual_seed(5000 + n_seq)
     Hq, Hkv, D = 4, 2, 128
     lens = [int(x) for x in torch.randint(0, 40, (n_seq,), generator=g)]
