@@ -33,8 +33,9 @@
 // AGPRs once per job; the output rows are normalised 32 at a time and leave whole through the wavefront's own shares
 // of the second K and V buffers, which nobody needs between the last tile of a job and the first boundary of the
 // next.  The next job is worked out at the top of the current one, and its first requests (K[0], query rows, V[0],
-// then K[1]) go out between the pieces of output work.  No ordinary vector load sits in the job loop, so the only
-// waits on memory are the ones written here (the compiler would add s_waitcnt vmcnt(0), which also waits for every
+// then K[1]) go out between the pieces of output work -- the query rows earlier still where a causal mask leaves
+// wavefronts without work in the last tiles of a job: they request them then, also for the others.  No ordinary
+// vector load sits in the job loop, so the only waits on memory are the ones written here (the compiler would add s_waitcnt vmcnt(0), which also waits for every
 // request in flight, in front of the first use of a loaded register).
 //
 // Hand-over protocol between the two (and between tiles), one "boundary" per tile t and wavefront: K[t] and V[t]
@@ -444,15 +445,17 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     // rows each, swizzled like a K tile (load i covers rows 4i + lane/16, and swz of that row is ((lane/16) << 2) |
     // (i & 3)); a row past the end of the sequence re-reads the last row (finite; nothing of it is ever stored) ----
     const uint32_t q_dst = __builtin_amdgcn_readfirstlane(lds_address(q_lds + wave * (64 * kWRow)));
-    // (loads 4 * part .. 4 * part + 3: rows 16 * part .. 16 * part + 15)
-    auto issue_q = [&](const Job& jb, int part) {
-        const int qw0 = jb.q0 + 64 * wave;
+    // (loads 4 * part .. 4 * part + 3: rows 16 * part .. 16 * part + 15 of wavefront `to`; a wavefront may request
+    // another one's rows, see the early requests below)
+    auto issue_q = [&](const Job& jb, int to, int part) {
+        const int qw0 = jb.q0 + 64 * to;
         const uint32_t row_bytes = (uint32_t)qs2 * 2u;
+        const uint32_t dst = q_dst + (uint32_t)((to - wave) * (64 * kWRow) + 4 * part * 1024);
         if (qw0 + 64 <= jb.sq) {
             const unsigned char* base = reinterpret_cast<const unsigned char*>(jb.qb + (int64_t)(qw0 + 16 * part) * qs2);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                dma_to_lds_16_m0(base + (size_t)(4 * j) * row_bytes, (uint32_t)ld_q * row_bytes + ((ld_c0 ^ j) << 4), q_dst + (4 * part + j) * 1024);
+                dma_to_lds_16_m0(base + (size_t)(4 * j) * row_bytes, (uint32_t)ld_q * row_bytes + ((ld_c0 ^ j) << 4), dst + j * 1024);
         } else {
             // (the empty statement keeps the arithmetic of this rare path inside the branch)
             int last = jb.sq - 1;
@@ -462,7 +465,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t row = (uint32_t)(min(qw0 + 16 * part + 4 * j + ld_q, last) - first);
-                dma_to_lds_16_m0(base, row * row_bytes + (uint32_t)((ld_c0 ^ j) << 4), q_dst + (4 * part + j) * 1024);
+                dma_to_lds_16_m0(base, row * row_bytes + (uint32_t)((ld_c0 ^ j) << 4), dst + j * 1024);
             }
         }
     };
@@ -485,13 +488,15 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     // once the output rows have left its buffer.  Six groups of four requests and a seventh: in the epilogue of a job
     // they go out one group at a time between pieces of vector work, so that the wavefront does not sit behind a
     // full request queue (the four wavefronts all do this at the same time).
-    auto prefetch_group = [&](const Job& jb, int group) {
+    // (n_early: how many of the job's sixteen parts of query rows -- part p = rows 16 (p % 4) .. of wavefront
+    // 3 - p / 4 -- were requested already, while the job before was still in its tile loop: see the early requests)
+    auto prefetch_group = [&](const Job& jb, int group, int n_early) {
         int t0, t1;
         share_of(jb, t0, t1);
         if (group == 0) {
             if (t1 > t0) issue_k(jb, t0, t0 & 1);
         } else if (group <= 4) {
-            issue_q(jb, group - 1);
+            if (4 * (3 - wave) + group - 1 >= n_early) issue_q(jb, wave, group - 1);
         } else if (group == 5) {
             if (t1 > t0) issue_v(jb, t0, t0 & 1);
         } else {
@@ -526,7 +531,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     bool have = next_job(cur, cur);
     if (have) {
 #pragma unroll
-        for (int group = 0; group < 7; ++group) prefetch_group(cur, group);
+        for (int group = 0; group < 7; ++group) prefetch_group(cur, group, 0);
     }
     int prev_stores = 0;       // output row stores of the job before `cur` that are younger than the requests for `cur`
     while (have) {
@@ -552,6 +557,29 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         const int share_tiles = n_tiles - t_first;
         // the job after this one (scalar work, done while the first tile is still landing)
         const bool have_next = next_job(nxt, cur);
+        // Early requests.  Under a causal mask the wavefronts with the upper rows of the query tile have nothing to
+        // compute in its last tiles ("hidden" steps: they only take part in the hand-over, in ordinary code) while
+        // the one with the lowest rows sets the pace.  In such a step a wavefront requests query rows of the NEXT
+        // job -- anybody's: the place in LDS is free once every wavefront has its fragments in registers, which the
+        // first hand-over of the job guarantees -- three parts per step, in an order every wavefront can work out
+        // (step by step, wavefront by wavefront; part p = rows 16 (p % 4) .. of wavefront 3 - p / 4, so the rows of
+        // the wavefront that is busiest at the end of a job go first).  What is left goes out after the tile loop.
+        const auto first_hidden_of = [&](int q_tile0, int off, int first, int tiles, int w) {
+            const int hidden = CAUSAL ? min(tiles, max(0, q_tile0 + 64 * w + 63 + off + kWBN) / kWBN) : tiles;
+            return max(hidden, first);
+        };
+        // number of (step, wavefront) slots in front of slot (tile, w)
+        const auto slots_before = [&](int q_tile0, int off, int first, int tiles, int tile, int w) {
+            int slots = 0;
+#pragma unroll
+            for (int other = 0; other < kWWaves; ++other) {
+                const int hidden = first_hidden_of(q_tile0, off, first, tiles, other);
+                slots += max(0, min(tile, tiles) - hidden) + (other < w && hidden <= tile ? 1 : 0);
+            }
+            return slots;
+        };
+        constexpr int kPartsPerSlot = 3;
+        const int n_early = have_next ? min(16, kPartsPerSlot * slots_before(q0, coff, t_first, n_tiles, n_tiles, 0)) : 0;
 
         // per column block: r_ref exponent reference in the log2 domain (-inf: none yet), nb = -r_ref - kBias
         float r_ref[2], nb[2], l_row[2];
@@ -562,7 +590,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         // values it needs that the compiler cannot trace back: what could be computed once per job would otherwise
         // be computed at the top of every job and wait in registers (spilled ones, mostly) for a tile that rarely comes.
         struct Fresh {
-            int sk, qw0, coff, n_tiles;
+            int sk, qw0, coff, n_tiles, q0, t_first, early;
         };
         // Scores of one 32-key half of a tile for one column block (reads K[tile]).
         auto scores = [&](auto c_c, int tile, int t) {
@@ -634,10 +662,11 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         };
         // a whole tile in ordinary code: scores from K[tile], boundary, everything else from V[tile]
         // (a tile past n_mask has nothing for this wavefront: it only takes part in the boundary)
-        auto step_cxx = [&](int tile) {
-            Fresh fr{sk, qw0, coff, n_tiles};
+        auto step_cxx = [&](int tile, bool early) {
+            Fresh fr{sk, qw0, coff, n_tiles, q0, t_first, early ? n_early : 0};
             int first_masked = n_plain, first_hidden = n_mask;
-            asm volatile("" : "+s"(fr.sk), "+s"(fr.qw0), "+s"(fr.coff), "+s"(fr.n_tiles), "+s"(first_masked), "+s"(first_hidden), "+s"(tile));
+            asm volatile("" : "+s"(fr.sk), "+s"(fr.qw0), "+s"(fr.coff), "+s"(fr.n_tiles), "+s"(first_masked), "+s"(first_hidden), "+s"(tile),
+                         "+s"(fr.q0), "+s"(fr.t_first), "+s"(fr.early));
             const bool visible = tile < first_hidden, masked = tile >= first_masked;
             constexpr std::integral_constant<int, 0> A{};
             constexpr std::integral_constant<int, 1> B{};
@@ -649,6 +678,16 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 sb1 = scores(B, tile, 1);
             }
             boundary(fr, tile);
+            if (!visible && fr.early > 0) {           // a hidden step of the first attempt: early requests
+                const int slot = slots_before(fr.q0, fr.coff, fr.t_first, fr.n_tiles, tile, wave);
+                Job jn = nxt;
+                asm volatile("" : "+s"(jn.qb), "+s"(jn.q0), "+s"(jn.sq));
+#pragma unroll 1
+                for (int i = 0; i < kPartsPerSlot; ++i) {
+                    const int part = kPartsPerSlot * slot + i;
+                    if (part < fr.early) issue_q(jn, 3 - part / 4, part % 4);
+                }
+            }
             if (visible) {
                 finish(fr, A, tile, 0, masked, sa0);
                 finish(fr, B, tile, 0, masked, sb0);
@@ -695,16 +734,17 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         // Wait for K[0] and the query rows.  Younger than the last request of those are the requests of V[0] and K[1]
         // and, the first time, the last output row stores of the job before this one.
         wait_all_but(young_dma + (preset ? prev_stores : 0));
+        __syncthreads();                      // everybody's share of K[0] and of the query rows is in
         if (preset) {                         // the query rows go to their registers
             uint32_t scratch;
             asm volatile(W64_QFRAGS : "=&v"(scratch) : "v"(q_rd0) : "memory", W64_CLOBBER_ACC);
         }
-        __syncthreads();                      // everybody's share of K[0] is in
         int tile = t_first;
-        const int n_loop = preset ? n_asm : 0;
+        // (the hand-scheduled loop ends where the wavefront's hidden steps begin: those run in ordinary code)
+        const int n_loop = preset ? min(n_asm, n_mask) : 0;
         while (tile < n_tiles) {
             if (tile >= n_loop) {
-                step_cxx(tile);
+                step_cxx(tile, preset);
                 ++tile;
                 continue;
             }
@@ -796,7 +836,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                             *reinterpret_cast<f32x4*>(po + 32 * dt + 8 * g) =
                                 f32x4{x[4 * g] * inv_p, x[4 * g + 1] * inv_p, x[4 * g + 2] * inv_p, x[4 * g + 3] * inv_p};
                     }
-                    if (have_next && 4 * c + dt < 6) prefetch_group(nxt, 4 * c + dt);
+                    if (have_next && 4 * c + dt < 6) prefetch_group(nxt, 4 * c + dt, n_early);
                 };
                 store_dt(std::integral_constant<int, 0>{});
                 store_dt(std::integral_constant<int, 1>{});
@@ -805,7 +845,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             };
             partial_block(std::integral_constant<int, 0>{});
             partial_block(std::integral_constant<int, 1>{});
-            if (have_next) prefetch_group(nxt, 6);
+            if (have_next) prefetch_group(nxt, 6, n_early);
             prev_stores = 0;                   // (the stores above are not counted: the next wait takes a few of them along)
             cur = nxt;
             have = have_next;
@@ -838,7 +878,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                     w[1] = pack_bf16(x[4 * g + 2] * inv, x[4 * g + 3] * inv);
                     *reinterpret_cast<u32x2*>(stage_w + (((4 * dt + g) ^ stage_wx) << 4)) = w;
                 }
-                if (have_next && 4 * c + dt < 6) prefetch_group(nxt, 4 * c + dt);
+                if (have_next && 4 * c + dt < 6) prefetch_group(nxt, 4 * c + dt, n_early);
             };
             stage_dt(std::integral_constant<int, 0>{});
             stage_dt(std::integral_constant<int, 1>{});
@@ -864,7 +904,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         store_block(std::integral_constant<int, 0>{});
         store_block(std::integral_constant<int, 1>{});
         // (the stores above took their data from the staged rows, so every read of them has returned)
-        if (have_next) prefetch_group(nxt, 6);
+        if (have_next) prefetch_group(nxt, 6, n_early);
         // (the rows of block A leave before the last query rows of the next job are requested; those of block B after)
         prev_stores = max(row_passes(cur) - 32 / kRowsPerPass, 0);
         cur = nxt;
