@@ -43,15 +43,26 @@ def _traffic(key):
         return None
 
 
-BURN_IN = 40        # untimed launches in front of the warm-up of an MFMA-bound leg (disclosed in the JSON line)
+BURN_MS = 40.0      # untimed launches for about this long in front of the warm-up of every leg but the two decode legs
+                    # (disclosed in the JSON line)
 
 
-def timed(fn, steps, warmup, burn_in=0):
+def timed(fn, steps, warmup, burn_ms=0.0):
     """Returns (wall ms/step, device ms/step): K launches between two syncs, HIP events on the launch stream.
-    `burn_in` extra untimed launches come first: the shader clock needs some tens of milliseconds of MFMA load
-    to leave its idle state, which a short warm-up does not give an MFMA-bound kernel."""
+    `burn_ms`: untimed launches for about that long come first.  A short warm-up leaves a short kernel inside the
+    clocks' transient: the shader clock needs some tens of milliseconds of MFMA load to leave its idle state, and a
+    0.15 ms streaming kernel runs its launches 10 to 50 about 10 % slower than the ones before and after."""
     import torch
-    for _ in range(burn_in + warmup):
+    if burn_ms > 0:
+        fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        one_ms = max((time.perf_counter() - t) * 1e3, 0.01)
+        for _ in range(min(int(burn_ms / one_ms) + 1, 1000)):
+            fn()
+    for _ in range(warmup):
         fn()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
@@ -120,7 +131,7 @@ def bench_prefill_backward(cfg, args):
     dout = torch.randn(out.shape, device=out.device, generator=g).to(torch.bfloat16)
     scale = 1.0 / (case.q.shape[-1] ** 0.5)
     wall_ms, dev_ms = timed(lambda: ops._prefill_backward(case.q, case.k, case.v, out, dout, lse, cu, cu, S, S, scale, 1),
-                            args.steps, args.warmup, BURN_IN)
+                            args.steps, args.warmup, BURN_MS)
     flops = case.flops() * 5 // 2
     return {
         "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
@@ -157,7 +168,7 @@ def bench_producers(args):
     v_cache = torch.zeros_like(k_cache)
     q_out = torch.empty_like(q)
     wall_ms, dev_ms = timed(lambda: mi355_attn.rope_and_cache(q, k, v, pos, freq, k_cache, v_cache, slots, out=q_out),
-                            args.steps, args.warmup)
+                            args.steps, args.warmup, BURN_MS)
     nbytes = 2 * (q.numel() + k.numel() + v.numel()) * 2 + T * 12 + freq.numel() * 4
     res["rope_and_cache"] = {
         "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 (fp32 rotation)",
@@ -175,7 +186,7 @@ def bench_producers(args):
     ks = torch.ones(n_blocks, Hkv, dtype=torch.float32, device=dev)
     vs = torch.ones_like(ks)
     wall_ms, dev_ms = timed(lambda: mi355_attn.rope_and_cache_fp8(q, k, v, pos, freq, k8, v8, ks, vs, slots, out=q_out),
-                            args.steps, args.warmup)
+                            args.steps, args.warmup, BURN_MS)
     nbytes = 2 * q.numel() * 2 + (k.numel() + v.numel()) * 3 + 2 * ks.numel() * 4 + T * 12 + freq.numel() * 4
     res["rope_and_cache_fp8"] = {
         "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 -> fp8-e4m3 (fp32 rotation)",
@@ -192,7 +203,7 @@ def bench_producers(args):
     pool = torch.randn(nb, Hkv, 16, D, device=dev, generator=g).to(torch.bfloat16)
     out8 = torch.empty(nb, Hkv, 16, D, dtype=torch.uint8, device=dev)
     scale = torch.empty(nb, Hkv, dtype=torch.float32, device=dev)
-    wall_ms, dev_ms = timed(lambda: mi355_attn.quantize_kv_cache_fp8(pool, out=(out8, scale)), args.steps, args.warmup)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.quantize_kv_cache_fp8(pool, out=(out8, scale)), args.steps, args.warmup, BURN_MS)
     nbytes = pool.numel() * 3 + scale.numel() * 4
     res["quantize_kv_fp8"] = {
         "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 -> fp8-e4m3",
@@ -218,7 +229,7 @@ def bench_layer_ops(args):
     x = torch.randn(T, d, device=dev, generator=g).to(torch.bfloat16)
     r = torch.randn(T, d, device=dev, generator=g).to(torch.bfloat16)
     w = torch.ones(d, device=dev)
-    wall_ms, dev_ms = timed(lambda: mi355_attn.rms_norm(x, w, 1e-5, residual=r, return_sum=True), args.steps, args.warmup)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.rms_norm(x, w, 1e-5, residual=r, return_sum=True), args.steps, args.warmup, BURN_MS)
     nbytes = 4 * T * d * 2 + d * 4                   # read x, residual; write y, sum
     res["rms_norm_residual"] = {
         "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 (fp32 math)",
@@ -229,7 +240,7 @@ def bench_layer_ops(args):
     }
     del x, r
     gu = torch.randn(T, 2 * ff, device=dev, generator=g).to(torch.bfloat16)
-    wall_ms, dev_ms = timed(lambda: mi355_attn.silu_mul(gu[:, :ff], gu[:, ff:]), args.steps, args.warmup)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.silu_mul(gu[:, :ff], gu[:, ff:]), args.steps, args.warmup, BURN_MS)
     nbytes = 3 * T * ff * 2
     res["silu_mul"] = {
         "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "bf16 (fp32 silu)",
@@ -412,7 +423,7 @@ def bench_prefill(cfg, args):
         def step():
             holder["out"] = mi355_attn.flash_attn_prefill(case.q, case.k, case.v, causal=True)
 
-    wall_ms, dev_ms = timed(step, args.steps, args.warmup, BURN_IN)
+    wall_ms, dev_ms = timed(step, args.steps, args.warmup, BURN_MS)
     flops = case.flops()
     res = {
         "value": flops / wall_ms / 1e9,
@@ -451,7 +462,7 @@ def bench_prefill_few_sequences(args):
         n_split = mi355_attn.suggest_kv_splits(1, Hq, D, Sq, Sk, Sq, True, q.device)
         ws = mi355_attn.prefill_splitkv_workspace(Sq, Hq, D, n_split, q.device) if n_split > 1 else None
         wall_ms, dev_ms = timed(lambda: mi355_attn.flash_attn_prefill(q, k, v, causal=True, kv_splits=n_split, workspace=ws),
-                                steps, warmup, BURN_IN)
+                                steps, warmup, BURN_MS)
         res = {
             "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
             "algorithmic_flops": flops, "kv_splits": n_split,
@@ -464,7 +475,7 @@ def bench_prefill_few_sequences(args):
                          "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms, "traffic": None},
         }
         if n_split > 1:
-            _, one_ms = timed(lambda: mi355_attn.flash_attn_prefill(q, k, v, causal=True, kv_splits=1), steps, warmup)
+            _, one_ms = timed(lambda: mi355_attn.flash_attn_prefill(q, k, v, causal=True, kv_splits=1), steps, warmup, BURN_MS)
             res["unsplit_device_ms"] = one_ms
             res["speedup_over_unsplit"] = one_ms / dev_ms
         out[name] = res
@@ -479,7 +490,7 @@ def bench_prefill_few_sequences(args):
     q, k, v = rnd(T, Hq, D), rnd(T, Hkv, D), rnd(T, Hkv, D)
     flops = sum(4.0 * Hq * D * n * n / 2.0 for n in lens)
     wall_ms, dev_ms = timed(lambda: mi355_attn.flash_attn_varlen_prefill(q, k, v, cu, cu, longest, longest, causal=True, kv_splits=1),
-                            steps, warmup, BURN_IN)
+                            steps, warmup, BURN_MS)
     out["ragged_batch_16"] = {
         "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
         "algorithmic_flops": flops, "kv_splits": 1,
@@ -565,7 +576,7 @@ def main():
     }
     # Every GPU leg runs first, back to back (the shader clock then stays in its loaded state: a GPU that idles
     # through a CPU leg starts the next kernel at a low clock); the CPU oracle legs follow on the kept outputs.
-    line["burn_in_launches_before_mfma_legs"] = BURN_IN
+    line["burn_in_ms_before_every_leg_but_decode"] = BURN_MS
     dec = pre = f8 = None
     kept = {}
     if args.only in (None, "decode"):
