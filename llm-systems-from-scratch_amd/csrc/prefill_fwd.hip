@@ -473,28 +473,50 @@ struct MergeParams {
     int64_t part_rows;
     int n_split, Hq, D, Sq_dense;        // Sq_dense: rows per batch entry of the dense layout, 0 = packed
 };
+// One (query row, head) per D/4 lanes: a lane owns four adjacent d of the row (16-byte loads of the partial rows, an
+// 8-byte store), and the partial rows of up to eight shares are in flight together.
 __global__ __launch_bounds__(256) void prefill_merge_kernel(MergeParams p) {
+    const int lanes_per_row = p.D / 4, rows_per_wave = 64 / lanes_per_row;
     const int lane = threadIdx.x & 63;
-    const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (w >= p.part_rows * p.Hq) return;
-    const int h = (int)(w % p.Hq);
-    const int64_t row = w / p.Hq;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t item = wave * rows_per_wave + lane / lanes_per_row;
+    if (item >= p.part_rows * p.Hq) return;
+    const int d = 4 * (lane % lanes_per_row);
+    const int h = (int)(item % p.Hq);
+    const int64_t row = item / p.Hq;
+    const int64_t share_stride = (int64_t)p.Hq * p.part_rows;          // rows from one share to the next
+    const int64_t prow0 = (int64_t)h * p.part_rows + row;
     float m = -INFINITY;
-    for (int c = 0; c < p.n_split; ++c) m = fmaxf(m, p.part_lse[((int64_t)c * p.Hq + h) * p.part_rows + row]);
+    for (int c = 0; c < p.n_split; ++c) m = fmaxf(m, p.part_lse[prow0 + c * share_stride]);
+    f32x4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+    for (int c0 = 0; c0 < p.n_split; c0 += 8) {
+        float wgt[8];
+        f32x4 part[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int64_t prow = prow0 + (int64_t)min(c0 + i, p.n_split - 1) * share_stride;
+            const float l = p.part_lse[prow];
+            // (a share that kept no key for the row has -inf here, and its partial row may never have been written)
+            wgt[i] = c0 + i < p.n_split && l != -INFINITY ? __expf(l - m) : 0.f;
+            part[i] = wgt[i] != 0.f ? *reinterpret_cast<const f32x4*>(p.part_o + prow * p.D + d) : f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (wgt[i] != 0.f) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) num[e] += wgt[i] * part[i][e];
+                den += wgt[i];
+            }
+        }
+    }
     __bf16* dst = p.Sq_dense ? p.out + (row / p.Sq_dense) * p.os[0] + (int64_t)h * p.os[1] + (row % p.Sq_dense) * p.os[2]
                              : p.out + row * p.os[2] + (int64_t)h * p.os[1];
-    for (int d = lane; d < p.D; d += 64) {
-        float num = 0.f, den = 0.f;
-        for (int c = 0; c < p.n_split; ++c) {
-            const int64_t prow = ((int64_t)c * p.Hq + h) * p.part_rows + row;
-            const float l = p.part_lse[prow];
-            if (l == -INFINITY) continue;                 // (its rows may never have been written)
-            const float wgt = __expf(l - m);
-            num += wgt * p.part_o[prow * p.D + d];
-            den += wgt;
-        }
-        dst[d] = (__bf16)(m == -INFINITY ? __builtin_nanf("") : num / den);
-    }
+    const float none = __builtin_nanf("");
+    u32x2 packed;
+    packed[0] = m == -INFINITY ? pack_bf16(none, none) : pack_bf16(num[0] / den, num[1] / den);
+    packed[1] = m == -INFINITY ? pack_bf16(none, none) : pack_bf16(num[2] / den, num[3] / den);
+    *reinterpret_cast<u32x2*>(dst + d) = packed;
 }
 
 static int launch_merge(const PrefillParams& p, int D, hipStream_t stream) {
@@ -508,7 +530,8 @@ static int launch_merge(const PrefillParams& p, int D, hipStream_t stream) {
     m.Hq = p.Hq;
     m.D = D;
     m.Sq_dense = (p.cu_q || p.block_table) ? 0 : p.Sq;
-    const int64_t wgs = (p.part_rows * p.Hq + 3) / 4;
+    const int64_t per_wg = 4 * (64 / (D / 4));                  // (row, head) items per workgroup of four wavefronts
+    const int64_t wgs = (p.part_rows * p.Hq + per_wg - 1) / per_wg;
     if (wgs > 0x7fffffffLL) return (int)hipErrorInvalidValue;
     hipLaunchKernelGGL(prefill_merge_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, m);
     return (int)hipGetLastError();
