@@ -765,7 +765,7 @@ extern "C" int mi355_prefill_suggest_kv_splits(int B, int Hq, int D, int Sq_max,
     }
     const double halves = nq >= 2 ? 2.0 : 1.0;
     const auto rounds = [&](double wgs) { return (double)(int64_t)((wgs + n_cu - 1) / n_cu); };
-    const auto partials = [&](int n) { return 8.0 + 2.0 * ((double)total_q_rows * Hq * (D + 1) * 4.0 * n) / 2.5e6; };
+    const auto partials = [&](int n) { return 8.0 + 2.0 * ((double)total_q_rows * Hq * (D + 1) * 4.0 * n) / 3.0e6; };
     double plain;
     int best_n = 1;
     static const int kCandidates[] = {2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
