@@ -216,7 +216,7 @@ size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx);
  * allocate or size a workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * Same arguments, kernels and results (bit for bit) as mi355_paged_decode_fwd otherwise.
  *   - a call whose partials need more than the array (mi355_paged_decode_workspace_bytes of the layout actually
- *     used, i.e. B * Hq * ceil(max_ctx / mi355_paged_decode_chunk_tokens(max_ctx)) * (D + 2) * 4 bytes plus padding)
+ *     used, i.e. B * Hq * ceil(max_ctx / mi355_paged_decode_chunk_tokens(B, Hq, Hkv, max_ctx)) * (D + 2) * 4 bytes plus padding)
  *     is rejected with MI355_EWORKSPACE; max_ctx up to one chunk needs no scratch at all;
  *   - all calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
  *     threads) race on it and must be serialised by the caller; the array's old contents never matter (every
@@ -232,8 +232,10 @@ int mi355_paged_decode_fwd_static(const void* q, const void* k_cache, const void
                                   int B, int Hq, int Hkv, int D, int block_size, int64_t num_blocks, int max_ctx,
                                   float softmax_scale, int kv_dtype, void* stream);
 
-/* Tokens of one sequence handled by one workgroup of the split-K pass (grows with max_ctx). */
-int mi355_paged_decode_chunk_tokens(int max_ctx);
+/* Tokens of one sequence handled by one workgroup of the split-K pass: grows with max_ctx (1024, 2048, 4096) and
+ * shrinks again, down to 256, while a batch of contexts beyond 1024 tokens has fewer workgroups than the GPU has
+ * compute units. */
+int mi355_paged_decode_chunk_tokens(int B, int Hq, int Hkv, int max_ctx);
 
 /*
  * RoPE + KV-cache write: the producer of the paged cache (the step right before the

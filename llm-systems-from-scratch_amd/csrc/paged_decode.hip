@@ -446,28 +446,46 @@ using namespace mi355;
 static size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // Tokens per wavefront grow with the longest context: short batches keep all four wavefronts of
-// a workgroup busy, long ones get long uninterrupted streams.
-static int tokens_per_wave_for(int max_ctx) {
-    return max_ctx >= 4096 ? kMaxTokensPerWave : (max_ctx >= 2048 ? 512 : 256);
+// a workgroup busy, long ones get long uninterrupted streams.  A small batch then has too few workgroups
+// for the GPU -- one sequence of 8192 tokens on 8 kv heads: 16 -- and gets shorter streams until there is
+// about a workgroup per compute unit (the same sequence: 256 workgroups of 4 x 64 tokens).
+// items = B * Hkv * (groups of 16 query heads per kv head): the workgroups per chunk.
+constexpr int kMinTokensPerWave = 64;
+constexpr int kTargetWorkgroups = 256;
+static int tokens_per_wave_for(int max_ctx, int64_t items) {
+    int tpw = max_ctx >= 4096 ? kMaxTokensPerWave : (max_ctx >= 2048 ? 512 : 256);
+    // (up to 1024 tokens one chunk serves a sequence and no combine pass is needed: worth more than shorter streams)
+    if (max_ctx <= kDecodeWaves * 256) return tpw;
+    while (tpw > kMinTokensPerWave && items * ((max_ctx + kDecodeWaves * tpw - 1) / (kDecodeWaves * tpw)) < kTargetWorkgroups) tpw /= 2;
+    return tpw;
+}
+static int n_groups_of(int Hq, int Hkv) { return (Hq / Hkv + 15) / 16; }
+
+extern "C" int mi355_paged_decode_chunk_tokens(int B, int Hq, int Hkv, int max_ctx) {
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || max_ctx <= 0) return 0;
+    return kDecodeWaves * tokens_per_wave_for(max_ctx, (int64_t)B * Hkv * n_groups_of(Hq, Hkv));
 }
 
-extern "C" int mi355_paged_decode_chunk_tokens(int max_ctx) { return kDecodeWaves * tokens_per_wave_for(max_ctx); }
-
-// Bytes of split-K partials for `chunks` chunks per (sequence, query head): O (D fp32), m, l.
-static size_t workspace_layout_bytes(size_t B, size_t Hq, size_t D, size_t chunks) {
-    const size_t rows = B * Hq * chunks;
+// Bytes of split-K partials for `rows` (sequence, query head, chunk) triples: O (D fp32), m, l.
+static size_t workspace_layout_bytes(size_t rows, size_t D) {
     return align_up(rows * D * 4, 256) + 2 * align_up(rows * 4, 256);
 }
 
-// The chunk size grows with max_ctx (1024, 2048, 4096 tokens), so the number of chunks a launch really uses,
-// ceil(max_ctx / chunk(max_ctx)), is not monotonic in max_ctx: it is at most 2 below 4096 tokens and
-// ceil(max_ctx / 4096) from there on.  The requirement reported here is the largest one over every bound up to
-// max_ctx, so a workspace sized for a caller's longest context serves every shorter one.
+// The chunk size depends on max_ctx (1024, 2048, 4096 tokens) and shrinks for small batches, so the number of
+// chunks a launch really uses is not monotonic in max_ctx or B.  The requirement reported here bounds it for every
+// launch with a batch up to B and a bound up to max_ctx: chunks of the full size need at most 2 per sequence below
+// 4096 tokens and ceil(max_ctx / 4096) from there on; shrunken chunks mean fewer than 2 * kTargetWorkgroups
+// workgroups, i.e. fewer than 32 * kTargetWorkgroups rows (a workgroup serves at most 16 query heads), and never
+// more than ceil(max_ctx / 256) per sequence.  A workspace sized for a caller's largest batch and longest context
+// therefore serves every smaller call.
 extern "C" size_t mi355_paged_decode_workspace_bytes(int B, int Hq, int D, int max_ctx) {
     if (B <= 0 || Hq <= 0 || D <= 0 || max_ctx <= 0) return 0;
     const size_t big = ((size_t)max_ctx + 4 * kMaxTokensPerWave - 1) / (4 * kMaxTokensPerWave);
     const size_t small = max_ctx > 4 * 256 ? 2 : 1;
-    return workspace_layout_bytes((size_t)B, (size_t)Hq, (size_t)D, big > small ? big : small);
+    const size_t full = (size_t)B * Hq * (big > small ? big : small);
+    const size_t finest = (size_t)B * Hq * (((size_t)max_ctx + kDecodeWaves * kMinTokensPerWave - 1) / (kDecodeWaves * kMinTokensPerWave));
+    const size_t shrunk = finest < (size_t)32 * kTargetWorkgroups ? finest : (size_t)32 * kTargetWorkgroups;
+    return workspace_layout_bytes(full > shrunk ? full : shrunk, (size_t)D);
 }
 
 // Argument checks and launches shared by the two entry points.  `static_scratch`: the workspace is the library's
@@ -484,11 +502,11 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || max_ctx <= 0)
         return set_error(MI355_EINVAL, "paged_decode: B, Hq, Hkv and max_ctx must be positive");
     if (Hq % Hkv != 0) return set_error(MI355_EINVAL, "paged_decode: Hq must be a multiple of Hkv");
-    const int n_groups = (Hq / Hkv + 15) / 16;
+    const int n_groups = n_groups_of(Hq, Hkv);
     if (block_size != kBlock) return set_error(MI355_EINVAL, "paged_decode: block_size must be 16");
     if (num_blocks <= 0 || num_blocks > 0x7fffffffLL)
         return set_error(MI355_EINVAL, "paged_decode: num_blocks must be positive (and below 2^31)");
-    const int chunk = mi355_paged_decode_chunk_tokens(max_ctx);
+    const int chunk = mi355_paged_decode_chunk_tokens(B, Hq, Hkv, max_ctx);
     if ((int64_t)((max_ctx + chunk - 1) / chunk) * Hkv * n_groups * B > 0x7fffffffLL)
         return set_error(MI355_EINVAL, "paged_decode: chunks * Hkv * B exceeds the grid limit");
     if (kv_dtype != MI355_BF16 && kv_dtype != MI355_FP8_E4M3)
@@ -499,7 +517,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
     if (!(D == 128 || D == 64 || (D == 32 && !fp8)))
         return set_error(MI355_EINVAL, "paged_decode: head_dim must be 64 or 128 (or 32 with a bf16 cache)");
     const int max_chunks = (max_ctx + chunk - 1) / chunk;
-    const size_t need = workspace_layout_bytes((size_t)B, (size_t)Hq, (size_t)D, (size_t)max_chunks);   // <= the reported bound
+    const size_t need = workspace_layout_bytes((size_t)B * Hq * max_chunks, (size_t)D);   // <= the reported bound
     if (static_scratch) {
         if (max_chunks > 1 && need > workspace_bytes)
             return set_error(MI355_EWORKSPACE,
@@ -536,7 +554,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
     p.max_chunks = max_chunks;
     p.max_ctx = max_ctx;
     p.n_groups = n_groups;
-    p.tokens_per_wave = tokens_per_wave_for(max_ctx);
+    p.tokens_per_wave = chunk / kDecodeWaves;
     p.scale_log2 = softmax_scale * kLog2e;
 
     hipStream_t s = (hipStream_t)stream;

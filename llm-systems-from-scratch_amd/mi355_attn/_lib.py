@@ -83,7 +83,7 @@ def load():
     lib.mi355_paged_decode_workspace_bytes.restype = sz
     lib.mi355_paged_decode_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.mi355_paged_decode_chunk_tokens.restype = i32
-    lib.mi355_paged_decode_chunk_tokens.argtypes = [i32]
+    lib.mi355_paged_decode_chunk_tokens.argtypes = [i32, i32, i32, i32]
     lib.mi355_rope_and_cache.restype = i32
     lib.mi355_rope_and_cache.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32,
                                          i64, i64, i64, i64, vp, i64, vp]

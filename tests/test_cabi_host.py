@@ -34,9 +34,17 @@ def test_library_exports_every_declared_symbol(lib):
 
 def test_version_and_workspace_queries(lib):
     assert b"gfx950" in lib.mi355_version()
-    assert lib.mi355_paged_decode_chunk_tokens(256) == 1024
-    assert lib.mi355_paged_decode_chunk_tokens(3000) == 2048
-    assert lib.mi355_paged_decode_chunk_tokens(16384) == 4096
+    # (batch, query heads, kv heads, longest context): a batch that fills the GPU gets chunks that grow with the context
+    assert lib.mi355_paged_decode_chunk_tokens(128, 32, 8, 256) == 1024
+    assert lib.mi355_paged_decode_chunk_tokens(128, 32, 8, 3000) == 2048
+    assert lib.mi355_paged_decode_chunk_tokens(128, 32, 8, 16384) == 4096
+    # ... and a small batch shorter ones, until it has about 256 workgroups (down to 4 x 64 tokens)
+    assert lib.mi355_paged_decode_chunk_tokens(1, 32, 8, 8192) == 256
+    assert lib.mi355_paged_decode_chunk_tokens(1, 32, 8, 131072) == 4096
+    assert lib.mi355_paged_decode_chunk_tokens(4, 32, 8, 8192) == 1024
+    assert lib.mi355_paged_decode_chunk_tokens(1, 32, 8, 100) == 1024          # one chunk and no combine pass up to 1024 tokens
+    assert lib.mi355_paged_decode_chunk_tokens(1, 32, 8, 1025) == 256
+    assert lib.mi355_paged_decode_chunk_tokens(0, 32, 8, 100) == 0 and lib.mi355_paged_decode_chunk_tokens(1, 32, 5, 100) == 0
     # one chunk -> still a (small) partial area; grows with chunks * B * Hq * D
     small = lib.mi355_paged_decode_workspace_bytes(4, 8, 64, 256)
     big = lib.mi355_paged_decode_workspace_bytes(128, 32, 128, 16384)
@@ -47,19 +55,33 @@ def test_version_and_workspace_queries(lib):
 
 
 def test_workspace_requirement_is_monotonic_in_max_ctx(lib):
-    """A workspace sized for the longest context must serve every shorter one, although the chunk size (and with it
-    the number of chunks a launch uses) changes at 2048 and 4096 tokens."""
-    for B, Hq, D in ((64, 16, 128), (3, 8, 64)):
+    """A workspace sized for the largest batch and the longest context must serve every smaller call, although the
+    chunk size (and with it the number of chunks a launch uses) changes at 2048 and 4096 tokens and shrinks for
+    small batches."""
+    def need(B, Hq, Hkv, D, m):          # what a launch with these bounds really lays out
+        chunk = lib.mi355_paged_decode_chunk_tokens(B, Hq, Hkv, m)
+        rows = B * Hq * ((m + chunk - 1) // chunk)
+        return rows * D * 4 + 2 * rows * 4
+
+    for B, Hq, Hkv, D in ((64, 16, 4, 128), (3, 8, 8, 64), (1, 32, 8, 128), (2, 64, 1, 128)):
         prev = 0
         for m in list(range(1, 9000, 7)) + [16384, 16385, 32768, 100000]:
             cur = lib.mi355_paged_decode_workspace_bytes(B, Hq, D, m)
             assert cur >= prev, (B, Hq, D, m)
-            chunk = lib.mi355_paged_decode_chunk_tokens(m)
-            rows = B * Hq * ((m + chunk - 1) // chunk)          # what a launch with this bound really lays out
-            assert cur >= rows * D * 4 + 2 * rows * 4, (B, Hq, D, m)
+            assert cur >= need(B, Hq, Hkv, D, m), (B, Hq, D, m)
             prev = cur
         # and in the batch and head counts
         assert lib.mi355_paged_decode_workspace_bytes(B - 1, Hq, D, 5000) <= lib.mi355_paged_decode_workspace_bytes(B, Hq, D, 5000)
+    # every smaller call fits the workspace of the largest one
+    Hq, Hkv, D = 32, 8, 128
+    for B_max, m_max in ((64, 32768), (8, 4096), (256, 2000)):
+        have = lib.mi355_paged_decode_workspace_bytes(B_max, Hq, D, m_max)
+        for B in sorted({1, 2, 3, 5, 8, 13, 32, 63, B_max}):
+            if B > B_max:
+                continue
+            for m in (1, 255, 257, 1000, 1025, 2047, 2048, 4095, 4096, 8191, 20000, m_max):
+                if m <= m_max:
+                    assert need(B, Hq, Hkv, D, m) <= have, (B_max, m_max, B, m)
 
 
 def test_prefill_rejects_bad_arguments_without_a_gpu(lib):

@@ -97,6 +97,26 @@ def test_decode_long_contexts_multi_chunk(ops, fp8):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("ctx", [1025, 9000])
+def test_decode_of_one_sequence_uses_the_shortest_chunks(ops, fp8, ctx):
+    """One sequence on two kv heads: far fewer workgroups than compute units at any chunk size, so the split-K pass
+    runs with its shortest chunks (4 wavefronts x 64 tokens; 5 and 36 chunks here, the last one partial) and the
+    combine pass merges them."""
+    print(f"case: decode one sequence ctx={ctx} fp8={fp8}", flush=True)
+    q, kc, vc, bt, cl = orc.make_paged_case(batch=1, n_q_heads=8, n_kv_heads=2, head_dim=128, block_size=16,
+                                            context_lens=[ctx], pool_factor=1.3, seed=91, dtype=torch.bfloat16)
+    if fp8:
+        k8, ks = orc.quantize_kv_fp8(kc)
+        v8, vs = orc.quantize_kv_fp8(vc)
+        got = run_decode(ops, q, k8, v8, bt, cl, k_scale=ks, v_scale=vs)
+        ref = orc.paged_decode_reference(q, k8, v8, bt, cl, k_scale=ks, v_scale=vs)
+    else:
+        got = run_decode(ops, q, kc, vc, bt, cl)
+        ref = orc.paged_decode_reference(q, kc, vc, bt, cl)
+    check(got, ref, what=f"one sequence ctx={ctx} fp8={fp8}")
+
+
+@pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("slope", [0.4, 0.02, -0.02, -0.4])
 def test_decode_scores_that_ramp_along_the_context(ops, fp8, slope):
     """Scores that rise (or fall) steadily with the token position, by much more or much less per 32-key step than
