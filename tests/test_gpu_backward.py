@@ -116,6 +116,37 @@ def test_backward_varlen_equals_per_sequence(ops):
 
 
 @pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("seed", [0, 1])
+def test_backward_packed_sequences_of_very_different_lengths(ops, D, seed):
+    """Packed sequences from one token to several query tiles, 8 query heads on 2 kv heads: the grids of the two
+    backward kernels then hold several chunks of workgroup ids per XCD, whole rounds of eight chunks and a partial
+    one, and many workgroups of short sequences that have nothing to do."""
+    g = torch.Generator().manual_seed(7000 + seed)
+    n_seq = int(torch.randint(6, 10, (1,), generator=g))
+    lens = [int(x) for x in torch.randint(1, 900, (n_seq,), generator=g)]
+    lens[int(torch.randint(0, n_seq, (1,), generator=g))] = 1
+    print(f"case: backward packed D={D} seed={seed} lens={lens}", flush=True)
+    Hq, Hkv = 8, 2
+    T = sum(lens)
+    cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32)
+    q, k, v, dout = (rnd(T, Hq, D, seed=7100 + seed), rnd(T, Hkv, D, seed=7200 + seed), rnd(T, Hkv, D, seed=7300 + seed),
+                     rnd(T, Hq, D, seed=7400 + seed))
+    qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+    out = ops.flash_attn_varlen_prefill(qg, kg, vg, cu.cuda(), cu.cuda(), max(lens), max(lens), causal=True)
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    dq_ref, dk_ref, dv_ref = torch.zeros(T, Hq, D), torch.zeros(T, Hkv, D), torch.zeros(T, Hkv, D)
+    for b in range(n_seq):
+        sl = slice(int(cu[b]), int(cu[b + 1]))
+        args = [t[sl].transpose(0, 1)[None] for t in (q, k, v, dout)]
+        a, bb, c, _ = orc.prefill_backward_reference(*args, causal=True)
+        dq_ref[sl], dk_ref[sl], dv_ref[sl] = a[0].transpose(0, 1), bb[0].transpose(0, 1), c[0].transpose(0, 1)
+    check_grad("dq", qg.grad, dq_ref)
+    check_grad("dk", kg.grad, dk_ref)
+    check_grad("dv", vg.grad, dv_ref)
+
+
+@pytest.mark.parametrize("D", [64, 128])
 def test_forward_lse_matches_oracle(ops, D):
     """head_dim 64: the 8-wavefront kernel; 128: the 64-query kernel, whose log-sum-exp comes from its row sums and
     the exponent reference that went into them -- also after that reference has moved (keys with runaway scores),
