@@ -253,6 +253,48 @@ def bench_layer_ops(args):
     return res
 
 
+def bench_decode_few_sequences(args):
+    """Decode attention of a few long sequences (the reference's `generate` is batch 1): too few (sequence, kv head)
+    pairs for the compute units at the chunk size of a large batch, so the split-K pass runs with shorter chunks.
+    Timed in a HIP graph of ten steps (the host takes longer to issue one eager step than the GPU to run it)."""
+    import torch
+    import mi355_attn
+    from mi355_attn import workloads
+
+    out = {}
+    for name, batch, ctx in (("one_sequence_8192", 1, 8192), ("one_sequence_32768", 1, 32768), ("four_sequences_8192", 4, 8192)):
+        case = workloads.make_decode_case(batch=batch, n_q_heads=32, n_kv_heads=8, head_dim=128, ctx_kind="fixed", ctx_lo=ctx,
+                                          ctx_hi=ctx, pool_factor=1.1, seed=args.seed)
+        B, Hq, D = case.q.shape
+        ws = mi355_attn.paged_decode_workspace(B, Hq, D, case.max_context, case.q.device)
+        res = torch.empty_like(case.q)
+
+        def step():
+            mi355_attn.paged_attention_decode(case.q, case.k_cache, case.v_cache, case.block_tables, case.context_lens,
+                                              max_context=case.max_context, workspace=ws, out=res)
+
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            step()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(10):
+                    step()
+        wall_ms, dev_ms = timed(graph.replay, max(1, args.steps // 2), args.warmup, BURN_MS)
+        nbytes = case.algorithmic_bytes()
+        out[name] = {
+            "us_per_step": dev_ms * 100.0, "algorithmic_bytes": nbytes,
+            "chunk_tokens": mi355_attn.decode_chunk_tokens(B, Hq, 8, case.max_context),
+            "config": {"workload": "paged decode attention, bf16 KV, %d sequence(s) of %d tokens, 32 q / 8 kv heads, "
+                                   "head_dim 128, ten steps per graph launch" % (batch, ctx)},
+            "roofline": {"bound": "hbm", "kernel": "paged_decode_split_kernel + paged_decode_combine_kernel",
+                         "achieved": nbytes / (dev_ms / 10.0) / 1e6, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": nbytes / (dev_ms / 10.0) / 1e6 / HBM_PEAK_GBPS, "device_ms": dev_ms / 10.0, "traffic": None},
+        }
+    return out
+
+
 def bench_decode_loop(args):
     """Decode steps of the KV-cached decoder at the reference's sample model (configures/sample.yaml:
     vocab 10000, context 256, d_model 512, 4 layers, 16 heads, d_ff 1344; random weights), batch 8:
@@ -616,6 +658,7 @@ def main():
     if args.only in (None, "layer"):
         line["layer_ops"] = bench_layer_ops(args)
     if args.only in (None, "loop"):
+        line["decode_few_sequences"] = bench_decode_few_sequences(args)
         line["decode_loop"] = bench_decode_loop(args)
 
     if with_cpu:

@@ -28,6 +28,7 @@ from .ops import (  # noqa: F401
     flash_attn_varlen_prefill,
     paged_attention_decode,
     paged_decode_workspace,
+    decode_chunk_tokens,
     prefill_splitkv_workspace,
     suggest_kv_splits,
     scaled_dot_product_attention,

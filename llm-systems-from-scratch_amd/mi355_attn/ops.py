@@ -383,6 +383,11 @@ def flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
     return out if out.dtype == out_dtype else out.to(out_dtype)
 
 
+def decode_chunk_tokens(batch, n_q_heads, n_kv_heads, max_context):
+    """Tokens of one sequence that one workgroup of the split-K decode pass handles for these bounds."""
+    return int(_lib.load().mi355_paged_decode_chunk_tokens(batch, n_q_heads, n_kv_heads, max_context))
+
+
 def paged_decode_workspace(batch, n_q_heads, head_dim, max_context, device):
     """Scratch tensor for paged_attention_decode.  The requirement is monotonic in every argument, so a tensor
     sized for the largest batch and longest context serves every smaller call."""
