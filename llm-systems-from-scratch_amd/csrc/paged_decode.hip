@@ -95,11 +95,26 @@ void paged_decode_split_kernel(DecodeParams p) {
     // with ragged lengths late chunks are mostly empty and the XCDs that own them would idle.
     // Chunks are dealt in DESCENDING order: the full chunks of the long sequences start first
     // and the first chunks of the short sequences (the smallest work items) form the tail.
+    // A kv head with more than 16 query heads is served by several workgroups per (sequence, chunk), 16 query heads
+    // each, which read the same K/V: they sit eight ids apart, i.e. on one XCD and next to each other in time, so that
+    // the stream comes from HBM once and from that XCD's L2 afterwards.
     const int wg = blockIdx.x;
-    const int hk = wg % p.Hkv;
-    const int grp = (wg / p.Hkv) % p.n_groups;           // which 16 query heads of the kv head (0 unless Hq/Hkv > 16)
-    const int b = (wg / (p.Hkv * p.n_groups)) % p.B;
-    const int chunk = p.max_chunks - 1 - wg / (p.Hkv * p.n_groups * p.B);
+    int item = wg, grp = 0;                               // item = (kv head, sequence, chunk); grp = which 16 query heads
+    if (p.n_groups > 1) {
+        const int items = gridDim.x / p.n_groups, whole = items / 8 * 8;
+        if (wg < whole * p.n_groups) {
+            const int within = wg % (8 * p.n_groups);
+            grp = within / 8;
+            item = wg / (8 * p.n_groups) * 8 + within % 8;
+        } else {
+            const int rest = wg - whole * p.n_groups;
+            grp = rest % p.n_groups;
+            item = whole + rest / p.n_groups;
+        }
+    }
+    const int hk = item % p.Hkv;
+    const int b = (item / p.Hkv) % p.B;
+    const int chunk = p.max_chunks - 1 - item / (p.Hkv * p.B);
     const int ctx = min(p.context_lens[b], p.max_ctx);     // a length beyond the promised bound is truncated, never chased
     const int chunk_tokens = kDecodeWaves * p.tokens_per_wave;
     const int chunk_start = chunk * chunk_tokens;

@@ -742,10 +742,12 @@ def test_prefill_varlen_sequence_longer_than_promised(ops):
 
 
 def test_decode_more_than_16_query_heads_per_kv_head(ops):
-    """Hq/Hkv = 32 and 20 (multi-query style): the kv head is streamed once per 16 query heads."""
-    for Hq, Hkv, D in ((32, 1, 128), (40, 2, 64)):
-        print(f"case: decode Hq/Hkv > 16: {Hq}/{Hkv}", flush=True)
-        ctx = [1, 17, 300, 5000]
+    """Hq/Hkv = 32, 20 and 48 (multi-query style): the kv head is streamed once per 16 query heads, by workgroups
+    that sit eight ids apart -- with whole blocks of eight (sequence, chunk) items, with fewer than eight items, and
+    with eleven."""
+    for Hq, Hkv, D, ctx in ((32, 1, 128, [1, 17, 300, 5000]), (40, 2, 64, [1, 17, 300, 5000]), (32, 1, 128, [5, 700, 1000]),
+                            (48, 1, 64, [900, 3, 1024, 77, 512, 1, 640, 999, 16, 17, 1000])):
+        print(f"case: decode Hq/Hkv > 16: {Hq}/{Hkv} ctx={ctx}", flush=True)
         q, kc, vc, bt, cl = orc.make_paged_case(batch=len(ctx), n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
                                                 context_lens=ctx, pool_factor=1.2, seed=Hq, dtype=torch.bfloat16)
         check(run_decode(ops, q, kc, vc, bt, cl), orc.paged_decode_reference(q, kc, vc, bt, cl), what=f"{Hq}/{Hkv}")
