@@ -13,8 +13,12 @@ The CPU baseline is the oracle (a restatement of the reference's PyTorch attenti
 timed on the host cores over a bounded sample of the same inputs; its outputs also
 check the GPU results of that sample.
 
-usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S] [--only decode|prefill|few|fp8|backward|producers|layer|loop]
-                       [--no-cpu]
+The line is kept short (the driver keeps only the end of stdout): the contract's fields for configs[3], then the
+fp8 decode, then one {ms, frac} pair per auxiliary leg under "legs", and the configs[2] `prefill` object LAST.
+`--full` prints every leg's whole object instead; `--detail PATH` writes that verbose form to a file.
+
+usage: python bench.py [--gpus 1] [--steps K=200] [--warmup W=50] [--seed S]
+                       [--only decode|prefill|small|few|fp8|backward|producers|layer|loop] [--no-cpu] [--full] [--detail PATH]
 """
 from __future__ import annotations
 
@@ -41,6 +45,11 @@ def _traffic(key):
             return json.load(f).get(key)
     except (OSError, ValueError):
         return None
+
+
+def _prefill_kernel(head_dim):
+    """Name of the kernel a causal, unsplit prefill of this head_dim runs on."""
+    return "prefill_fwd_w64_kernel<causal>" if head_dim == 128 else "prefill_fwd_kernel<%d, causal>" % head_dim
 
 
 BURN_MS = 40.0      # untimed launches for about this long in front of the warm-up of every leg but the two decode legs
@@ -473,13 +482,73 @@ def bench_prefill(cfg, args):
         "ms_per_step": wall_ms,
         "algorithmic_flops": flops,
         "roofline": {
-            "bound": "mfma", "kernel": "prefill_fwd_w64_kernel<causal>" if case.q.shape[-1] == 128 else "prefill_fwd_kernel",
+            "bound": "mfma", "kernel": _prefill_kernel(case.q.shape[-1]),
             "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms,
             "traffic": _traffic(f"prefill_cfg{cfg}"),
         },
     }
     return res, (case, holder["out"])
+
+
+def bench_prefill_small(args, with_cpu):
+    """The two small prefill shapes: configs[1] (dense, batch 4, 16 heads, head_dim 64, 1024 tokens) and the attention
+    call of the reference's sample model (configures/sample.yaml:2-12: batch 64, 16 heads of head_dim 32, context 256,
+    through the slot at llm-core/llm_core/model.py:382 with V as the strided view of its projection).  A few
+    microseconds of MFMA work each: the figures are launch-bound latencies, reported with their roofline fraction
+    but not part of the target.  CPU baseline: the oracle on the whole shape, 1 warm-up + best of 3 passes."""
+    import torch
+    import mi355_attn
+    from mi355_attn import workloads
+
+    out = {}
+    case = workloads.prefill_config(1, seed=args.seed)
+    B, H, S, D = 64, 16, 256, 32
+    g = torch.Generator(device="cuda").manual_seed(args.seed + 3)
+    qs = (torch.randn(B, H, S, D, generator=g, device="cuda") * 0.5).to(torch.bfloat16)
+    ks = (torch.randn(B, H, S, D, generator=g, device="cuda") * 0.5).to(torch.bfloat16)
+    vs = (torch.randn(B, S, H * D, generator=g, device="cuda") * 0.5).to(torch.bfloat16).view(B, S, H, D).permute(0, 2, 1, 3)
+    for name, (q, k, v), what in (
+            ("prefill_cfg1", (case.q, case.k, case.v),
+             "configs[1]: causal prefill forward, bf16, dense, batch 4, 16 heads, head_dim 64, seq 1024, seed %d" % args.seed),
+            ("prefill_sample_model", (qs, ks, vs),
+             "the reference sample model's attention call (sample.yaml: batch 64, 16 heads, head_dim 32, context 256), "
+             "V a strided view, through sdpa_slot")):
+        holder = {}
+
+        def step():
+            holder["out"] = mi355_attn.sdpa_slot(q, k, v, is_causal=True)
+
+        wall_ms, dev_ms = timed(step, args.steps, args.warmup, BURN_MS)
+        b, h, n, d = q.shape
+        flops = 4 * b * h * d * n * n // 2
+        res = {
+            "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
+            "algorithmic_flops": flops, "config": {"workload": what},
+            "roofline": {"bound": "mfma", "kernel": _prefill_kernel(d),
+                         "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms, "traffic": None,
+                         "note": "a few microseconds of MFMA work: launch-bound latency figure"},
+        }
+        if with_cpu:
+            from oracle import attention_oracle as orc
+            qc, kc, vc = q.cpu(), k.cpu(), v.cpu()
+            torch.set_num_threads(min(os.cpu_count() or 1, 16))
+            ref = orc.prefill_reference(qc, kc, vc, causal=True, head_chunk=h)
+            best = float("inf")
+            for _ in range(3):
+                t0 = time.perf_counter()
+                ref = orc.prefill_reference(qc, kc, vc, causal=True, head_chunk=h)
+                best = min(best, time.perf_counter() - t0)
+            err = (holder["out"].float().cpu() - ref).abs()
+            res["cpu_baseline"] = {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                                   "kind": "port", "seconds_per_pass": best,
+                                   "sample": "whole shape, 1 warm-up + best of 3 passes of oracle prefill_reference, "
+                                             "torch CPU fp32, causal-convention FLOPs"}
+            res["parity"] = {"max_abs_err": float(err.max()),
+                             "within_2e-2_abs_1e-2_rel": bool((err <= 2e-2 + 1e-2 * ref.abs()).all())}
+        out[name] = res
+    return out
 
 
 def bench_prefill_few_sequences(args):
@@ -576,14 +645,87 @@ def cpu_prefill(case, gpu_out, cfg, n_heads=8):
     return base, parity
 
 
+LINE_BUDGET = 7000        # characters of the printed line
+PREFILL_TAIL = 1800       # the `prefill` object must sit inside this many last characters
+
+
+def _sig(x, digits=5):
+    """Floats cut to `digits` significant digits (the line is read by people and kept short); the rest unchanged."""
+    if isinstance(x, float):
+        return float(f"{x:.{digits}g}")
+    if isinstance(x, dict):
+        return {k: _sig(v, digits) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [_sig(v, digits) for v in x]
+    return x
+
+
+def _short_cpu(c):
+    return None if c is None else {k: c[k] for k in ("value", "unit", "cores", "kind", "sample") if k in c}
+
+
+def _leg(o):
+    """One auxiliary leg as {ms, frac[, cpu]}: device time per launch and the fraction of its roofline."""
+    r = o.get("roofline", {})
+    d = {"ms": r.get("device_ms", o.get("ms_per_step")), "frac": r.get("frac"), "bound": r.get("bound")}
+    if "kv_splits" in o and o["kv_splits"] != 1:
+        d["kv_splits"] = o["kv_splits"]
+    if "cpu_baseline" in o:
+        c = o["cpu_baseline"]
+        d["cpu"] = {"value": c["value"], "unit": c["unit"], "cores": c["cores"]}
+        d["parity_ok"] = o.get("parity", {}).get("within_2e-2_abs_1e-2_rel")
+    return d
+
+
+def compact_line(full):
+    """The printed form of the line: headline fields untouched (floats shortened), auxiliary legs as {ms, frac}
+    under "legs", the configs[2] prefill object last and whole (value, ms_per_step, roofline, cpu_baseline, parity)."""
+    out = {}
+    groups = ("prefill_few_sequences", "prefill_small_shapes", "cache_producers", "layer_ops", "decode_few_sequences")
+    tail_keys = ("decode_fp8", "prefill")
+    for k, v in full.items():
+        if k in groups or k in tail_keys or k in ("prefill_backward", "decode_loop", "config0"):
+            continue
+        out[k] = v
+    if "cpu_baseline" in out:
+        out["cpu_baseline"] = _short_cpu(out["cpu_baseline"])
+    legs = {}
+    for gname in groups:
+        for name, o in full.get(gname, {}).items():
+            legs[name] = _leg(o)
+    if "prefill_backward" in full:
+        legs["prefill_backward_cfg2"] = _leg(full["prefill_backward"])
+    if "decode_loop" in full:
+        dl = full["decode_loop"]
+        legs["decode_loop_sample_model"] = {"eager_ms": dl["eager"]["ms_per_step"], "hip_graph_ms": dl["hip_graph"]["ms_per_step"]}
+    if "config0" in full:
+        c0 = full["config0"]
+        legs["config0"] = {"cpu": {"value": c0["cpu_baseline"]["value"], "unit": c0["cpu_baseline"]["unit"],
+                                   "cores": c0["cpu_baseline"]["cores"]},
+                           "gpu_ms": c0["gpu"]["device_ms"], "parity_ok": c0["parity"]["within_2e-2_abs_1e-2_rel"]}
+    if legs:
+        out["legs"] = legs
+    for k in tail_keys:
+        if k in full:
+            o = dict(full[k])
+            if "cpu_baseline" in o:
+                o["cpu_baseline"] = _short_cpu(o["cpu_baseline"])
+            o.pop("algorithmic_bytes", None)
+            out[k] = o
+    return {k: (v if isinstance(v, float) else _sig(v)) for k, v in out.items()}     # headline floats stay exact
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--only", choices=["decode", "prefill", "few", "fp8", "backward", "producers", "layer", "loop"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "small", "few", "fp8", "backward", "producers", "layer", "loop"],
+                    default=None)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--full", action="store_true", help="print every leg's whole object (a line of about 10 KB)")
+    ap.add_argument("--detail", default=None, metavar="PATH", help="also write the verbose form to this file")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the 1 GiB plain copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
@@ -635,12 +777,13 @@ def main():
         pre["config"] = {"workload": "configs[2]: causal prefill forward, bf16, packed varlen, batch 8, 32 q / 8 kv "
                                      "heads, head_dim 128, seq 4096, seed %d" % args.seed}
         pre["dtype"] = "bf16"
-        line["prefill"] = pre
         if args.only == "prefill":
             line.update({"value": pre["value"], "unit": "TFLOP/s", "ms_per_step": pre["ms_per_step"], "dtype": "bf16",
                          "config": pre["config"], "roofline": pre["roofline"]})
     if args.only in (None, "few"):
         line["prefill_few_sequences"] = bench_prefill_few_sequences(args)
+    if args.only in (None, "small"):
+        line["prefill_small_shapes"] = bench_prefill_small(args, with_cpu)
     if args.only in (None, "backward"):
         line["prefill_backward"] = bench_prefill_backward(2, args)
     if args.only in (None, "fp8"):
@@ -675,7 +818,12 @@ def main():
                 line["cpu_baseline"] = f8["cpu_baseline"]
         if args.only in (None, "decode"):
             line["config0"] = cpu_config0(args)
-    print(json.dumps(line))
+    if pre is not None:
+        line["prefill"] = pre                     # last key of the line: the other half of the metric
+    if args.detail:
+        with open(args.detail, "w") as f:
+            json.dump(line, f, indent=1)
+    print(json.dumps(line if args.full else compact_line(line)))
 
 
 if __name__ == "__main__":

@@ -283,8 +283,9 @@ int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, float* scale,
  * decode step produces them).  Slots outside [0, 16*num_blocks) are skipped.  Needs 16-byte
  * aligned tensors, token strides that are multiples of 8, D in {32, 64, 128}.  k_out (optional)
  * receives the rotated keys in bf16, packed (T,Hkv,D), as in mi355_rope_and_cache: a prefill over
- * the tokens of this call then attends to unquantised keys.  No reference counterpart (the reference
- * has no KV cache).
+ * the tokens of this call then attends to unquantised keys; unlike there it must NOT overlap k_in
+ * (MI355_EINVAL): here the keys are read a second time, by other workgroups of the same launch, for
+ * the quantised write.  No reference counterpart (the reference has no KV cache).
  */
 int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, const void* v_in, void* q_out,
                              void* k_cache_fp8, void* v_cache_fp8, float* k_scale, float* v_scale,

@@ -65,11 +65,9 @@ Register map (physical, fixed; the block loads them itself from its operands, se
   s40 / s41 bytes from one tile to the next in K / V, s42 "a row sum reached 2"; every other scalar is a named operand
 """
 import os
+import sys
 
-# timing experiments only (results wrong): nobarrier, nodma, nocheck, noexp, novalu, nosum, nofma
-ABL = os.environ.get("W64_ABL", "").split(",")
-
-EXP = "v_mov_b32" if "noexp" in ABL else "v_exp_f32"
+EXP = "v_exp_f32"
 S = {("A", 0): 0, ("B", 0): 16, ("A", 1): 32, ("B", 1): 48}
 P = {0: {"A": 64, "B": 72}, 1: {"A": 80, "B": 88}}          # + 4 * slice inside the half
 KF = 200                            # AGPRs: LDS reads land there directly, the MFMAs take them as A operands
@@ -148,8 +146,6 @@ def mfma_o(c, j, p):
 
 
 def mfma_sum(c, p):
-    if "nosum" in ABL:
-        return "s_nop 0"
     acc = LREG[c]
     return f"v_mfma_f32_16x16x32_bf16 a{rng(acc, 4)}, v{rng(SUMA, 4)}, v{rng(p, 4)}, a{rng(acc, 4)}"
 
@@ -175,8 +171,6 @@ def exp_ops(h, mask, blocks="AB"):
     may not feed the next vector instruction, so the packing of a pair trails its exponentials.  Accumulator register
     i of a lane holds key 32h + 8(i/4) + 4(lane/32) + i%4 of the tile; where mask[c] is set the score is kept only if
     that index is <= the lane's threshold (the lane part of the index is folded into the threshold)."""
-    if "novalu" in ABL:
-        return []
     ops, pend = [], []
     i = 0
     for c in blocks:
@@ -184,17 +178,12 @@ def exp_ops(h, mask, blocks="AB"):
         for w in range(8):                      # packed word w of the block: accumulator registers 2w, 2w+1
             t0, t1 = ETMP[2 * (i % 4)], ETMP[2 * (i % 4) + 1]
             for tmp, r in ((t0, 2 * w), (t1, 2 * w + 1)):
-                if "nofma" not in ABL or mask[c]:
-                    ops.append(f"v_fma_f32 {tmp}, v{S[(c, h)] + r}, %[scale], v{NB[c]}")
+                ops.append(f"v_fma_f32 {tmp}, v{S[(c, h)] + r}, %[scale], v{NB[c]}")
                 if mask[c]:
                     ops.append(f"v_cmp_le_i32_e64 vcc, {32 * h + 8 * (r // 4) + r % 4}, v{THR[c]}")
                     ops.append(f"v_cndmask_b32 {tmp}, v{NEGINF}, {tmp}, vcc")
-            if "nofma" in ABL and not mask[c]:
-                ops.append(f"{EXP} {t0}, v{S[(c, h)] + 2 * w}")
-                ops.append(f"{EXP} {t1}, v{S[(c, h)] + 2 * w + 1}")
-            else:
-                ops.append(f"{EXP} {t0}, {t0}")
-                ops.append(f"{EXP} {t1}, {t1}")
+            ops.append(f"{EXP} {t0}, {t0}")
+            ops.append(f"{EXP} {t1}, {t1}")
             ops += pend
             pend = [f"v_cvt_pk_bf16_f32 v{dst + w}, {t0}, {t1}"]
             i += 1
@@ -288,8 +277,7 @@ def check_sums(e, flagged_label):
     e.raw(f"v_max_f32 {t[0]}, {t[0]}, {t[3]}")
     e.raw(f"v_cmp_nlt_f32_e64 vcc, {t[0]}, 2.0")
     e.raw("s_nop 1")
-    if "nocheck" not in ABL:
-        e.raw(f"s_cbranch_vccnz {flagged_label}")
+    e.raw(f"s_cbranch_vccnz {flagged_label}")
 
 
 def dma_chunks(which, buf):
@@ -302,8 +290,7 @@ def dma_chunks(which, buf):
             continue
         for j in range(4):
             c = [f"s_add_u32 m0, %[ldsdst], {lds0 + j * 1024}", "s_nop 0"]
-            if "nodma" not in ABL:
-                c.append(f"global_load_lds_dwordx4 v{DMAOFF + j0 + j}, s[{ptr}:{ptr + 1}]")
+            c.append(f"global_load_lds_dwordx4 v{DMAOFF + j0 + j}, s[{ptr}:{ptr + 1}]")
             chunks.append(c)
         chunks.append([f"s_add_u32 s{ptr}, s{ptr}, s{step}", f"s_addc_u32 s{ptr + 1}, s{ptr + 1}, 0"])
     return chunks
@@ -315,8 +302,7 @@ def wait_and_meet(e):
     e.raw("; boundary")
     e.drain()
     e.raw("s_waitcnt vmcnt(0)")
-    if "nobarrier" not in ABL:
-        e.raw("s_barrier")
+    e.raw("s_barrier")
 
 
 def boundary_plain(e, buf, tag, after):
@@ -755,10 +741,12 @@ def as_macro(name, lines):
     return f"#define {name} \\\n{body}\n\n"
 
 
-def main():
+def main(out_path=None):
+    """Writes the include file next to this script, or to `out_path` (first command-line argument)."""
     here = os.path.dirname(os.path.abspath(__file__))
+    out_path = out_path or os.path.join(here, "prefill_w64_asm.inc")
     lines = generate()
-    with open(os.path.join(here, "prefill_w64_asm.inc"), "w") as f:
+    with open(out_path, "w") as f:
         f.write(HEADER)
         f.write(as_macro("W64_LOOP", lines))
         for name, body in snippets().items():
@@ -767,8 +755,8 @@ def main():
         f.write(f"#define W64_CLOBBER_ACC {acc}\n")
         f.write("#define W64_CLOBBER_LOOP_VGPRS " + ", ".join('"v%d"' % i for i in range(N_FIXED_VGPRS)) + "\n")
     n_mfma = sum(1 for l in lines if l.startswith("v_mfma"))
-    print(f"wrote prefill_w64_asm.inc: loop of {len(lines)} lines, {n_mfma} MFMAs")
+    print(f"wrote {out_path}: loop of {len(lines)} lines, {n_mfma} MFMAs")
 
 
 if __name__ == "__main__":
-    main()
+    main(sys.argv[1] if len(sys.argv) > 1 else None)

@@ -464,6 +464,16 @@ extern "C" int mi355_rope_and_cache_fp8(const void* q_in, const void* k_in, cons
         !aligned16(k_in) || !aligned16(v_in) || !aligned16(q_out) || !aligned16(k_cache_fp8) || !aligned16(v_cache_fp8) ||
         !aligned16(freq_cache) || !aligned16(k_out) || (k_out && (k_out_token_stride & 7) != 0))
         return set_error(MI355_EINVAL, "rope_and_cache_fp8: tensors must be 16-byte aligned with token strides that are multiples of 8");
+    if (k_out && T > 0) {
+        // The packed rotated keys are written by the query workgroups while the key/value workgroups of the same
+        // launch read k_in, in no order: a k_out that shares memory with k_in would hand some of them rotated rows
+        // to rotate again.  (mi355_rope_and_cache reads and writes a row in one thread, so it may alias.)
+        const uintptr_t in_lo = reinterpret_cast<uintptr_t>(k_in), out_lo = reinterpret_cast<uintptr_t>(k_out);
+        const uintptr_t in_hi = in_lo + ((uintptr_t)(T - 1) * (uintptr_t)k_token_stride + (uintptr_t)Hkv * D) * 2;
+        const uintptr_t out_hi = out_lo + ((uintptr_t)(T - 1) * (uintptr_t)k_out_token_stride + (uintptr_t)Hkv * D) * 2;
+        if (in_lo < out_hi && out_lo < in_hi)
+            return set_error(MI355_EINVAL, "rope_and_cache_fp8: k_out must not overlap k_in (the keys are read again after k_out is written)");
+    }
     if (T == 0) return MI355_OK;
     hipStream_t s = (hipStream_t)stream;
     // queries (and, when asked for, the packed rotated keys): the body of the bf16 kernel, without a cache

@@ -569,6 +569,15 @@ def _packed_k_out(k_out, k):
     return k_out
 
 
+def _overlap(a, b):
+    """Do the memory spans of two (tokens, heads, d_head) tensors with contiguous heads intersect?"""
+    def span(t):
+        lo = t.data_ptr()
+        return lo, lo + ((t.shape[0] - 1) * t.stride(0) + t.shape[1] * t.shape[2]) * t.element_size()
+    (a0, a1), (b0, b1) = span(a), span(b)
+    return a0 < b1 and b0 < a1
+
+
 def rope_and_cache(q, k, v, positions, freq_cache, k_cache=None, v_cache=None, slot_mapping=None, *, out=None,
                    k_out=None):
     """RoPE on q and k (interleaved pairs, llm-core/llm_core/model.py:93-104) and scatter of the
@@ -630,7 +639,8 @@ def rope_and_cache_fp8(q, k, v, positions, freq_cache, k_cache, v_cache, k_scale
     kept equal to absmax/448 of its valid rows; rows already in a block are re-expressed when new rows
     raise the scale.  Tokens that share a block must be adjacent with consecutive slots, one such run
     per block and call (what a prefill or a decode step produces).  Returns the rotated q, or, with
-    `k_out` (True or a tensor to fill), (rotated q, rotated keys in bf16, packed (T,Hkv,D))."""
+    `k_out` (True or a tensor to fill; not k itself or a view of it -- unlike in rope_and_cache the keys are read
+    again, by other workgroups, after k_out is written), (rotated q, rotated keys in bf16, packed (T,Hkv,D))."""
     for n, t in (("q", q), ("k", k), ("v", v)):
         _require_gpu_bf16(n, t)
         if t.dim() != 3 or t.stride(2) != 1 or t.stride(1) != t.shape[2]:
@@ -668,6 +678,8 @@ def rope_and_cache_fp8(q, k, v, positions, freq_cache, k_cache, v_cache, k_scale
                 or q_out.data_ptr() % 16 != 0:
             raise ValueError("out must have q's shape with contiguous heads, 16-byte aligned")
     k_rot = _packed_k_out(k_out, k)
+    if k_rot is not None and T and _overlap(k_rot, k):
+        raise ValueError("k_out must not share memory with k (the fp8 write reads the keys again after k_out is written)")
     if T == 0:
         return q_out if k_rot is None else (q_out, k_rot)
     with _on(q, k, v, q_out, freq_cache, positions, slot_mapping, k_cache, v_cache, k_scale, v_scale, k_rot) as stream:

@@ -168,6 +168,23 @@ def test_decode_rejects_bad_arguments_without_a_gpu(lib):
     assert call(max_ctx=100000, ws_bytes=16) == -2 and b"workspace" in lib.mi355_last_error()
 
 
+def test_fp8_cache_write_rejects_a_k_out_that_overlaps_k_in(lib):
+    """The fp8 cache write reads the keys twice (query workgroups emit k_out, key/value workgroups quantise): k_out on
+    top of k_in would hand rotated rows to the second reader.  The argument check refuses it before any launch."""
+    buf = (C.c_char * 8192)()
+    base = (C.addressof(buf) + 15) & ~15
+
+    def call(k_in, k_out, T=4, Hkv=2, D=32, k_stride=64, ko_stride=64):
+        return lib.mi355_rope_and_cache_fp8(base, k_in, base, base, base, base, base, base, base, base, base,
+                                            8, T, 2, Hkv, D, 16, 64, k_stride, 64, 64, k_out, ko_stride, None)
+
+    assert call(base, base) == -1 and b"overlap" in lib.mi355_last_error()
+    assert call(base, base + 3 * 128 + 96) == -1                   # last 32 bytes of k_in's last row
+    assert call(base + 496, base) == -1 and b"overlap" in lib.mi355_last_error()    # k_out's last 16 bytes reach into k_in
+    # the same pointers with no tokens: nothing is read, nothing to refuse
+    assert call(base, base, T=0) == 0
+
+
 def test_host_ops_validate_before_launch():
     q = torch.zeros(2, 4, 64, dtype=torch.bfloat16)
     kc = torch.zeros(8, 2, 16, 64, dtype=torch.bfloat16)
@@ -210,3 +227,19 @@ def test_workload_draws_match_the_configurations():
     from oracle import attention_oracle as orc
     assert torch.equal(c3, orc.draw_context_lens("uniform", 128, 512, 16384, 0))
     assert torch.equal(c4, orc.draw_context_lens("loguniform", 256, 128, 32768, 0))
+
+
+def test_committed_assembly_include_is_what_the_generator_writes(tmp_path):
+    """csrc/prefill_w64_asm.inc is generated text that every build rewrites: the committed copy must be the generator's
+    output byte for byte (a hand edit or a stale commit would otherwise be invisible), and the generator must take no
+    switches from the environment."""
+    import subprocess
+    import sys
+
+    csrc = os.path.join(ROOT, "llm-systems-from-scratch_amd", "csrc")
+    gen = os.path.join(csrc, "gen_prefill_w64_loop.py")
+    out = tmp_path / "w64.inc"
+    env = dict(os.environ, W64_ABL="nobarrier,nodma,nocheck,noexp,novalu,nosum,nofma")     # must have no effect
+    subprocess.run([sys.executable, gen, str(out)], check=True, capture_output=True, env=env)
+    assert out.read_bytes() == open(os.path.join(csrc, "prefill_w64_asm.inc"), "rb").read()
+    assert "environ" not in open(gen).read()
