@@ -172,6 +172,34 @@ int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* o
                       float softmax_scale, int mask_mode, int dtype, void* stream);
 
 /*
+ * The training pair for an explicit mask: what autograd needs behind
+ * scaled_dot_product_attention(Q, K, V, mask) of model.py:308-325 as the reference's non-flash
+ * branch calls it (model.py:384-385, under loss.backward() at train.py:224).
+ * mi355_prefill_fwd_mask_lse is mi355_prefill_fwd in mode MI355_MASK_BOOL (dense layout only) that
+ * also writes lse (layout as in mi355_prefill_fwd_lse; a row whose keys are all masked gets -inf
+ * and a NaN output row, as the reference's softmax gives it).  mi355_prefill_bwd_mask is
+ * mi355_prefill_bwd under the same mask: every tile takes the per-element select and fetches its
+ * mask bytes, so it is the general path, slower than the causal one.  For the backward the mask
+ * pointer and its three byte strides must be multiples of 4 (keys are fetched four at a time), and a
+ * row must be readable up to the next multiple of 4 past Sk.  A fully masked row contributes zero
+ * gradients (the reference propagates its NaN instead).
+ */
+int mi355_prefill_fwd_mask_lse(const void* q, const void* k, const void* v, void* out, float* lse,
+                               const int64_t q_strides[3], const int64_t k_strides[3],
+                               const int64_t v_strides[3], const int64_t o_strides[3],
+                               const int64_t lse_strides[2], const uint8_t* mask,
+                               const int64_t mask_strides[3], int B, int Hq, int Hkv, int Sq, int Sk, int D,
+                               float softmax_scale, int dtype, void* stream);
+int mi355_prefill_bwd_mask(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                           const float* lse, float* delta, void* dq, void* dk, void* dv,
+                           const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                           const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
+                           const int64_t dk_strides[3], const int64_t dv_strides[3],
+                           const int64_t lse_strides[2], const uint8_t* mask, const int64_t mask_strides[3],
+                           int B, int Hq, int Hkv, int Sq, int Sk, int D, float softmax_scale, int dtype,
+                           void* stream);
+
+/*
  * Paged-KV decode attention, one query token per sequence (split-K + combine).
  *
  * No counterpart exists in the reference: it is what a KV-cached replacement of

@@ -82,6 +82,78 @@ def check_w64_registers() -> str:
     return "prefill_fwd_w64.hip: no compiler-generated instruction touches a[0:%d]" % (n_agprs - 1)
 
 
+_SREG = re.compile(r"\bs\[(\d+):(\d+)\]|\bs(\d+)\b")
+
+
+def _sregs(text):
+    out = set()
+    for m in _SREG.finditer(text):
+        if m.group(3) is not None:
+            out.add(int(m.group(3)))
+        else:
+            out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+    return out
+
+
+def check_scalar_address_hazards(src: str) -> str:
+    """gfx9 wants five wait states between a VECTOR instruction that writes a scalar register (v_readlane restoring a
+    spilled value, v_readfirstlane, a compare or a carry-out) and a vector-memory instruction that reads that register
+    as its address.  The compiler inserts them for the instructions it emits, but it cannot see inside an
+    inline-assembly statement, and the direct-to-LDS loads of these kernels live in such statements.  This compiles
+    `src` to assembly and fails the build if a memory instruction inside a statement reads a scalar register that a
+    vector instruction wrote fewer than five wait states earlier on the straight-line path in front of it."""
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, "k.s")
+        _run([HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", asm])
+        lines = open(asm).read().splitlines()
+    bad, inside, n_checked = [], False, 0
+    code = []                     # (line number, text) of instructions, in order
+    for no, raw in enumerate(lines, 1):
+        text = raw.split(";")[0].strip()
+        if "#ASMSTART" in raw:
+            inside = True
+            continue
+        if "#ASMEND" in raw:
+            inside = False
+            continue
+        if not text or text.startswith(".") or text.endswith(":"):
+            continue
+        code.append((no, text, inside))
+    for i, (no, text, in_asm) in enumerate(code):
+        op = text.split()[0]
+        if not in_asm or not op.startswith(("global_", "buffer_", "flat_", "scratch_")):
+            continue
+        addr = _sregs(text)
+        if not addr:
+            continue
+        n_checked += 1
+        states, j = 0, i - 1
+        while j >= 0 and states < 5:
+            _, prev, _ = code[j]
+            pop = prev.split()[0]
+            if pop == "s_nop":
+                states += int(prev.split()[1], 0) + 1
+            else:
+                # destination operands of a vector instruction: everything in front of the first source; an SGPR
+                # there (v_readlane sN, v_cmp_* s[a:b], the carry-out of v_mad_u64_u32 / v_add_co) is a vector write
+                if pop.startswith("v_"):
+                    ops = prev[len(pop):].split(",")
+                    n_dst = 2 if pop.startswith(("v_mad_u64", "v_mad_i64", "v_add_co", "v_sub_co", "v_addc", "v_subb",
+                                                  "v_div_scale")) else 1
+                    written = set()
+                    for o in ops[:n_dst]:
+                        written |= _sregs(o)
+                    if written & addr:
+                        bad.append("%s:%d: `%s` reads s%s, written %d wait state(s) earlier by `%s`"
+                                   % (src, no, text, sorted(written & addr), states, prev))
+                        break
+                states += 1
+            j -= 1
+    if bad:
+        raise RuntimeError("scalar address hazard in inline assembly:\n" + "\n".join(bad[:20]))
+    return "%s: %d inline-assembly memory instructions, none reads a scalar register within five wait states of a vector write" % (src, n_checked)
+
+
 def build_library(verbose: bool = True) -> str:
     # the hand-scheduled assembly of prefill_fwd_w64.hip is generated text: regenerate it so that it cannot go stale
     _run([sys.executable, os.path.join(CSRC, "gen_prefill_w64_loop.py")])
@@ -94,12 +166,15 @@ def build_library(verbose: bool = True) -> str:
         log = _run([HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj])
         return obj, log
 
+    # sources whose kernels issue memory instructions from inline assembly
+    asm_dma = [s for s in ("prefill_fwd.hip", "prefill_fwd_w64.hip", "prefill_bwd.hip") if s in srcs]
     with ThreadPoolExecutor(max_workers=4) as ex:
         check = ex.submit(check_w64_registers)
+        hazards = [ex.submit(check_scalar_address_hazards, s) for s in asm_dma]
         results = list(ex.map(compile_one, srcs))
-        note = check.result()
+        notes = [check.result()] + [h.result() for h in hazards]
     if verbose:
-        print(note)
+        print("\n".join(notes))
     for _, log in results:
         if verbose and log.strip():
             print(log)

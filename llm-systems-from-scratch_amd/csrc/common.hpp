@@ -125,11 +125,14 @@ __device__ __forceinline__ float xor32_sum(float v) {
 // gbase: wave-uniform global base address; voff: this lane's byte offset from it (unsigned,
 // < 2^32); lds_addr: wave-uniform LDS byte address the wavefront's 1 KiB lands at.
 // The LDS address travels in m0 as a declared register operand: the compiler writes m0 itself and knows
-// that this statement reads it, so its own uses of m0 elsewhere in a kernel stay correct.  (The leading
-// s_nop covers the wait state the hardware wants between a write of m0 and an LDS-DMA instruction; the
-// compiler cannot see the instruction inside the statement and would not insert it.)
+// that this statement reads it, so its own uses of m0 elsewhere in a kernel stay correct.  The leading
+// s_nop 4 covers two wait-state rules that the compiler cannot apply to an instruction it does not see: one
+// state between a write of m0 and an LDS-DMA instruction, and FIVE between a vector instruction that writes a
+// scalar register and a vector-memory instruction that reads it as its address -- which is what happens when
+// the compiler keeps `gbase` in a spilled scalar register and restores it (v_readlane) directly in front of the
+// statement.  (With one state only, a kernel variant with scalar spills fetched from a stale base address.)
 __device__ __forceinline__ void dma_to_lds_16(const void* gbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voff), "s"(gbase), "{m0}"(lds_addr)
                  : "memory");

@@ -64,7 +64,9 @@ struct DecodeLds {
     static constexpr int kVBytes = kStage * kVRow;           // per-wavefront V tile
     static constexpr int kKRow = FP8 ? D : D * 2;            // bytes per staged K row (raw cache bytes, swizzled)
     static constexpr int kKBytes = kStage * kKRow;           // per-wavefront K tile
-    static constexpr int kPartFloats = 16 * D + 32;          // per-wavefront (O, m, l)
+    static constexpr int kPartRow = D + 4;                   // floats per row of a wavefront's partial O: the padding puts the
+                                                             // 16-byte pieces that 16 lanes write together into 16 bank groups
+    static constexpr int kPartFloats = 16 * kPartRow + 32;   // per-wavefront (O, m, l)
     static constexpr int kTiles = kVBytes + kKBytes;
     static constexpr int kWaveBytes = kTiles > kPartFloats * 4 ? kTiles : kPartFloats * 4;
 };
@@ -86,6 +88,7 @@ void paged_decode_split_kernel(DecodeParams p) {
     constexpr int kKChunks = kKRow / 16;              // 16-byte chunks per staged K row
     constexpr int kKRowsPer256 = 256 / kKRow > 0 ? 256 / kKRow : 1;
     constexpr int kWaveBytes = DecodeLds<D, FP8>::kWaveBytes;
+    constexpr int kPartRow = DecodeLds<D, FP8>::kPartRow;
     static_assert(!FP8 || D >= 64, "fp8 KV needs head_dim >= 64");
 
     __shared__ __attribute__((aligned(16))) unsigned char smem[kDecodeWaves * kWaveBytes];
@@ -366,14 +369,14 @@ void paged_decode_split_kernel(DecodeParams p) {
     // ---- merge the four wavefronts ------------------------------------------
     l_run = xor_sum_16_32(l_run);
     {
+        // (one 16-byte write per d-tile; with unpadded rows of D floats the sixteen lanes of a query column group
+        // all wrote the same bank: a third of this kernel's LDS time on short streams)
         float* part = reinterpret_cast<float*>(wsm);
 #pragma unroll
-        for (int dt = 0; dt < NT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) part[r * D + 16 * dt + 4 * kg + i] = o[dt][i];
+        for (int dt = 0; dt < NT; ++dt) *reinterpret_cast<f32x4*>(part + r * kPartRow + 16 * dt + 4 * kg) = o[dt];
         if (kg == 0) {
-            part[16 * D + r] = m_run;
-            part[16 * D + 16 + r] = l_run;
+            part[16 * kPartRow + r] = m_run;
+            part[16 * kPartRow + 16 + r] = l_run;
         }
     }
     __syncthreads();
@@ -385,7 +388,7 @@ void paged_decode_split_kernel(DecodeParams p) {
         float M = -INFINITY;
 #pragma unroll
         for (int w = 0; w < kDecodeWaves; ++w) {
-            mw[w] = reinterpret_cast<const float*>(smem + w * kWaveBytes)[16 * D + qi];
+            mw[w] = reinterpret_cast<const float*>(smem + w * kWaveBytes)[16 * kPartRow + qi];
             M = fmaxf(M, mw[w]);
         }
         float num = 0.f, den = 0.f;
@@ -393,8 +396,8 @@ void paged_decode_split_kernel(DecodeParams p) {
         for (int w = 0; w < kDecodeWaves; ++w) {
             const float* part = reinterpret_cast<const float*>(smem + w * kWaveBytes);
             const float f = fast_exp2(mw[w] - M);       // a wavefront without keys has m = -inf -> 0
-            num += f * part[qi * D + d];
-            den += f * part[16 * D + 16 + qi];
+            num += f * part[qi * kPartRow + d];
+            den += f * part[16 * kPartRow + 16 + qi];
         }
         const int64_t row = (int64_t)b * p.Hq + h0 + qi;
         if (n_chunks == 1) {

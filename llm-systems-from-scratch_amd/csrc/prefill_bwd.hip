@@ -16,6 +16,10 @@
 // (dQ^T += K^T dS^T; dV^T += dO^T P, dK^T += Q^T dS), and the matching A operand is a transposed
 // LDS read (ds_read_b64_tr_b16) of the streamed tile with the same row permutation.
 // 7 GEMM-sized products are executed (S and dP in both kernels) where 5 are needed.
+//
+// Masks: none, causal (bottom-right aligned, as in the forward), or an explicit boolean keep-mask (the mask argument
+// of llm-core/llm_core/model.py:308-325, which its non-flash branch passes at model.py:384-385).  The explicit mask is
+// the general, slower path: every tile takes the per-element select and reads its mask bytes from global memory.
 #include <type_traits>
 
 #include "common.hpp"
@@ -43,6 +47,8 @@ struct BwdParams {
     int64_t ls[2];                                                          // lse / delta: batch, head strides
     const int32_t* cu_q;
     const int32_t* cu_k;
+    const uint8_t* mask;          // MI355_MASK_BOOL: (B, Hq, Sq, Sk) bytes, non-zero = keep; rows 4-byte aligned
+    int64_t ms[3];                // batch, head, row strides of the mask in bytes (0 = broadcast), multiples of 4
     int B, Hq, Hkv, Sq, Sk;
     float scale, scale_log2;
     int n_qtiles, n_ktiles;
@@ -100,8 +106,9 @@ struct TileReads {
 // ---------------------------------------------------------------------------------------------
 // dQ: one workgroup per tile of 128 queries of one (batch, query head); K/V stream through LDS.
 // Per wavefront: Q and dO fragments of its 32 query columns in registers (64), dQ^T accumulators (64).
-template <int D, bool CAUSAL>
+template <int D, int MODE>
 __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
+    constexpr bool CAUSAL = MODE == MI355_MASK_CAUSAL, BOOLM = MODE == MI355_MASK_BOOL;
     constexpr int NWV = kBwWaves;
     using R = TileReads<D>;
     constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
@@ -210,6 +217,11 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
         const int n_tiles = (kv_end + kBwRows - 1) / kBwRows;
         const int last_key = CAUSAL ? min(sk - 1, qi + coff) : sk - 1;      // last key this lane's query sees
         const int wave_last_key = CAUSAL ? min(sk - 1, qw0 + coff) : sk - 1;   // ... and the last one ALL queries of the wavefront see
+        // explicit mask: the row of this lane's query (a padded lane re-reads the last row; its lse keeps P at 0);
+        // four keys at a time as one 32-bit word (rows are 4-byte aligned; a word past the last key is the last word)
+        const uint8_t* mrow = nullptr;
+        if constexpr (BOOLM) mrow = p.mask + (int64_t)b * p.ms[0] + (int64_t)h * p.ms[1] + (int64_t)min(qi, sq - 1) * p.ms[2];
+        const int last_word = (sk - 1) & ~3;
         const auto issue = [&](int tile) {
             const int r0 = tile * kBwRows, buf = (tile & 1) * kTile;
             ld.issue(p.k + k_base + (int64_t)r0 * p.ks[2], (int)p.ks[2], sk - 1 - r0, dst + buf);
@@ -240,6 +252,12 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
             const unsigned char* v_lds = k_lds + 2 * kTile;
             const int key_lim = last_key - k0 - 4 * kg;      // element (t,i) is kept iff its tile-relative key index <= key_lim
             u32x4 ds[4];
+            uint32_t mw[8] = {};
+            if constexpr (BOOLM && MASKED) {
+#pragma unroll
+                for (int g = 0; g < 8; ++g)      // keys k0 + 32(g/4) + 8(g%4) + 4kg .. + 3
+                    mw[g] = *reinterpret_cast<const uint32_t*>(mrow + min(k0 + 32 * (g >> 2) + 8 * (g & 3) + 4 * kg, last_word));
+            }
             // one 32-key half at a time: element i of this lane is key k0 + 32t + 8(i/4) + 4kg + i%4, query qi
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
@@ -252,7 +270,9 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
                     x[i] = pr * dp_acc[i];                                             // dS (without the scale factor)
                     if constexpr (MASKED) {
                         // key index relative to the tile (compile-time part) against this lane's last visible key
-                        x[i] = (32 * t + 8 * (i >> 2) + (i & 3) <= key_lim) ? x[i] : 0.f;
+                        bool keep = 32 * t + 8 * (i >> 2) + (i & 3) <= key_lim;
+                        if constexpr (BOOLM) keep = keep & (((mw[4 * t + (i >> 2)] >> (8 * (i & 3))) & 0xffu) != 0u);
+                        x[i] = keep ? x[i] : 0.f;
                     }
                 }
 #pragma unroll
@@ -282,7 +302,7 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
         // Two loops over the tile stream: first the tiles that every query of the wavefront sees in full, then
         // those that reach past wave_last_key (the diagonal, a ragged end), which run the instantiation with the
         // per-element compare/select.  (Two loops, not a branch in one: each loop body is scheduled on its own.)
-        const int n_full = min(n_tiles, max(0, wave_last_key + 1) / kBwRows);
+        const int n_full = BOOLM ? 0 : min(n_tiles, max(0, wave_last_key + 1) / kBwRows);
         if (n_tiles > 0) issue(0);
         for (int tile = 0; tile < n_full; ++tile) {
             wait_vmcnt<0>();                                   // this wavefront's share of tile `tile` has landed
@@ -330,8 +350,9 @@ __global__ __launch_bounds__(kBwWaves * 64, 1) void bwd_dq_kernel(BwdParams p) {
 constexpr int kFuPairs = 4;
 constexpr int kFuCols = 32 * kFuPairs;
 
-template <int D, bool CAUSAL>
+template <int D, int MODE>
 __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams p) {
+    constexpr bool CAUSAL = MODE == MI355_MASK_CAUSAL, BOOLM = MODE == MI355_MASK_BOOL;
     constexpr int NWV = 2 * kFuPairs;
     using R = TileReads<D>;
     constexpr int NS = R::NS, NDT = R::NDT, kRow = R::kRow, kTile = kBwRows * kRow;
@@ -518,6 +539,15 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             const float* lse_lds = lse_lds2 + (st & 1) * kBwRows;
             unsigned char* out = p_lds + (st & 1) * (kFuPairs * kPSlab);
             const int row_lim = CAUSAL ? kj - coff - ps.r0 - 4 * kg : -1;
+            // explicit mask: the bytes (row, this lane's key) of the step's 64 rows (a row or key past the end re-reads
+            // the last one: its P is 0 through lse = inf, or its column is never stored)
+            uint8_t mb[32] = {};
+            if constexpr (BOOLM && MASKED) {
+                const uint8_t* mcol = p.mask + (int64_t)b * p.ms[0] + (int64_t)(hk * G + ps.hq) * p.ms[1] + min(kj, sk - 1);
+#pragma unroll
+                for (int e = 0; e < 32; ++e)     // row r0 + 32(e/16) + 8((e/4)%4) + 4kg + e%4
+                    mb[e] = mcol[(int64_t)min(ps.r0 + 32 * (e >> 4) + 8 * ((e >> 2) & 3) + 4 * kg + (e & 3), sq - 1) * p.ms[2]];
+            }
             // one 32-row half at a time: element i of this lane is query row r0 + 32t + 8(i/4) + 4kg + i%4, key kj
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
@@ -530,7 +560,11 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
                     for (int r = 0; r < 4; ++r) {
                         float x = fast_exp2(fmaf(s_acc[4 * j + r], p.scale_log2, -l4[r]));
                         // kept iff kj <= row + coff, i.e. the tile-relative row (compile-time part) >= row_lim
-                        if constexpr (MASKED) x = (32 * t + 8 * j + r >= row_lim) ? x : 0.f;
+                        if constexpr (MASKED) {
+                            bool keep = 32 * t + 8 * j + r >= row_lim;
+                            if constexpr (BOOLM) keep = keep & (mb[16 * t + 4 * j + r] != 0);
+                            x = keep ? x : 0.f;
+                        }
                         x4[r] = x;
                     }
                     *reinterpret_cast<f32x4*>(out + (4 * t + j) * 1024) = x4;
@@ -603,7 +637,7 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
             for (int i = -1; i < n_steps; ++i) {
                 open_iteration(i);
                 if (i >= 0 && !idle(ps0)) update(lds + (3 + (i & 1)) * kTile, p_cur);      // dV^T += dO(i)^T P(i)
-                if (i + 1 < n_steps && !idle(ps1)) make_p(std::integral_constant<bool, CAUSAL>{}, i + 1, ps1, s_a);
+                if (i + 1 < n_steps && !idle(ps1)) make_p(std::integral_constant<bool, CAUSAL || BOOLM>{}, i + 1, ps1, s_a);
                 close_iteration(i);
             }
         } else {
@@ -632,15 +666,18 @@ __global__ __launch_bounds__(2 * kFuPairs * 64, 1) void bwd_dkv_kernel(BwdParams
 }
 
 template <int D>
-static int launch_bwd(const BwdParams& p, bool causal, hipStream_t stream) {
+static int launch_bwd(const BwdParams& p, int mask_mode, hipStream_t stream) {
     const dim3 block(kBwWaves * 64), block_kv(2 * kFuPairs * 64);
     const dim3 grid_q((unsigned)((p.n_qtiles + 1) / 2 * p.Hq * p.B)), grid_k((unsigned)((p.n_ktiles + 1) / 2 * p.Hkv * p.B));
-    if (causal) {
-        hipLaunchKernelGGL((bwd_dq_kernel<D, true>), grid_q, block, 0, stream, p);                // dQ, writes delta
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, true>), grid_k, block_kv, 0, stream, p);      // dK and dV, reads delta
+    if (mask_mode == MI355_MASK_CAUSAL) {
+        hipLaunchKernelGGL((bwd_dq_kernel<D, MI355_MASK_CAUSAL>), grid_q, block, 0, stream, p);        // dQ, writes delta
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, MI355_MASK_CAUSAL>), grid_k, block_kv, 0, stream, p);    // dK and dV, reads delta
+    } else if (mask_mode == MI355_MASK_BOOL) {
+        hipLaunchKernelGGL((bwd_dq_kernel<D, MI355_MASK_BOOL>), grid_q, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, MI355_MASK_BOOL>), grid_k, block_kv, 0, stream, p);
     } else {
-        hipLaunchKernelGGL((bwd_dq_kernel<D, false>), grid_q, block, 0, stream, p);
-        hipLaunchKernelGGL((bwd_dkv_kernel<D, false>), grid_k, block_kv, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dq_kernel<D, MI355_MASK_NONE>), grid_q, block, 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkv_kernel<D, MI355_MASK_NONE>), grid_k, block_kv, 0, stream, p);
     }
     return (int)hipGetLastError();
 }
@@ -649,14 +686,14 @@ static int launch_bwd(const BwdParams& p, bool causal, hipStream_t stream) {
 
 using namespace mi355;
 
-extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout,
-                                 const float* lse, float* delta, void* dq, void* dk, void* dv,
-                                 const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
-                                 const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
-                                 const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[2],
-                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int B, int Hq,
-                                 int Hkv, int Sq_max, int Sk_max, int D, float softmax_scale, int mask_mode, int dtype,
-                                 void* stream) {
+static int prefill_bwd_common(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                              const float* lse, float* delta, void* dq, void* dk, void* dv,
+                              const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                              const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
+                              const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[2],
+                              const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, const uint8_t* mask,
+                              const int64_t* mask_strides, int B, int Hq, int Hkv, int Sq_max, int Sk_max, int D,
+                              float softmax_scale, int mask_mode, int dtype, void* stream) {
     if (!q || !k || !v || !out || !dout || !lse || !delta || !dq || !dk || !dv)
         return set_error(MI355_EINVAL, "prefill_bwd: null pointer argument");
     if (!q_strides || !k_strides || !v_strides || !o_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides ||
@@ -669,8 +706,15 @@ extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, co
     if (!(D == 128 || D == 64 || D == 32)) return set_error(MI355_EINVAL, "prefill_bwd: head_dim must be 32, 64 or 128");
     if ((cu_seqlens_q == nullptr) != (cu_seqlens_k == nullptr))
         return set_error(MI355_EINVAL, "prefill_bwd: cu_seqlens_q and cu_seqlens_k must be given together");
-    if (mask_mode != MI355_MASK_NONE && mask_mode != MI355_MASK_CAUSAL)
-        return set_error(MI355_EINVAL, "prefill_bwd: mask_mode must be MI355_MASK_NONE or MI355_MASK_CAUSAL");
+    if (mask_mode < MI355_MASK_NONE || mask_mode > MI355_MASK_BOOL) return set_error(MI355_EINVAL, "prefill_bwd: unknown mask_mode");
+    if (mask_mode == MI355_MASK_BOOL) {
+        if (!mask || !mask_strides || cu_seqlens_q)
+            return set_error(MI355_EINVAL, "prefill_bwd: MI355_MASK_BOOL needs mask + mask_strides and the dense layout");
+        if (((uintptr_t)mask | (uintptr_t)mask_strides[0] | (uintptr_t)mask_strides[1] | (uintptr_t)mask_strides[2]) & 3)
+            return set_error(MI355_EINVAL, "prefill_bwd: the mask and its strides must be multiples of 4 bytes");
+        if (mask_strides[0] < 0 || mask_strides[1] < 0 || mask_strides[2] < 0)
+            return set_error(MI355_EINVAL, "prefill_bwd: mask strides must not be negative");
+    }
     const int64_t* all[8] = {q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides};
     for (const int64_t* st : all)
         for (int i = 0; i < 3; ++i)
@@ -708,6 +752,8 @@ extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, co
     p.ls[1] = lse_strides[1];
     p.cu_q = cu_seqlens_q;
     p.cu_k = cu_seqlens_k;
+    p.mask = mask_mode == MI355_MASK_BOOL ? mask : nullptr;
+    for (int i = 0; i < 3; ++i) p.ms[i] = mask_mode == MI355_MASK_BOOL ? mask_strides[i] : 0;
     p.B = B;
     p.Hq = Hq;
     p.Hkv = Hkv;
@@ -721,9 +767,36 @@ extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, co
         return set_error(MI355_EINVAL, "prefill_bwd: too many workgroups");
 
     hipStream_t s = (hipStream_t)stream;
-    const bool causal = mask_mode == MI355_MASK_CAUSAL;
-    int rc = D == 128 ? launch_bwd<128>(p, causal, s)
-                      : (D == 64 ? launch_bwd<64>(p, causal, s) : launch_bwd<32>(p, causal, s));
+    int rc = D == 128 ? launch_bwd<128>(p, mask_mode, s)
+                      : (D == 64 ? launch_bwd<64>(p, mask_mode, s) : launch_bwd<32>(p, mask_mode, s));
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;
+}
+
+extern "C" int mi355_prefill_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                                 const float* lse, float* delta, void* dq, void* dk, void* dv,
+                                 const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                                 const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
+                                 const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[2],
+                                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int B, int Hq,
+                                 int Hkv, int Sq_max, int Sk_max, int D, float softmax_scale, int mask_mode, int dtype,
+                                 void* stream) {
+    if (mask_mode == MI355_MASK_BOOL)
+        return set_error(MI355_EINVAL, "prefill_bwd: mask_mode must be MI355_MASK_NONE or MI355_MASK_CAUSAL (an explicit mask goes through mi355_prefill_bwd_mask)");
+    return prefill_bwd_common(q, k, v, out, dout, lse, delta, dq, dk, dv, q_strides, k_strides, v_strides, o_strides,
+                              do_strides, dq_strides, dk_strides, dv_strides, lse_strides, cu_seqlens_q, cu_seqlens_k,
+                              nullptr, nullptr, B, Hq, Hkv, Sq_max, Sk_max, D, softmax_scale, mask_mode, dtype, stream);
+}
+
+extern "C" int mi355_prefill_bwd_mask(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                                      const float* lse, float* delta, void* dq, void* dk, void* dv,
+                                      const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                                      const int64_t o_strides[3], const int64_t do_strides[3], const int64_t dq_strides[3],
+                                      const int64_t dk_strides[3], const int64_t dv_strides[3],
+                                      const int64_t lse_strides[2], const uint8_t* mask, const int64_t mask_strides[3],
+                                      int B, int Hq, int Hkv, int Sq, int Sk, int D, float softmax_scale, int dtype,
+                                      void* stream) {
+    return prefill_bwd_common(q, k, v, out, dout, lse, delta, dq, dk, dv, q_strides, k_strides, v_strides, o_strides,
+                              do_strides, dq_strides, dk_strides, dv_strides, lse_strides, nullptr, nullptr, mask,
+                              mask_strides, B, Hq, Hkv, Sq, Sk, D, softmax_scale, MI355_MASK_BOOL, dtype, stream);
 }

@@ -680,6 +680,17 @@ extern "C" int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v
                           stream);
 }
 
+extern "C" int mi355_prefill_fwd_mask_lse(const void* q, const void* k, const void* v, void* out, float* lse,
+                                          const int64_t q_strides[3], const int64_t k_strides[3],
+                                          const int64_t v_strides[3], const int64_t o_strides[3],
+                                          const int64_t lse_strides[2], const uint8_t* mask,
+                                          const int64_t mask_strides[3], int B, int Hq, int Hkv, int Sq, int Sk, int D,
+                                          float softmax_scale, int dtype, void* stream) {
+    if (!lse || !lse_strides) return set_error(MI355_EINVAL, "prefill_fwd_mask_lse: null lse argument");
+    return prefill_common(q, k, v, out, q_strides, k_strides, v_strides, o_strides, nullptr, nullptr, mask, mask_strides,
+                          B, Hq, Hkv, Sq, Sk, D, softmax_scale, MI355_MASK_BOOL, dtype, lse, lse_strides, stream);
+}
+
 extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
                                        int64_t q_token_stride, int64_t out_token_stride, const int32_t* cu_seqlens_q,
                                        const int32_t* block_tables, int64_t table_stride, const int32_t* context_lens,

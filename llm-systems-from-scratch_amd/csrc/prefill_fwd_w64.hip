@@ -121,8 +121,11 @@ constexpr int kWMaxSeqs = 4096;      // sequences of a packed batch
 // the compiler's idea of what m0 holds.  (m0 cannot be named in a clobber list -- the compiler treats it as reserved
 // and warns that clobbering it is undefined -- and it needs no naming: the compiler keeps nothing in m0 across
 // statements, it writes m0 directly in front of each of its own instructions that read it.)
+// The s_nop 3 makes five wait states between anything in front of the statement and the load: a scalar register
+// that a vector instruction wrote (v_readlane restoring a spilled `gbase`, v_readfirstlane) may be read as a
+// vector-memory address only five states later, and the compiler does not see the load inside the statement.
 __device__ __forceinline__ void dma_to_lds_16_m0(const void* gbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(voff), "s"(gbase), "s"(lds_addr)
                  : "memory");

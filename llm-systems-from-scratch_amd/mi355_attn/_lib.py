@@ -21,6 +21,8 @@ EXPORTS = (
     "mi355_prefill_fwd",
     "mi355_prefill_fwd_lse",
     "mi355_prefill_bwd",
+    "mi355_prefill_fwd_mask_lse",
+    "mi355_prefill_bwd_mask",
     "mi355_paged_decode_fwd",
     "mi355_paged_decode_fwd_static",
     "mi355_paged_decode_workspace_bytes",
@@ -64,6 +66,12 @@ def load():
     lib.mi355_prefill_bwd.restype = i32
     lib.mi355_prefill_bwd.argtypes = [vp] * 10 + [_i64x3] * 8 + [_i64x2, vp, vp,
                                                                  i32, i32, i32, i32, i32, i32, f32, i32, i32, vp]
+    lib.mi355_prefill_fwd_mask_lse.restype = i32
+    lib.mi355_prefill_fwd_mask_lse.argtypes = [vp, vp, vp, vp, vp, _i64x3, _i64x3, _i64x3, _i64x3, _i64x2, vp, _i64x3,
+                                               i32, i32, i32, i32, i32, i32, f32, i32, vp]
+    lib.mi355_prefill_bwd_mask.restype = i32
+    lib.mi355_prefill_bwd_mask.argtypes = [vp] * 10 + [_i64x3] * 8 + [_i64x2, vp, _i64x3,
+                                                                      i32, i32, i32, i32, i32, i32, f32, i32, vp]
     lib.mi355_prefill_paged_fwd.restype = i32
     lib.mi355_prefill_paged_fwd.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, i64, vp,
                                             i32, i32, i32, i32, i32, i32, i64, f32, i32, i32, i64, vp, sz, vp]

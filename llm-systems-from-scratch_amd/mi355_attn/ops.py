@@ -127,6 +127,15 @@ def _prefill(q, k, v, out, cu_q, cu_k, mask, B, Hq, Hkv, Sq, Sk, D, scale, mode,
                 workspace.data_ptr(), workspace.numel() * workspace.element_size(), stream)
         _lib.check(rc, "mi355_prefill_fwd_splitkv")
         return
+    if lse is not None and mask is not None:
+        qs, ks, vs, os_ = (x.stride()[:3] for x in (q, k, v, out))
+        with _on(q, k, v, out, lse, mask) as stream:
+            rc = lib.mi355_prefill_fwd_mask_lse(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_), _lib.strides2(lse.stride()[:2]),
+                mask.data_ptr(), _lib.strides3(mask.stride()[:3]), B, Hq, Hkv, Sq, Sk, D, float(scale), _lib.MI355_BF16, stream)
+        _lib.check(rc, "mi355_prefill_fwd_mask_lse")
+        return
     if lse is not None:
         packed = cu_q is not None
         qs, ks, vs, os_ = (_packed_or_dense_strides(x, packed) for x in (q, k, v, out))
@@ -189,8 +198,9 @@ def _grad_like(t):
     return g if ok else torch.empty(t.shape, dtype=t.dtype, device=t.device)
 
 
-def _prefill_backward(q, k, v, out, dout, lse, cu_q, cu_k, Sq, Sk, scale, mode):
-    """dq, dk, dv through mi355_prefill_bwd; tensors dense (B,H,S,D) or packed (T,H,D)."""
+def _prefill_backward(q, k, v, out, dout, lse, cu_q, cu_k, Sq, Sk, scale, mode, mask=None):
+    """dq, dk, dv through mi355_prefill_bwd (mi355_prefill_bwd_mask with an explicit (B,H,Sq,Sk) uint8 mask);
+    tensors dense (B,H,S,D) or packed (T,H,D)."""
     packed = cu_q is not None
     q, k, v, out, dout = (_rows16(n, t) for n, t in (("q", q), ("k", k), ("v", v), ("out", out), ("dout", dout)))
     dq, dk, dv = _grad_like(q), _grad_like(k), _grad_like(v)
@@ -204,6 +214,14 @@ def _prefill_backward(q, k, v, out, dout, lse, cu_q, cu_k, Sq, Sk, scale, mode):
         (B, Hq, _, D), Hkv = q.shape, k.shape[1]
         ls = lse.stride()[:2]
     st = [_lib.strides3(_packed_or_dense_strides(t, packed)) for t in (q, k, v, out, dout, dq, dk, dv)]
+    if mask is not None:
+        with _on(q, k, v, out, dout, lse, mask) as stream:
+            rc = _lib.load().mi355_prefill_bwd_mask(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), *st, _lib.strides2(ls), mask.data_ptr(),
+                _lib.strides3(mask.stride()[:3]), B, Hq, Hkv, int(Sq), int(Sk), D, float(scale), _lib.MI355_BF16, stream)
+        _lib.check(rc, "mi355_prefill_bwd_mask")
+        return dq, dk, dv
     with _on(q, k, v, out, dout, lse, cu_q, cu_k) as stream:
         rc = _lib.load().mi355_prefill_bwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
@@ -231,6 +249,38 @@ class _DensePrefillFn(torch.autograd.Function):
         q, k, v, out, lse = ctx.saved_tensors
         dq, dk, dv = _prefill_backward(q, k, v, out, dout, lse, None, None, q.shape[2], k.shape[2], ctx.scale, ctx.mode)
         return dq, dk, dv, None, None
+
+
+def _mask_words(m4):
+    """A (B|1, H|1, Sq, Sk) uint8 keep-mask as the backward kernel reads it: four keys per 32-bit word, so rows,
+    strides and the base address are multiples of 4 bytes and a row is readable up to the next multiple of 4 past Sk.
+    Broadcast dimensions (stride 0) stay broadcast; anything else that does not fit is copied into padded rows."""
+    nk = m4.shape[-1]
+    st = m4.stride()
+    if m4.data_ptr() % 4 == 0 and nk % 4 == 0 and st[3] == 1 and all(x % 4 == 0 for x in st[:3]):
+        return m4
+    lead = [1 if st[i] == 0 else m4.shape[i] for i in range(2)]
+    buf = torch.zeros(*lead, m4.shape[2], (nk + 3) // 4 * 4, dtype=torch.uint8, device=m4.device)
+    buf[..., :nk] = m4[:lead[0], :lead[1]]
+    return buf[..., :nk].expand(m4.shape)
+
+
+class _MaskedPrefillFn(torch.autograd.Function):
+    """out = attention(q, k, v) under an explicit keep-mask (the call of model.py:384-385): the masked forward that
+    also writes the log-sum-exp, and the backward kernels in their explicit-mask mode."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, m4):
+        out, lse = _dense(q, k, v, m4, _lib.MASK_BOOL, None, want_lse=True)
+        ctx.save_for_backward(q, k, v, out, lse, m4)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, m4 = ctx.saved_tensors
+        dq, dk, dv = _prefill_backward(q, k, v, out, dout, lse, None, None, q.shape[2], k.shape[2],
+                                       1.0 / math.sqrt(q.shape[-1]), _lib.MASK_BOOL, mask=m4)
+        return dq, dk, dv, None
 
 
 class _VarlenPrefillFn(torch.autograd.Function):
@@ -291,9 +341,11 @@ def scaled_dot_product_attention(Q, K, V, mask=None):
     scale is 1/sqrt(d_k).  A query row whose keys are all masked yields NaN, as
     the reference softmax (llm-core/llm_core/nn_functional.py:8-11) does.
     Restrictions of the HIP path: d_v == d_k in {32, 64, 128}; bfloat16 or float32 tensors (bf16 math, see
-    _to_bf16).  Differentiable for mask=None (dq/dk/dv from the HIP backward kernels); the backward kernels have
-    no explicit-mask mode, so a call with a mask whose inputs require grad raises instead of returning a
-    result that autograd cannot see (use flash_attn_prefill(causal=True) for the causal mask in training).
+    _to_bf16).  Differentiable with and without a mask (dq/dk/dv from the HIP backward kernels), so the reference's
+    non-flash training branch (model.py:384-385: the tril mask rebuilt per call) runs through it unchanged; the
+    explicit-mask kernels read the mask element by element, so flash_attn_prefill(causal=True) remains the fast way
+    to train with a causal mask.  A fully masked query row gives NaN outputs like the reference but zero gradients
+    (the reference propagates the NaN).
     """
     if Q.dim() < 2 or K.dim() != Q.dim() or V.dim() != Q.dim():
         raise ValueError("Q, K and V need the same number of dimensions (>= 2)")
@@ -316,18 +368,17 @@ def scaled_dot_product_attention(Q, K, V, mask=None):
     q4, k4, v4 = as4(Q, nq), as4(K, nk), as4(V, nk)
     m4 = None
     mode = _lib.MASK_NONE
-    if _needs_grad(Q, K, V):
-        if mask is not None:
-            raise NotImplementedError(
-                "scaled_dot_product_attention with an explicit mask is forward-only on the HIP path (the backward "
-                "kernels know no-mask and causal); for causal training use flash_attn_prefill / sdpa_slot")
-        out = _DensePrefillFn.apply(q4, k4, v4, False, None)
-        return out.reshape(*lead, nq, d).to(out_dtype)
     if mask is not None:
         m4 = as4(mask.expand(*mask.shape[:-2], nq, nk), nq).view(torch.uint8)
         if m4.stride(-1) != 1:
             m4 = m4.contiguous()
         mode = _lib.MASK_BOOL
+    if _needs_grad(Q, K, V):
+        if mask is not None:
+            out = _MaskedPrefillFn.apply(q4, k4, v4, _mask_words(m4))
+        else:
+            out = _DensePrefillFn.apply(q4, k4, v4, False, None)
+        return out.reshape(*lead, nq, d).to(out_dtype)
     out = _dense(q4, k4, v4, m4, mode, None, kv_splits=None)
     return out.reshape(*lead, nq, d).to(out_dtype)
 

@@ -247,3 +247,75 @@ def test_backward_rows_without_keys_and_empty_sequences(ops):
     check_grad("dq", qg.grad, dq_ref)
     check_grad("dk", kg.grad, dk_ref)
     check_grad("dv", vg.grad, dv_ref)
+
+
+def oracle_masked_grads(q, k, v, mask, dout):
+    """autograd through the oracle's restatement of model.py:308-325 in fp32: what the reference's own training step
+    derives behind its non-flash branch."""
+    qq, kk, vv = (t.float().requires_grad_() for t in (q, k, v))
+    out = orc.scaled_dot_product_attention(qq, kk, vv, mask)
+    out.backward(dout.float())
+    return out.detach(), qq.grad, kk.grad, vv.grad
+
+
+@pytest.mark.parametrize("S,D", [(256, 32), (200, 64), (131, 128), (384, 128)])
+def test_masked_sdpa_trains_like_the_reference_non_flash_branch(ops, S, D):
+    """llm-core/llm_core/model.py:384-385 as the reference runs it under autograd: the tril keep-mask rebuilt per call,
+    handed to scaled_dot_product_attention with inputs that require grad.  Outputs and gradients against the oracle's
+    causal backward (S = 131: rows that are no multiple of 4 bytes go through the padded copy of the mask)."""
+    print(f"case: sdpa(Q, K, V, tril mask) under autograd S={S} D={D}", flush=True)
+    B, H = 2, 4
+    q, k, v, dout = (rnd(B, H, S, D, seed=300 + i + S) for i in range(4))
+    qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+    causal_mask = torch.tril(torch.ones(S, S, dtype=torch.bool, device="cuda"))          # model.py:384
+    out = ops.scaled_dot_product_attention(qg, kg, vg, causal_mask)                        # model.py:385
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    dq, dk, dv, _ = orc.prefill_backward_reference(q, k, v, dout, causal=True)
+    torch.testing.assert_close(out.detach().float().cpu(), orc.prefill_reference(q, k, v, causal=True), atol=2e-2, rtol=1e-2)
+    check_grad("dq", qg.grad, dq)
+    check_grad("dk", kg.grad, dk)
+    check_grad("dv", vg.grad, dv)
+
+
+@pytest.mark.parametrize("mask_lead", ["none", "batch", "full"])
+def test_masked_sdpa_backward_with_an_arbitrary_mask(ops, mask_lead):
+    """A random keep-mask (no row fully masked), more keys than queries, the mask broadcast over heads and/or batch:
+    gradients against autograd through the oracle's scaled_dot_product_attention."""
+    print(f"case: sdpa backward, random mask, lead={mask_lead}", flush=True)
+    B, H, Sq, Sk, D = 2, 3, 150, 212, 64
+    q, k, v, dout = rnd(B, H, Sq, D, seed=400), rnd(B, H, Sk, D, seed=401), rnd(B, H, Sk, D, seed=402), rnd(B, H, Sq, D, seed=403)
+    g = torch.Generator().manual_seed(404)
+    lead = {"none": (), "batch": (B, 1), "full": (B, H)}[mask_lead]
+    mask = torch.rand(*lead, Sq, Sk, generator=g) < 0.6
+    mask[..., torch.arange(Sq), torch.arange(Sq)] = True
+    qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+    out = ops.scaled_dot_product_attention(qg, kg, vg, mask.cuda())
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    ref, dq, dk, dv = oracle_masked_grads(q, k, v, mask, dout)
+    torch.testing.assert_close(out.detach().float().cpu(), ref, atol=2e-2, rtol=1e-2)
+    check_grad("dq", qg.grad, dq)
+    check_grad("dk", kg.grad, dk)
+    check_grad("dv", vg.grad, dv)
+
+
+def test_masked_sdpa_backward_of_a_fully_masked_row(ops):
+    """A query row whose keys are all masked: NaN output row like the reference softmax; its gradients are zero here
+    (the reference propagates the NaN) and every other row's gradients are those of the problem without that row."""
+    print("case: sdpa backward, one fully masked row", flush=True)
+    B, H, S, D = 1, 2, 96, 64
+    q, k, v, dout = (rnd(B, H, S, D, seed=500 + i) for i in range(4))
+    mask = torch.tril(torch.ones(S, S, dtype=torch.bool))
+    mask[17] = False
+    qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+    out = ops.scaled_dot_product_attention(qg, kg, vg, mask.cuda())
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(out[:, :, 17].float()).all())
+    keep = [i for i in range(S) if i != 17]
+    _, dq, dk, dv = oracle_masked_grads(q[:, :, keep], k, v, mask[keep], dout[:, :, keep])
+    assert bool((qg.grad[:, :, 17] == 0).all())
+    check_grad("dq", qg.grad[:, :, keep], dq)
+    check_grad("dk", kg.grad, dk)
+    check_grad("dv", vg.grad, dv)

@@ -705,8 +705,8 @@ def test_sdpa_slot_trains_through_the_reference_dtype_flow(ops):
 
 def test_sdpa_reference_signature_autograd(ops):
     """scaled_dot_product_attention (the model.py:384-385 branch, used in training without --flash-attn): with
-    mask=None the result carries a grad_fn and the gradients match the oracle; with a mask it raises instead of
-    silently returning a detached result."""
+    with or without a mask the result carries a grad_fn and the gradients match the oracle (the masked cases have their
+    own tests in test_gpu_backward.py)."""
     print("case: sdpa signature autograd", flush=True)
     B, H, S, D = 1, 2, 80, 64
     q, k, v, dout = (rnd(B, H, S, D, seed=s, scale=0.5) for s in (51, 52, 53, 54))
@@ -719,8 +719,15 @@ def test_sdpa_reference_signature_autograd(ops):
     for name, got, ref in (("dq", Q.grad, dq), ("dk", K.grad, dk), ("dv", V.grad, dv)):
         check(got, ref, atol=2e-2 * float(ref.abs().max()), rtol=2e-2, what=name)
     tril = torch.tril(torch.ones(S, S, dtype=torch.bool, device="cuda"))
-    with pytest.raises(NotImplementedError, match="forward-only"):
-        ops.scaled_dot_product_attention(Q, K, V, tril)
+    for t in (Q, K, V):
+        t.grad = None
+    out = ops.scaled_dot_product_attention(Q, K, V, tril)
+    assert out.requires_grad and out.grad_fn is not None
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    dq, dk, dv, _ = orc.prefill_backward_reference(q, k, v, dout, causal=True)
+    for name, got, ref in (("dq", Q.grad, dq), ("dk", K.grad, dk), ("dv", V.grad, dv)):
+        check(got, ref, atol=2e-2 * float(ref.abs().max()), rtol=2e-2, what=name)
     with torch.no_grad():                                              # forward-only use is unaffected
         assert not ops.scaled_dot_product_attention(Q, K, V, tril).requires_grad
 
