@@ -146,8 +146,15 @@ __device__ __forceinline__ void load_bounds(const int32_t* cu_q, const int32_t* 
     k_hi = kb[1];
 }
 
+// heads_per_wg: how the four wavefronts of a workgroup divide a job.
+//   1: a job is 256 query rows of one head, 64 rows per wavefront.  Under a causal mask the wavefronts then see
+//      different numbers of K/V tiles -- in the last four tile steps of a job one to three of them have nothing to
+//      compute and wait at the hand-over for the one with the lowest rows.
+//   4: a job is 64 query rows of FOUR query heads that share a K/V head, one head per wavefront.  The same K/V tiles
+//      serve all four, every wavefront sees the same keys, nobody waits: the launch code takes this whenever a K/V
+//      head has a multiple of four query heads and the mask is causal.
 template <bool CAUSAL>
-__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int tiles_per_unit) {
+__global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int tiles_per_unit, int heads_per_wg) {
     constexpr int D = kWD, NS = D / 16, NDT = D / 32, CPR = D / 8;
     constexpr float kBias = 32.0f;             // the largest weight sits at 2^-kBias when a reference is set
     constexpr float kUnderflow = 0x1p-92f;     // a row sum below this may have lost terms (see the file header)
@@ -167,6 +174,9 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31;          // query column inside a block / key row of K / d row of V^T
     const int kg = lane >> 5;
+    const bool by_head = heads_per_wg == kWWaves;
+    const int bm = by_head ? 64 : kWBM;               // query rows of a job
+    const int wave_rows = by_head ? 0 : 64;           // rows from one wavefront's first query to the next one's
 
     // ---- jobs: a workgroup works through query tiles, one "job" each.  What is dealt to workgroups are UNITS of one
     // (sequence, head [, share of the keys]), all units of the launch forming one list sorted by cost, in one of two
@@ -199,15 +209,16 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const int n_split = p.n_split > 1 ? p.n_split : 1;
     // head and row strides fit 32 bits (the host checks), so an address takes two scalar multiplications
     const int qs2 = (int)p.qs[2], ks2 = (int)p.ks[2], vs2 = (int)p.vs[2], os2 = (int)p.os[2];
-    const int Hq = p.Hq, Hkv = p.Hkv, inner = Hq * n_split;
-    const int group = Hq / Hkv, group_shift = (group & (group - 1)) == 0 ? __builtin_ctz(group) : -1;
+    // (the "query head" digit of a unit counts whole workgroups: single heads, or sets of four heads of one K/V head)
+    const int Hq = p.Hq, Hkv = p.Hkv, Hu = by_head ? Hq / kWWaves : Hq, inner = Hu * n_split;
+    const int group = Hu / Hkv, group_shift = (group & (group - 1)) == 0 ? __builtin_ctz(group) : -1;
     const bool packed = p.cu_q != nullptr;
     const int n_seq_chunks = (p.B + 63) / 64;
     // numbers of query tiles per sequence (packed layout; zero past the last sequence) and the first class
     int cls;
     if (packed) {
         for (int b = tid; b < 64 * n_seq_chunks; b += kWWaves * 64)
-            nq_lds[b] = b < p.B ? (p.cu_q[b + 1] - p.cu_q[b] + kWBM - 1) / kWBM : 0;
+            nq_lds[b] = b < p.B ? (p.cu_q[b + 1] - p.cu_q[b] + bm - 1) / bm : 0;
         __syncthreads();
     }
     const bool pairs = tiles_per_unit == 2;
@@ -263,7 +274,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         for (int d = 32; d >= 1; d >>= 1) most = max(most, __shfl_xor(most, d, 64));
         cls = __builtin_amdgcn_readfirstlane(most);
     } else {
-        cls = (p.Sq + kWBM - 1) / kWBM;
+        cls = (p.Sq + bm - 1) / bm;
     }
     // place of this workgroup in a round: neighbours of the list go to the workgroups of one XCD -- in pairs mode
     // as many as the XCD has workgroups; in single-tile mode, where neighbours cost the same, only the query heads
@@ -295,7 +306,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         j = prev;                             // the sequence-level fields stay while the unit stays
         if (pairs && job_half == 0 && job_unit != job_tiles - 1 - job_unit) {      // second query tile of the pair
             job_half = 1;
-            j.q0 = job_unit * kWBM;
+            j.q0 = job_unit * bm;
             return true;
         }
         const int64_t at = (int64_t)round * G + ((round & 1) ? G - 1 - place : place);
@@ -315,7 +326,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         const int above = group_shift >= 0 ? rest >> group_shift : __builtin_amdgcn_readfirstlane(rest / group);      // (share, K/V head, unit)
         const int head_share = __builtin_amdgcn_readfirstlane(above / units), unit = above - head_share * units;
         const int share = n_split > 1 ? __builtin_amdgcn_readfirstlane(head_share / Hkv) : 0, hk = head_share - share * Hkv;
-        const int h = hk * group + g;
+        const int h = by_head ? (hk * group + g) * kWWaves + wave : hk * group + g;     // (this wavefront's query head)
         const int b = __builtin_amdgcn_readfirstlane(seq_of(cls, seq_rank));
         const ParamsPtr a = args();
         const int qs1 = (int)a->qs[1], ks1 = (int)a->ks[1], vs1 = (int)a->vs[1], os1 = (int)a->os[1], ls1 = (int)a->ls[1];
@@ -352,7 +363,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         job_tiles = cls;
         job_unit = unit;
         job_half = 0;
-        j.q0 = (cls - 1 - unit) * kWBM;
+        j.q0 = (cls - 1 - unit) * bm;
         return true;
     };
 
@@ -395,7 +406,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     // number of K/V tiles of a job (the same for the four wavefronts)
     auto tiles_of = [&](const Job& jb) {
         int kv_end = jb.sk;
-        if (CAUSAL) kv_end = max(0, min(jb.sk, min(jb.sq, jb.q0 + kWBM) + (jb.sk - jb.sq)));
+        if (CAUSAL) kv_end = max(0, min(jb.sk, min(jb.sq, jb.q0 + bm) + (jb.sk - jb.sq)));
         return (kv_end + kWBN - 1) / kWBN;
     };
 
@@ -451,11 +462,14 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     // (loads 4 * part .. 4 * part + 3: rows 16 * part .. 16 * part + 15 of wavefront `to`; a wavefront may request
     // another one's rows, see the early requests below)
     auto issue_q = [&](const Job& jb, int to, int part) {
-        const int qw0 = jb.q0 + 64 * to;
+        const int qw0 = jb.q0 + wave_rows * to;
         const uint32_t row_bytes = (uint32_t)qs2 * 2u;
         const uint32_t dst = q_dst + (uint32_t)((to - wave) * (64 * kWRow) + 4 * part * 1024);
+        // (jb.qb is this wavefront's head; another wavefront's rows may be another head's)
+        const __bf16* qb_to = jb.qb;
+        if (by_head && to != wave) qb_to += (int64_t)(to - wave) * (int)args()->qs[1];
         if (qw0 + 64 <= jb.sq) {
-            const unsigned char* base = reinterpret_cast<const unsigned char*>(jb.qb + (int64_t)(qw0 + 16 * part) * qs2);
+            const unsigned char* base = reinterpret_cast<const unsigned char*>(qb_to + (int64_t)(qw0 + 16 * part) * qs2);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 dma_to_lds_16_m0(base + (size_t)(4 * j) * row_bytes, (uint32_t)ld_q * row_bytes + ((ld_c0 ^ j) << 4), dst + j * 1024);
@@ -464,7 +478,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             int last = jb.sq - 1;
             asm volatile("" : "+s"(last));
             const int first = min(qw0, last);              // (a wavefront wholly past the end reads the last row 64 times)
-            const unsigned char* base = reinterpret_cast<const unsigned char*>(jb.qb + (int64_t)first * qs2);
+            const unsigned char* base = reinterpret_cast<const unsigned char*>(qb_to + (int64_t)first * qs2);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t row = (uint32_t)(min(qw0 + 16 * part + 4 * j + ld_q, last) - first);
@@ -510,7 +524,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     // past the end of the sequence is jumped over, so the count is known here.  (The one or two stores of a
     // log-sum-exp output are not counted: a count that is too low only makes a wait take a little more than it must.)
     auto row_passes = [&](const Job& jb) {
-        return min(max((jb.sq - (jb.q0 + 64 * wave) + kRowsPerPass - 1) / kRowsPerPass, 0), 64 / kRowsPerPass);
+        return min(max((jb.sq - (jb.q0 + wave_rows * wave) + kRowsPerPass - 1) / kRowsPerPass, 0), 64 / kRowsPerPass);
     };
     // waits until at most `young` (rounded down to a multiple of 4) of this wavefront's vector-memory operations
     // are in flight; they complete in order, so everything older than the youngest `young` has then arrived
@@ -540,7 +554,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     while (have) {
         const int sq = cur.sq, sk = cur.sk, q0 = cur.q0;
         const int coff = sk - sq;                          // bottom-right aligned causal diagonal
-        const int qw0 = q0 + 64 * wave;                    // first query of this wavefront
+        const int qw0 = q0 + wave_rows * wave;             // first query of this wavefront
         // the job's tiles are [t_first, n_tiles): all of the query tile's, or its share of them
         int t_first, n_tiles;
         share_of(cur, t_first, n_tiles);
@@ -568,7 +582,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         // (step by step, wavefront by wavefront; part p = rows 16 (p % 4) .. of wavefront 3 - p / 4, so the rows of
         // the wavefront that is busiest at the end of a job go first).  What is left goes out after the tile loop.
         const auto first_hidden_of = [&](int q_tile0, int off, int first, int tiles, int w) {
-            const int hidden = CAUSAL ? min(tiles, max(0, q_tile0 + 64 * w + 63 + off + kWBN) / kWBN) : tiles;
+            const int hidden = CAUSAL ? min(tiles, max(0, q_tile0 + wave_rows * w + 63 + off + kWBN) / kWBN) : tiles;
             return max(hidden, first);
         };
         // number of (step, wavefront) slots in front of slot (tile, w)
@@ -935,12 +949,17 @@ int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
     if (e == hipSuccess) e = hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return (int)e;
     const int n_split = p.n_split > 1 ? p.n_split : 1;
+    // Causal mask and a multiple of four query heads per K/V head: the four wavefronts of a workgroup take the same 64
+    // rows of four heads (every wavefront then sees the same keys); otherwise 4 x 64 rows of one head.
+    const bool by_head = p.mask_mode == MI355_MASK_CAUSAL && (p.Hq / p.Hkv) % kWWaves == 0;
+    const int heads_per_wg = by_head ? kWWaves : 1;
+    const int64_t n_qtiles = by_head ? (p.Sq + 63) / 64 : p.n_qtiles, n_heads = p.Hq / heads_per_wg;
     // Units are pairs of query tiles (equal causal work per unit of a sequence, neighbours that share K/V) unless
     // pairs would leave compute units idle: when every single tile can have a compute unit of its own, or when the
     // pairs make few rounds and the last of them is far from full (judged for sequences of Sq_max rows; then single
     // tiles, dealt by cost, fill the gap better than half as many pairs).
-    const int64_t most_tiles = (int64_t)p.n_qtiles * p.Hq * p.B * n_split;
-    const int64_t most_pairs = (int64_t)((p.n_qtiles + 1) / 2) * p.Hq * p.B * n_split;
+    const int64_t most_tiles = n_qtiles * n_heads * p.B * n_split;
+    const int64_t most_pairs = (n_qtiles + 1) / 2 * n_heads * p.B * n_split;
     const int64_t rounds = (most_pairs + n_cu - 1) / n_cu;
     const bool singles = most_tiles <= n_cu || (rounds < 8 && most_pairs * 100 < rounds * n_cu * 97);
     const int tiles_per_unit = singles ? 1 : 2;
@@ -951,9 +970,9 @@ int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
     if (grid >= 8) grid -= grid % 8;          // whole number of workgroups per XCD
     dim3 block(kWWaves * 64);
     if (p.mask_mode == MI355_MASK_CAUSAL)
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit, heads_per_wg);
     else
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit, heads_per_wg);
     return (int)hipGetLastError();
 }
 
