@@ -93,14 +93,16 @@ int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out
 
 /*
  * Causal prefill of a CHUNK of new tokens on top of context that is already in a paged bf16 cache
- * (chunked prefill / prefix reuse).  The keys and values of all context_lens[b] tokens of sequence b
+ * (chunked prefill / prefix reuse; an fp8 cache: mi355_gather_kv_fp8 below).  The keys and values of all context_lens[b] tokens of sequence b
  * -- the chunk's own included: write them first with mi355_rope_and_cache -- are read through
  * block_tables (the layout of mi355_paged_decode_fwd: int32 (B, table_stride), entry j = physical
  * block of tokens [16j, 16j+16); k_cache/v_cache (num_blocks,Hkv,16,D) bf16).  The chunk's queries
  * are packed: q/out (T,Hq,D) with contiguous heads, sequence b owning rows
  * [cu_seqlens_q[b], cu_seqlens_q[b+1]); its query i keeps key j iff
  * j <= i + (context_lens[b] - chunk length), the bottom-right aligned mask of MI355_MASK_CAUSAL.
- * Only table entries of blocks that hold a valid key are read.  Sq_max = longest chunk.
+ * Only table entries of blocks that hold a valid key are read, and never more than max_blocks per row
+ * (the width of the table, <= table_stride): a context_lens[b] beyond 16 * max_blocks is cut to it,
+ * as mi355_paged_decode_fwd cuts one beyond max_ctx.  Sq_max = longest chunk.
  * Same mathematics as mi355_prefill_fwd (model.py:308-325 / :382) -- the reference has no cache,
  * so it has no counterpart of the table walk; what it replaces is re-running the whole prefix at
  * model.py:218 when a prompt arrives in pieces.
@@ -112,10 +114,29 @@ int mi355_prefill_fwd_lse(const void* q, const void* k, const void* v, void* out
 int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
                             int64_t q_token_stride, int64_t out_token_stride,
                             const int32_t* cu_seqlens_q, const int32_t* block_tables, int64_t table_stride,
-                            const int32_t* context_lens, int B, int Hq, int Hkv, int Sq_max, int D,
-                            int block_size, int64_t num_blocks, float softmax_scale, int kv_dtype,
+                            int64_t max_blocks, const int32_t* context_lens, int B, int Hq, int Hkv, int Sq_max,
+                            int D, int block_size, int64_t num_blocks, float softmax_scale, int kv_dtype,
                             int n_split, int64_t total_q_rows, void* workspace, size_t workspace_bytes,
                             void* stream);
+
+/*
+ * The same chunk over an fp8-e4m3 cache goes in two steps: mi355_gather_kv_fp8 reads every sequence's keys
+ * and values through the block tables and writes them dequantised -- bf16(fp8 * scale of the (block, kv
+ * head) slab) -- as packed rows, k_out / v_out (rows, Hkv, D) bf16 with token stride out_token_stride,
+ * sequence b owning rows [cu_seqlens_k[b], cu_seqlens_k[b+1]) (cu_seqlens_k = running sum of the context
+ * lengths, int32 (B+1), on the device); mi355_prefill_fwd (or _splitkv) then runs on q with cu_seqlens_q
+ * and on those rows with cu_seqlens_k -- the packed layout with more keys than queries per sequence,
+ * bottom-right aligned causal mask -- on the same kernels as any bf16 prefill.
+ * k_scale / v_scale: fp32 (num_blocks, Hkv) as in mi355_paged_decode_fwd.  max_blocks: width of the table
+ * (a longer context_lens[b] is cut to 16 * max_blocks); rows at or past max_rows (the capacity of k_out /
+ * v_out in rows) are not written.  block_size must be 16; D in {32, 64, 128}.
+ * No reference counterpart (the reference has no cache).
+ */
+int mi355_gather_kv_fp8(const void* k_cache_fp8, const void* v_cache_fp8, const float* k_scale,
+                        const float* v_scale, const int32_t* block_tables, int64_t table_stride,
+                        int64_t max_blocks, const int32_t* context_lens, const int32_t* cu_seqlens_k,
+                        void* k_out, void* v_out, int64_t out_token_stride, int64_t max_rows, int B, int Hkv,
+                        int D, int block_size, int64_t num_blocks, void* stream);
 
 /*
  * mi355_prefill_fwd with the keys of every sequence split over n_split workgroups (flash-decoding for

@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     if constexpr (PAGED) {
         const int q_start = p.cu_q[b];
         sq = p.cu_q[b + 1] - q_start;
-        sk = p.ctx_lens[b];
+        sk = min(p.ctx_lens[b], 16 * p.max_blocks);      // a length beyond what the table row addresses is cut, never chased
         qb = p.q + (int64_t)q_start * p.qs[2] + (int64_t)h * p.qs[1];
         kb = vb = nullptr;
         ob = p.out + (int64_t)q_start * p.os[2] + (int64_t)h * p.os[1];
@@ -634,6 +634,7 @@ static int prefill_common(const void* q, const void* k, const void* v, void* out
     p.ctx_lens = nullptr;
     p.table_stride = 0;
     p.num_blocks = 0;
+    p.max_blocks = 0;
     if (int e = set_split(p, D, n_split, total_q_rows, workspace, workspace_bytes, cu_seqlens_q ? -1 : (int64_t)B * Sq_max))
         return e;
     if ((int64_t)p.n_pairs * Hq * B > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill: too many workgroups");
@@ -693,7 +694,8 @@ extern "C" int mi355_prefill_fwd_mask_lse(const void* q, const void* k, const vo
 
 extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const void* v_cache, void* out,
                                        int64_t q_token_stride, int64_t out_token_stride, const int32_t* cu_seqlens_q,
-                                       const int32_t* block_tables, int64_t table_stride, const int32_t* context_lens,
+                                       const int32_t* block_tables, int64_t table_stride, int64_t max_blocks,
+                                       const int32_t* context_lens,
                                        int B, int Hq, int Hkv, int Sq_max, int D, int block_size, int64_t num_blocks,
                                        float softmax_scale, int kv_dtype, int n_split, int64_t total_q_rows,
                                        void* workspace, size_t workspace_bytes, void* stream) {
@@ -706,6 +708,8 @@ extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const
     if (!(D == 128 || D == 64 || D == 32)) return set_error(MI355_EINVAL, "prefill_paged: head_dim must be 32, 64 or 128");
     if (num_blocks <= 0 || num_blocks > 0x7fffffffLL || table_stride <= 0)
         return set_error(MI355_EINVAL, "prefill_paged: num_blocks and table_stride must be positive");
+    if (max_blocks <= 0 || max_blocks > table_stride || max_blocks > 0x7ffffff)
+        return set_error(MI355_EINVAL, "prefill_paged: max_blocks must be in 1..table_stride");
     if ((q_token_stride | out_token_stride) & 7)
         return set_error(MI355_EINVAL, "prefill_paged: token strides must be multiples of 8 elements (16-byte rows)");
     if (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15)
@@ -735,6 +739,7 @@ extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const
     p.ctx_lens = context_lens;
     p.table_stride = table_stride;
     p.num_blocks = (int)num_blocks;
+    p.max_blocks = (int)max_blocks;
     if (int e = set_split(p, D, n_split, total_q_rows, workspace, workspace_bytes, -1)) return e;
     if ((int64_t)p.n_pairs * Hq * B > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill_paged: too many workgroups");
     hipStream_t s = (hipStream_t)stream;

@@ -28,6 +28,7 @@ struct PrefillParams {
     const int32_t* ctx_lens;
     int64_t table_stride;
     int num_blocks;
+    int max_blocks;                       // entries of a table row that may be read: a longer context is cut to 16 * max_blocks keys
     // split keys (n_split > 1): workgroup (.., split c) serves the c-th share of every query tile's K/V tiles and
     // writes, instead of `out`, a normalised fp32 partial result and its log-sum-exp per query row:
     //   part_o  (n_split, Hq, part_rows, D)    part_lse (n_split, Hq, part_rows)

@@ -6,7 +6,7 @@ llm-core/llm_core/model.py:308-325 and the SDPA slot at model.py:382):
     scaled_dot_product_attention(Q, K, V, mask=None)
     flash_attn_prefill(q, k, v, causal=True)            # f(Q, K, V, is_causal=True) slot
     flash_attn_varlen_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, ...)
-    flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, context_lens, max_seqlen_q)
+    flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, context_lens, max_seqlen_q)   # bf16 or fp8 cache
     paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, ...)
     rope_and_cache(q, k, v, positions, freq_cache, k_cache, v_cache, slot_mapping)   # cache producer
     quantize_kv_cache_fp8(cache)
@@ -24,6 +24,7 @@ from .ops import (  # noqa: F401
     rope_and_cache_fp8,
     silu_mul,
     flash_attn_paged_prefill,
+    gather_kv_fp8,
     flash_attn_prefill,
     flash_attn_varlen_prefill,
     paged_attention_decode,

@@ -28,6 +28,7 @@ EXPORTS = (
     "mi355_paged_decode_workspace_bytes",
     "mi355_paged_decode_chunk_tokens",
     "mi355_prefill_paged_fwd",
+    "mi355_gather_kv_fp8",
     "mi355_prefill_fwd_splitkv",
     "mi355_prefill_splitkv_workspace_bytes",
     "mi355_prefill_suggest_kv_splits",
@@ -73,8 +74,10 @@ def load():
     lib.mi355_prefill_bwd_mask.argtypes = [vp] * 10 + [_i64x3] * 8 + [_i64x2, vp, _i64x3,
                                                                       i32, i32, i32, i32, i32, i32, f32, i32, vp]
     lib.mi355_prefill_paged_fwd.restype = i32
-    lib.mi355_prefill_paged_fwd.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, i64, vp,
+    lib.mi355_prefill_paged_fwd.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, i64, i64, vp,
                                             i32, i32, i32, i32, i32, i32, i64, f32, i32, i32, i64, vp, sz, vp]
+    lib.mi355_gather_kv_fp8.restype = i32
+    lib.mi355_gather_kv_fp8.argtypes = [vp, vp, vp, vp, vp, i64, i64, vp, vp, vp, vp, i64, i64, i32, i32, i32, i32, i64, vp]
     lib.mi355_prefill_fwd_splitkv.restype = i32
     lib.mi355_prefill_fwd_splitkv.argtypes = [vp, vp, vp, vp, _i64x3, _i64x3, _i64x3, _i64x3, vp, vp,
                                               i32, i32, i32, i32, i32, i32, f32, i32, i32, i32, i64, vp, sz, vp]

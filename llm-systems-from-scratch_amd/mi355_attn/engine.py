@@ -59,6 +59,7 @@ class PrefillPlan:
     # then reads all keys and values through the block tables
     tables: torch.Tensor | None = None        # (B, max_blocks) int32
     context_lens: torch.Tensor | None = None  # (B,) int32: tokens in the cache, this chunk included
+    total_context: int = 0                    # their sum (sizes the dequantised rows of an fp8 cache)
 
 
 @dataclass
@@ -177,7 +178,8 @@ class PagedAttentionEngine:
     def plan_prefill(self, seq_ids, lens) -> PrefillPlan:
         """Reserves cache slots for the next `lens[i]` prompt tokens of each sequence in `seq_ids`.  A sequence
         may be new (the usual case) or already hold tokens -- a further chunk of a long prompt, or a prompt on
-        top of a cached prefix: the chunk's queries then attend to everything cached so far (bf16 cache only)."""
+        top of a cached prefix: the chunk's queries then attend to everything cached so far (with an fp8 cache: to
+        the quantised keys and values, the chunk's own included, as every later decode step will)."""
         if len(seq_ids) != len(lens) or not seq_ids:
             raise ValueError("seq_ids and lens must be non-empty and of equal length")
         if len(set(seq_ids)) != len(seq_ids):
@@ -186,9 +188,6 @@ class PagedAttentionEngine:
             if n < 1 or self.lengths[sid] + n > self.context_length:
                 raise ValueError(f"prompt lengths must be in 1..{self.context_length} (tokens already cached included)")
         chunked = any(self.lengths[sid] != 0 for sid in seq_ids)
-        if chunked and self.kv_dtype != "bf16":
-            raise NotImplementedError("a further chunk of a prompt needs a bf16 cache: the chunk would attend to "
-                                      "quantised keys and values of its own prefix")
         need = sum((self.lengths[sid] + n + BLOCK - 1) // BLOCK - len(self.blocks[sid]) for sid, n in zip(seq_ids, lens))
         if need > self.allocator.num_free:
             raise OutOfBlocks(f"prefill needs {need} blocks, {self.allocator.num_free} free")
@@ -211,6 +210,7 @@ class PagedAttentionEngine:
                 rows[i, :len(b)] = torch.tensor(b, dtype=torch.int32)
             plan.tables = rows.to(dev)
             plan.context_lens = torch.tensor([self.lengths[sid] for sid in seq_ids], dtype=torch.int32, device=dev)
+            plan.total_context = sum(self.lengths[sid] for sid in seq_ids)
         return plan
 
     def _reserve_decode(self, seq_ids):
@@ -288,8 +288,10 @@ class PagedAttentionEngine:
             raise ValueError("the plan and the packed tensors disagree on the number of tokens")
         if plan.tables is not None:
             q_rot = self._write_cache(layer, plan, q, k, v)
+            scales = {} if self.kv_dtype == "bf16" else {"k_scale": self.k_scales[layer], "v_scale": self.v_scales[layer],
+                                                         "total_context": plan.total_context}
             return ops.flash_attn_paged_prefill(q_rot, self.k_caches[layer], self.v_caches[layer], plan.cu_seqlens,
-                                                plan.tables, plan.context_lens, plan.max_len)
+                                                plan.tables, plan.context_lens, plan.max_len, **scales)
         q_rot, k_rot = self._write_cache(layer, plan, q, k, v, k_out=True)
         return ops.flash_attn_varlen_prefill(q_rot, k_rot, v, plan.cu_seqlens, plan.cu_seqlens, plan.max_len,
                                              plan.max_len, causal=True)

@@ -532,8 +532,9 @@ def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, s
 
 
 def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, context_lens, max_seqlen_q, *,
-                             softmax_scale=None, out=None, max_context=None, kv_splits=None, workspace=None):
-    """Causal prefill of a chunk of new tokens over context that already sits in a paged bf16 cache.
+                             softmax_scale=None, out=None, max_context=None, kv_splits=None, workspace=None,
+                             k_scale=None, v_scale=None, total_context=None):
+    """Causal prefill of a chunk of new tokens over context that already sits in a paged cache.
 
     q (T,Hq,D) bf16, packed, contiguous heads (token stride free): sequence b owns rows
     [cu_seqlens_q[b], cu_seqlens_q[b+1]).  k_cache, v_cache (num_blocks,Hkv,16,D) bf16 hold ALL
@@ -542,9 +543,18 @@ def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, co
     j <= i + (context_lens[b] - chunk length).  max_seqlen_q = longest chunk.  Returns (T,Hq,D) bf16.
     max_context bounds context_lens (default: what block_tables can address) and only guides the choice of
     kv_splits (see flash_attn_prefill): a short chunk over a long context is split over many workgroups.
+    A context length beyond what a row of block_tables addresses is cut to it.
+    With k_scale and v_scale (num_blocks,Hkv) fp32 the cache is fp8-e4m3 (uint8 / float8_e4m3fn, the layout
+    of paged_attention_decode): the sequences' keys and values are first gathered and dequantised into packed
+    bf16 rows (mi355_gather_kv_fp8; value = bf16(fp8 * scale)), then attended to by the packed prefill kernels.
+    total_context (host int, optional): an upper bound on sum(context_lens) that sizes those rows (default
+    batch * max_context).
     The mathematics is that of llm-core/llm_core/model.py:308-325 with the mask of :384; the reference
     itself would re-run the whole prefix (model.py:218)."""
     _require_gpu_bf16("q", q)
+    if k_scale is not None or v_scale is not None:
+        return _paged_prefill_fp8(q, k_cache, v_cache, k_scale, v_scale, cu_seqlens_q, block_tables, context_lens,
+                                  max_seqlen_q, softmax_scale, out, max_context, kv_splits, workspace, total_context)
     if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
         raise ValueError("q must be (tokens, heads, d_head) with contiguous heads")
     T, Hq, D = q.shape
@@ -591,12 +601,79 @@ def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, co
     with _on(q, k_cache, v_cache, out, cu_seqlens_q, block_tables, context_lens, workspace) as stream:
         rc = _lib.load().mi355_prefill_paged_fwd(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), q.stride(0), out.stride(0),
-            cu_seqlens_q.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
+            cu_seqlens_q.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), block_tables.shape[1],
+            context_lens.data_ptr(),
             B, Hq, Hkv, int(max_seqlen_q), D, _BLOCK, k_cache.shape[0], float(scale), _lib.MI355_BF16,
             n_split, T, None if workspace is None else workspace.data_ptr(),
             0 if workspace is None else workspace.numel() * workspace.element_size(), stream)
     _lib.check(rc, "mi355_prefill_paged_fwd")
     return out
+
+
+def gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens, *, max_context=None, total_context=None):
+    """The keys and values of a batch of sequences out of an fp8 paged cache, dequantised, as packed bf16 rows.
+    Returns (k (rows,Hkv,D), v (rows,Hkv,D), cu_seqlens_k int32 (B+1,)): sequence b owns rows
+    [cu_seqlens_k[b], cu_seqlens_k[b+1]), cu_seqlens_k the running sum of min(context_lens, max_context);
+    rows = total_context when given (a host-side bound on that sum), else batch * max_context.  Nothing is read
+    back from the device."""
+    for n, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+        if c.dtype not in (torch.uint8, torch.float8_e4m3fn) or c.dim() != 4 or c.shape[2] != _BLOCK or not c.is_contiguous() \
+                or not c.is_cuda:
+            raise ValueError(f"{n} must be a contiguous uint8/float8_e4m3fn GPU tensor (num_blocks, kv_heads, {_BLOCK}, d_head)")
+    if k_cache.shape != v_cache.shape:
+        raise ValueError("k_cache and v_cache must have the same shape")
+    nb, Hkv, _, D = k_cache.shape
+    if D not in (32, 64, 128):
+        raise ValueError("d_head must be 32, 64 or 128")
+    if k_scale is None or v_scale is None:
+        raise ValueError("k_scale and v_scale must be given together")
+    for n, c in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if c.dtype != torch.float32 or tuple(c.shape) != (nb, Hkv) or not c.is_contiguous():
+            raise ValueError(f"{n} must be a contiguous float32 (num_blocks, kv_heads) tensor")
+    if block_tables.dtype != torch.int32 or context_lens.dtype != torch.int32:
+        raise TypeError("block_tables and context_lens must be int32")
+    B = context_lens.numel()
+    if block_tables.dim() != 2 or block_tables.shape[0] != B or block_tables.stride(1) != 1 or block_tables.shape[1] < 1:
+        raise ValueError("block_tables must be (batch, max_blocks) with unit column stride")
+    if context_lens.shape != (B,) or not context_lens.is_contiguous():
+        raise ValueError("context_lens must be a contiguous (batch,) tensor")
+    width = block_tables.shape[1] * _BLOCK
+    max_context = width if max_context is None else min(int(max_context), width)
+    rows = B * max_context if total_context is None else min(int(total_context), B * max_context)
+    dev = k_cache.device
+    cu_k = torch.zeros(B + 1, dtype=torch.int32, device=dev)
+    if B:
+        cu_k[1:] = torch.cumsum(context_lens.clamp(max=max_context), 0)
+    k_lin = torch.empty(max(rows, 1), Hkv, D, dtype=torch.bfloat16, device=dev)
+    v_lin = torch.empty(max(rows, 1), Hkv, D, dtype=torch.bfloat16, device=dev)
+    if B and rows:
+        with _on(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens) as stream:
+            rc = _lib.load().mi355_gather_kv_fp8(
+                k_cache.data_ptr(), v_cache.data_ptr(), k_scale.data_ptr(), v_scale.data_ptr(), block_tables.data_ptr(),
+                block_tables.stride(0), (max_context + _BLOCK - 1) // _BLOCK, context_lens.data_ptr(), cu_k.data_ptr(),
+                k_lin.data_ptr(), v_lin.data_ptr(), Hkv * D, rows, B, Hkv, D, _BLOCK, nb, stream)
+        _lib.check(rc, "mi355_gather_kv_fp8")
+    return k_lin, v_lin, cu_k
+
+
+def _paged_prefill_fp8(q, k_cache, v_cache, k_scale, v_scale, cu_seqlens_q, block_tables, context_lens, max_seqlen_q,
+                       softmax_scale, out, max_context, kv_splits, workspace, total_context):
+    """flash_attn_paged_prefill over an fp8 cache: gather + dequantise, then the packed prefill with more keys than
+    queries per sequence (bottom-right aligned causal mask)."""
+    if q.dim() != 3:
+        raise ValueError("q must be (tokens, heads, d_head)")
+    if block_tables.dim() != 2:
+        raise ValueError("block_tables must be (batch, max_blocks)")
+    width = block_tables.shape[1] * _BLOCK
+    max_context = width if max_context is None else min(int(max_context), width)
+    k_lin, v_lin, cu_k = gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens,
+                                       max_context=max_context, total_context=total_context)
+    res = flash_attn_varlen_prefill(q, k_lin, v_lin, cu_seqlens_q, cu_k, max_seqlen_q, max_context, causal=True,
+                                    softmax_scale=softmax_scale, kv_splits=kv_splits, workspace=workspace)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
 
 
 def build_rope_cache(context_length, d, theta=10000.0, device="cuda"):

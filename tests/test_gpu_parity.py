@@ -448,6 +448,71 @@ def test_prefill_head_dim_128_two_kernels_agree_on_random_shapes(ops, seed):
 
 
 @pytest.mark.parametrize("seed", [0, 1, 2])
+def test_prefill_head_dim_128_four_heads_per_workgroup_on_random_shapes(ops, seed):
+    """Causal prefill with a multiple of four query heads per K/V head: the 64-query kernel then gives the four wavefronts
+    of a workgroup the same 64 rows of four heads (one head each) instead of 4 x 64 rows of one head.  Drawn shapes --
+    4, 8 or 12 query heads per K/V head, ragged query and key counts, more keys than queries, runaway keys -- against
+    the oracle and against the other kernel; with the keys split (partial rows per head), with the log-sum-exp output,
+    and the gradients that the training forward feeds."""
+    g = torch.Generator().manual_seed(7000 + seed)
+    for case in range(4):
+        B = int(torch.randint(1, 3, (1,), generator=g))
+        Hkv = int(torch.randint(1, 3, (1,), generator=g))
+        Hq = Hkv * 4 * int(torch.randint(1, 4, (1,), generator=g))
+        Sq = int(torch.randint(1, 700, (1,), generator=g))
+        Sk = Sq + int(torch.randint(0, 500, (1,), generator=g)) * int(torch.randint(0, 2, (1,), generator=g))
+        print(f"case: four heads per workgroup seed={seed} #{case} B={B} Hq={Hq} Hkv={Hkv} Sq={Sq} Sk={Sk}", flush=True)
+        q = torch.randn(B, Hq, Sq, 128, generator=g).to(torch.bfloat16)
+        k = torch.randn(B, Hkv, Sk, 128, generator=g)
+        v = torch.randn(B, Hkv, Sk, 128, generator=g).to(torch.bfloat16)
+        for _ in range(int(torch.randint(0, 4, (1,), generator=g))):          # runaway keys
+            j = int(torch.randint(0, Sk, (1,), generator=g))
+            k[:, :, j:j + int(torch.randint(1, 70, (1,), generator=g))] *= float(torch.tensor([6.0, 20.0, -15.0, 45.0])[int(torch.randint(0, 4, (1,), generator=g))])
+        k = k.to(torch.bfloat16)
+        ref = orc.prefill_reference(q, k, v, causal=True)
+        fast = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=True, kv_splits=1)
+        keep = torch.tril(torch.ones(Sq, Sk, dtype=torch.bool), diagonal=Sk - Sq)
+        slow = ops.scaled_dot_product_attention(q.cuda(), k.cuda().repeat_interleave(Hq // Hkv, 1),
+                                                v.cuda().repeat_interleave(Hq // Hkv, 1), keep.cuda())
+        shared = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=True, kv_splits=2 + (seed + case) % 3)
+        from mi355_attn import ops as raw
+        out2, lse = raw._dense(q.cuda(), k.cuda(), v.cuda(), None, 1, None, want_lse=True)
+        torch.cuda.synchronize()
+        check(fast, ref, what=f"four heads per workgroup seed {seed} #{case}")
+        check(slow, ref, what=f"8-wavefront kernel seed {seed} #{case}")
+        check(shared, ref, what=f"four heads per workgroup, keys split, seed {seed} #{case}")
+        assert torch.equal(out2, fast)
+        s_ = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float().repeat_interleave(Hq // Hkv, 1)) / math.sqrt(128)
+        torch.testing.assert_close(lse.cpu(), torch.logsumexp(s_.masked_fill(~keep, float("-inf")), -1), atol=3e-3, rtol=1e-3)
+
+
+def test_prefill_head_dim_128_four_heads_per_workgroup_packed_and_trained(ops):
+    """The same job layout on a packed batch of drawn lengths (an empty sequence and a one-token one included), and
+    through autograd: the forward with the log-sum-exp runs on this layout, the backward kernels read what it wrote."""
+    print("case: four heads per workgroup, packed + backward", flush=True)
+    Hq, Hkv, D = 8, 2, 128
+    lens = [300, 0, 1, 129, 517, 64]
+    T = sum(lens)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    q, k, v, dout = rnd(T, Hq, D, seed=7100), rnd(T, Hkv, D, seed=7101), rnd(T, Hkv, D, seed=7102), rnd(T, Hq, D, seed=7103)
+    ref = orc.varlen_prefill_reference(q, k, v, cu, cu, causal=True)
+    qg, kg, vg = (t.cuda().requires_grad_() for t in (q, k, v))
+    out = ops.flash_attn_varlen_prefill(qg, kg, vg, cu.cuda(), cu.cuda(), max(lens), max(lens), causal=True)
+    out.backward(dout.cuda())
+    torch.cuda.synchronize()
+    check(out.detach(), ref, what="packed, four heads per workgroup")
+    for b, n in enumerate(lens):
+        if n == 0:
+            continue
+        a, e = int(cu[b]), int(cu[b + 1])
+        args = [t[a:e].transpose(0, 1)[None] for t in (q, k, v, dout)]
+        dq, dk, dv, _ = orc.prefill_backward_reference(*args, causal=True)
+        for name, got, want in (("dq", qg.grad[a:e], dq), ("dk", kg.grad[a:e], dk), ("dv", vg.grad[a:e], dv)):
+            want = want[0].transpose(0, 1)
+            check(got, want, atol=1e-4 + 2e-2 * float(want.abs().max()), rtol=2e-2, what=f"{name} of sequence {b}")
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
 def test_prefill_head_dim_128_packed_sequences_of_drawn_lengths(ops, seed):
     """Packed sequences of drawn lengths (empty ones included) through the persistent 64-query kernel: a workgroup
     walks from job to job across sequences of different lengths, prefetching the next job's rows and tiles; with
@@ -635,6 +700,84 @@ def test_paged_prefill_ragged_chunks_match_the_oracle(ops, D, Hq, Hkv):
     ret = ops.flash_attn_paged_prefill(wide[:, :Hq], kc2.to(dev), vc2.to(dev), cu.to(dev), bt2.to(dev), cl.to(dev),
                                        max(chunk), out=out)
     assert ret is out and torch.equal(out, got)
+
+
+@pytest.mark.parametrize("D,Hq,Hkv", [(128, 8, 2), (64, 4, 4), (128, 32, 8)])
+def test_paged_prefill_over_an_fp8_cache_matches_the_oracle(ops, D, Hq, Hkv):
+    """The same ragged chunks over an fp8-e4m3 cache with per-(block, kv head) scales: gathered and dequantised by
+    mi355_gather_kv_fp8, attended to by the packed prefill kernels.  Kernel parity: within the bf16 tolerance of the
+    oracle on the DEQUANTISED cache.  Quantisation noise: against the oracle on the bf16 cache the result stays within
+    |err| <= 0.15 + 2^-4 |ref| with a relative rms error under 6 % (the bound of the fp8 decode)."""
+    ctx = [700, 391, 64, 1500, 17, 300]
+    chunk = [203, 391, 1, 1, 17, 299]
+    print(f"case: paged prefill over fp8 D={D} Hq={Hq} Hkv={Hkv}", flush=True)
+    _, kc, vc, bt, cl = orc.make_paged_case(batch=len(ctx), n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                            context_lens=ctx, pool_factor=1.3, seed=31, dtype=torch.bfloat16)
+    # the tail of a sequence's last block holds zeros (what a cache writer leaves there), so that a block's scale
+    # comes from its valid rows
+    for b, c in enumerate(ctx):
+        if c % 16:
+            last = int(bt[b, (c - 1) // 16])
+            kc[last, :, c % 16:] = 0
+            vc[last, :, c % 16:] = 0
+    k8, ks = orc.quantize_kv_fp8(kc)
+    v8, vs = orc.quantize_kv_fp8(vc)
+    cu = torch.tensor([0] + list(torch.tensor(chunk).cumsum(0)), dtype=torch.int32)
+    q = rnd(int(cu[-1]), Hq, D, seed=32)
+    ref8 = orc.paged_prefill_reference(q, orc.dequantize_kv_fp8(k8, ks), orc.dequantize_kv_fp8(v8, vs), cu, bt, cl)
+    ref16 = orc.paged_prefill_reference(q, kc, vc, cu, bt, cl)
+    dev = "cuda:0"
+    bt2 = bt.clone()
+    for b, c in enumerate(ctx):
+        bt2[b, (c + 15) // 16:] = 2 ** 30                      # the table tail is never read
+    args = (q.to(dev), k8.to(dev), v8.to(dev), cu.to(dev), bt2.to(dev), cl.to(dev), max(chunk))
+    got = ops.flash_attn_paged_prefill(*args, k_scale=ks.to(dev), v_scale=vs.to(dev))
+    tight = ops.flash_attn_paged_prefill(*args, k_scale=ks.to(dev), v_scale=vs.to(dev), total_context=sum(ctx), kv_splits=1)
+    torch.cuda.synchronize()
+    check(got, ref8, what="paged prefill over fp8, oracle on the dequantised cache")
+    check(tight, ref8, what="paged prefill over fp8, rows sized by total_context")
+    e16 = (got.float().cpu() - ref16).abs()
+    assert bool((e16 <= 0.15 + 2.0 ** -4 * ref16.abs()).all()), float(e16.max())
+    assert float((got.float().cpu() - ref16).pow(2).mean().sqrt() / ref16.pow(2).mean().sqrt()) <= 0.06
+    # the gathered rows themselves: bf16(fp8 * scale), row by row
+    kl, vl, cu_k = ops.gather_kv_fp8(k8.to(dev), v8.to(dev), ks.to(dev), vs.to(dev), bt2.to(dev), cl.to(dev))
+    assert cu_k.tolist() == [0] + list(torch.tensor(ctx).cumsum(0))
+    for b in (0, 3, 4):
+        want = orc.gather_paged_kv(orc.dequantize_kv_fp8(k8, ks), bt[b], ctx[b]).transpose(0, 1).to(torch.bfloat16)
+        assert torch.equal(kl[int(cu_k[b]):int(cu_k[b + 1])].cpu(), want)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_paged_prefill_cuts_a_context_length_beyond_the_table(ops, fp8):
+    """A context_lens entry larger than what a row of the block table addresses (a corrupted length) must not walk
+    past the row: the sequence is served as if its length were 16 * (table width), finite and equal to that call."""
+    print(f"case: paged prefill, context length beyond the table, fp8={fp8}", flush=True)
+    Hq, Hkv, D = 4, 2, 64
+    ctx, chunk = [160, 96], [40, 96]
+    _, kc, vc, bt, cl = orc.make_paged_case(batch=2, n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                            context_lens=ctx, seed=9, dtype=torch.bfloat16)
+    assert bt.shape[1] == 10
+    cu = torch.tensor([0, 40, 136], dtype=torch.int32)
+    q = rnd(136, Hq, D, seed=10)
+    dev = "cuda:0"
+    kw = {}
+    kcd, vcd = kc.to(dev), vc.to(dev)
+    if fp8:
+        k8, ks = orc.quantize_kv_fp8(kc)
+        v8, vs = orc.quantize_kv_fp8(vc)
+        kcd, vcd, kw = k8.to(dev), v8.to(dev), {"k_scale": ks.to(dev), "v_scale": vs.to(dev)}
+    good = ops.flash_attn_paged_prefill(q.to(dev), kcd, vcd, cu.to(dev), bt.to(dev), cl.to(dev), 96, **kw)
+    wild = torch.tensor([160 + 5000, 96], dtype=torch.int32)
+    # (the last sequence's row is the end of the table's memory: a walk past it would leave the allocation)
+    wild2 = torch.tensor([160, 96 + 70000], dtype=torch.int32)
+    got = ops.flash_attn_paged_prefill(q.to(dev), kcd, vcd, cu.to(dev), bt.to(dev), wild.to(dev), 96, **kw)
+    got2 = ops.flash_attn_paged_prefill(q.to(dev), kcd, vcd, cu.to(dev), bt.to(dev), wild2.to(dev), 96, **kw)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(got.float()).all()) and bool(torch.isfinite(got2.float()).all())
+    # sequence 0 with the wild length sees all 160 keys of its row as context: its 40 queries sit at the END of them
+    assert torch.equal(got[:40], good[:40]) and torch.equal(got[40:], good[40:])
+    # sequence 1 is cut to 160 keys = its 96 + 64 from blocks the row lists beyond its length (zeros in the table -> block 0)
+    assert torch.equal(got2[:40], good[:40])
 
 
 def test_paged_prefill_equals_dense_prefill_on_the_gathered_rows(ops):
