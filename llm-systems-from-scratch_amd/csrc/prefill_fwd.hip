@@ -49,8 +49,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     constexpr int NT = kBN * CPR / 64;            // direct-to-LDS instructions per tile and tensor
     constexpr int NI = (NT + kPfWaves - 1) / kPfWaves;   // ... per wavefront (the last wavefronts may have none)
 
-    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kTile];
-    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kTile];
+    // K/V tile buffers: tile t lives in buffer t % NB, and while tile t is computed tile t+1 is landing.  (Four buffers
+    // with three tiles in flight were tried for head_dim 64 and 32, where a tile is only a few hundred cycles of work:
+    // the larger LDS footprint leaves room for fewer workgroups per compute unit, and every shape but the smallest
+    // launches ran 10-23 % slower.  The code below is written for any power of two.)
+    constexpr int NB = 2;
+    constexpr int kAhead = NB - 1;
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[NB * kTile];
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[NB * kTile];
     // Staging of the query rows on their way in and of the output rows on their way out, one private slab per
     // wavefront (32 rows of D bf16, rows padded by 16 bytes): fragments and accumulators hold a query per lane,
     // so direct accesses would touch 16- or 8-byte pieces of 32 different rows per instruction; through the
@@ -102,8 +108,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     }
     // Causal work grows with the query-tile index, so a workgroup takes the tiles
     // (nq-1-pair) and (pair): every workgroup of a sequence then carries the same load.
+    // (A launch that would leave compute units without a workgroup deals single query tiles instead, heaviest first:
+    // p.n_pairs then counts tiles.)
     const int nq = (sq + kBM - 1) / kBM;
-    if (2 * pair0 >= nq) return;         // (a sequence without keys still gets its rows written: no key kept -> NaN)
+    const bool singles = p.single_tiles != 0;
+    if ((singles ? pair0 : 2 * pair0) >= nq) return;         // (a sequence without keys still gets its rows written: no key kept -> NaN)
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -203,8 +212,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     // The grid holds n_pairs workgroups per (batch, head), sized from the caller's Sq_max.  A packed sequence that is
     // longer than that promise is still computed in full: its workgroups walk on through the remaining tile pairs
     // (with a correct Sq_max this loop runs once).
-    for (int pair = pair0; 2 * pair < nq; pair += p.n_pairs)
-    for (int half = 0; half < 2; ++half) {
+    for (int pair = pair0; (singles ? pair : 2 * pair) < nq; pair += p.n_pairs)
+    for (int half = 0; half < (singles ? 1 : 2); ++half) {
         const int qtile = half == 0 ? nq - 1 - pair : pair;
         if (half == 1 && qtile == nq - 1 - pair) break;         // odd tile count: the middle tile has no partner
         const int q0 = qtile * kBM;
@@ -222,10 +231,11 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
             t1 = min(n_tiles, t0 + per);
         }
 
-        // the first K/V tile is requested before the query rows, so that the two latencies overlap
-        // (tile t lives in buffer t % 2)
+        // the first K/V tiles are requested before the query rows, so that the latencies overlap
         __syncthreads();                     // the previous query tile's readers are done with the LDS buffers
-        if (t1 > t0) issue_tile(t0, t0 & 1);
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i)
+            if (t0 + i < t1) issue_tile(t0 + i, (t0 + i) & (NB - 1));
 
         // ---- Q^T fragments: step s covers d = 16s + 8kg + j ----------------------
         // rows come in whole (CPR lanes per row) and go through the wavefront's slab (private, and LDS operations
@@ -272,24 +282,48 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
 
         f32x16 s_acc[2];
         float mx = 0.f;
-        const auto flip = [&]() {            // the per-lane read offsets carry the LDS buffer bit
+        // the per-lane read offsets carry the LDS buffer of the tile being read
+        const auto set_buf = [&](int buf) {
 #pragma unroll
-            for (int s = 0; s < NS; ++s) k_off[s] ^= kTile;
+            for (int s = 0; s < NS; ++s) k_off[s] = (k_off[s] & (kTile - 1)) | (buf * kTile);
 #pragma unroll
             for (int e = 0; e < 2; ++e)
 #pragma unroll
-                for (int dt = 0; dt < NDT; ++dt) v_off[e][dt] ^= kTile;
+                for (int dt = 0; dt < NDT; ++dt) v_off[e][dt] = (v_off[e][dt] & (kTile - 1)) | (buf * kTile);
+        };
+        int cur_tile = t0;                   // the tile the offsets point at
+        const auto flip = [&]() {            // on to the next tile's buffer
+            ++cur_tile;
+            if constexpr (NB == 2) {
+#pragma unroll
+                for (int s = 0; s < NS; ++s) k_off[s] ^= kTile;
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+#pragma unroll
+                    for (int dt = 0; dt < NDT; ++dt) v_off[e][dt] ^= kTile;
+            } else {
+                set_buf(cur_tile & (NB - 1));
+            }
         };
 
         // First half of a KV tile: wait for it, start the next one, S^T = K . Q^T, mask, row max.
         // Returns false when the whole tile lies above this wavefront's diagonal (nothing to add).
         auto head = [&](auto masked_c, int tile) -> bool {
             constexpr bool MASKED = decltype(masked_c)::value;
-            wait_vmcnt<0>();                 // this wavefront's share of tile `tile` has landed
-            __syncthreads();                 // ... and everybody's; also: all are done reading the other buffer
+            // this wavefront's share of tile `tile` has landed: its loads are older than those of the tiles requested
+            // after it (2 * NI instructions each), which may stay in flight
+            if constexpr (NB == 2) {
+                wait_vmcnt<0>();
+            } else {
+                const int younger = min(kAhead - 1, t1 - 1 - tile);
+                if (younger >= 2) wait_vmcnt<4 * NI>();
+                else if (younger == 1) wait_vmcnt<2 * NI>();
+                else wait_vmcnt<0>();
+            }
+            __syncthreads();                 // ... and everybody's; also: all are done reading the buffer of the tile before
 
-            // The next tile's direct-to-LDS loads go out first: a whole tile of work hides their latency.
-            if (tile + 1 < t1) issue_tile(tile + 1, (tile + 1) & 1);
+            // The loads of the tile that takes that buffer go out first: the work of kAhead tiles hides their latency.
+            if (tile + kAhead < t1) issue_tile(tile + kAhead, (tile + kAhead) & (NB - 1));
 
             const int k0 = tile * kBN;
             if (causal && MASKED && k0 > qw0 + 31 + coff) return false;
@@ -391,10 +425,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
             }
         };
 
-        if (t1 > t0 && (t0 & 1)) flip();     // the offsets start at the first tile's buffer ...
+        set_buf(t0 & (NB - 1));              // the offsets start at the first tile's buffer
         run_tiles(std::false_type{}, t0, min(n_plain, t1));
         run_tiles(std::true_type{}, max(n_plain, t0), t1);
-        if (t1 > t0 && (t1 & 1)) flip();     // ... and are left pointing at buffer 0 for the next query tile
 
         // ---- normalise and store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4 ---
         l_run = xor32_sum(l_run);
@@ -449,9 +482,28 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     }
 }
 
+// Pairs of query tiles carry equal causal work, but a launch with fewer pairs than the GPU can hold at once (two
+// workgroups per compute unit) leaves compute units idle and makes every workgroup walk two tiles: such a launch
+// deals single tiles instead.
+static PrefillParams with_units(const PrefillParams& p0) {
+    PrefillParams p = p0;
+    p.single_tiles = 0;
+    int dev = 0, n_cu = 0;
+    if (p.n_qtiles > 1 && hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess) {
+        const int64_t wgs = (int64_t)p.n_pairs * p.Hq * p.B * (p.n_split > 1 ? p.n_split : 1);
+        if (wgs < 2 * (int64_t)n_cu) {
+            p.single_tiles = 1;
+            p.n_pairs = p.n_qtiles;
+        }
+    }
+    return p;
+}
+
 template <int D>
-static int launch_prefill(const PrefillParams& p, hipStream_t stream) {
-    // one workgroup per PAIR of query tiles, 1-D in x (see the id remap); y = share of the keys
+static int launch_prefill(const PrefillParams& p0, hipStream_t stream) {
+    const PrefillParams p = with_units(p0);
+    // one workgroup per PAIR of query tiles (or per tile), 1-D in x (see the id remap); y = share of the keys
     dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B), (unsigned)(p.n_split > 1 ? p.n_split : 1));
     dim3 block(kPfWaves * 64);
     if (p.mask_mode == MI355_MASK_CAUSAL)
@@ -538,7 +590,8 @@ static int launch_merge(const PrefillParams& p, int D, hipStream_t stream) {
 }
 
 template <int D>
-static int launch_prefill_paged(const PrefillParams& p, hipStream_t stream) {
+static int launch_prefill_paged(const PrefillParams& p0, hipStream_t stream) {
+    const PrefillParams p = with_units(p0);
     dim3 grid((unsigned)(p.n_pairs * p.Hq * p.B), (unsigned)(p.n_split > 1 ? p.n_split : 1));
     hipLaunchKernelGGL((prefill_fwd_kernel<D, MI355_MASK_CAUSAL, true>), grid, dim3(kPfWaves * 64), 0, stream, p);
     return (int)hipGetLastError();
@@ -630,6 +683,7 @@ static int prefill_common(const void* q, const void* k, const void* v, void* out
     p.mask_mode = mask_mode;
     p.n_qtiles = (Sq_max + kBM - 1) / kBM;
     p.n_pairs = (p.n_qtiles + 1) / 2;
+    p.single_tiles = 0;
     p.block_table = nullptr;
     p.ctx_lens = nullptr;
     p.table_stride = 0;
@@ -735,6 +789,7 @@ extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const
     p.mask_mode = MI355_MASK_CAUSAL;
     p.n_qtiles = (Sq_max + kBM - 1) / kBM;
     p.n_pairs = (p.n_qtiles + 1) / 2;
+    p.single_tiles = 0;
     p.block_table = block_tables;
     p.ctx_lens = context_lens;
     p.table_stride = table_stride;

@@ -21,7 +21,8 @@ struct PrefillParams {
     float scale_log2;
     int mask_mode;
     int n_qtiles;
-    int n_pairs;
+    int n_pairs;                          // units per (batch, head) of the 8-wavefront kernel's grid: pairs of query tiles, or ...
+    int single_tiles;                     // ... single query tiles when this is set (launches that would not fill the GPU)
     // paged keys and values (prefill of a chunk on top of cached context): k, v are cache pools
     // (num_blocks, Hkv, 16, D); sequence b owns blocks block_table[b * table_stride + j] and ctx_lens[b] keys
     const int32_t* block_table;
