@@ -623,6 +623,40 @@ def bench_prefill_few_sequences(args):
                      "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms, "traffic": None},
     }
+    # Chunks of prompts over context that is already in the paged cache (4 sequences, 2048 new rows each over 8192
+    # tokens of context, chunk included), keys and values read through the block table: a bf16 cache by the prefill
+    # kernel itself, an fp8 cache through the gather-and-dequantise pass in front of it.
+    B, chunk, ctx = 4, 2048, 8192
+    nblk = ctx // 16
+    g2 = torch.Generator(device="cuda").manual_seed(args.seed + 12)
+    pool = B * nblk + 7
+    kc = (torch.randn(pool, Hkv, 16, D, device="cuda", generator=g2) * 0.5).to(torch.bfloat16)
+    vc = (torch.randn(pool, Hkv, 16, D, device="cuda", generator=g2) * 0.5).to(torch.bfloat16)
+    table = torch.randperm(pool, device="cuda", generator=g2)[:B * nblk].view(B, nblk).to(torch.int32)
+    lens = torch.full((B,), ctx, dtype=torch.int32, device="cuda")
+    cu = (torch.arange(B + 1, device="cuda") * chunk).to(torch.int32)
+    q = rnd(B * chunk, Hq, D)
+    k8, ks = mi355_attn.quantize_kv_cache_fp8(kc)
+    v8, vs = mi355_attn.quantize_kv_cache_fp8(vc)
+    flops = 4.0 * Hq * D * B * (chunk * (ctx - chunk) + chunk * chunk / 2.0)
+    for name, fn, kernel in (
+            ("paged_chunks_4x2048_over_8192",
+             lambda: mi355_attn.flash_attn_paged_prefill(q, kc, vc, cu, table, lens, chunk, kv_splits=1),
+             "prefill_fwd_w64_kernel<causal, block table>"),
+            ("paged_chunks_4x2048_over_8192_fp8",
+             lambda: mi355_attn.flash_attn_paged_prefill(q, k8, v8, cu, table, lens, chunk, k_scale=ks, v_scale=vs,
+                                                         total_context=B * ctx, kv_splits=1),
+             "gather_kv_fp8_kernel + prefill_fwd_w64_kernel<causal>")):
+        wall_ms, dev_ms = timed(fn, steps, warmup, BURN_MS)
+        out[name] = {
+            "value": flops / wall_ms / 1e9, "unit": "TFLOP/s", "ms_per_step": wall_ms, "dtype": "bf16",
+            "algorithmic_flops": flops, "kv_splits": 1,
+            "config": {"workload": "causal prefill of 4 chunks of 2048 rows over 8192 tokens of paged context each, "
+                                   "32 q / 8 kv heads, head_dim 128, block 16" + (", fp8-e4m3 cache" if name.endswith("fp8") else "")},
+            "roofline": {"bound": "mfma", "kernel": kernel, "achieved": flops / dev_ms / 1e9, "peak": MFMA_BF16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": flops / dev_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, "device_ms": dev_ms,
+                         "traffic": None},
+        }
     return out
 
 

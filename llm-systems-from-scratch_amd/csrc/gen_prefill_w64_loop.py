@@ -63,6 +63,13 @@ Register map (physical, fixed; the block loads them itself from its operands, se
   AGPRs directly and the MFMAs take them as A operands, which leaves the vector registers to the compiler
   s[36:37] / s[38:39] global address of the wavefront's first DMA row of K[t+2] / V[t+1] (advanced per tile),
   s40 / s41 bytes from one tile to the next in K / V, s42 "a row sum reached 2"; every other scalar is a named operand
+
+The block-table variant (W64_LOOP_PAGED: K and V live in a paged cache of 16-row blocks, and a wavefront's share of a
+tile -- 16 rows -- is exactly one block).  It differs in where the two addresses come from, nothing else: operand
+`ids` holds, in lane l, the physical block of this wavefront's share of tile (first tile of this entry) + 1 + l;
+s40 / s41 are the lanes of K[t+2] / V[t+1]; after a tensor's four requests its lane moves on by one and the address
+becomes base (operands klo:khi / vlo:vhi: block 0 of the K/V head) + id * blk (operand: bytes per block), s43 / s44
+scratch.  The caller sizes an entry so that no lane beyond 63 is ever used for a request: at most 63 tiles per entry.
 """
 import os
 import sys
@@ -88,6 +95,8 @@ QREG = {"A": 136, "B": 168}
 N_ACC = 136                         # a[0:135]: what ordinary code reaches through the snippets
 N_AGPRS = 248
 KPTR, VPTR, FLAG, KSTEP16, VSTEP16 = 36, 38, 42, 40, 41
+KLANE, VLANE, PTMP = 40, 41, 43     # block-table variant: lanes of `ids` for K[t+2] / V[t+1]; two scratch registers
+PAGED = False                       # which variant is being generated
 K_TILE = 16384                      # bytes of one K (or V) tile in LDS: 64 rows x 256 bytes
 ROW = 256
 NONE = {"A": False, "B": False}
@@ -292,8 +301,25 @@ def dma_chunks(which, buf):
             c = [f"s_add_u32 m0, %[ldsdst], {lds0 + j * 1024}", "s_nop 0"]
             c.append(f"global_load_lds_dwordx4 v{DMAOFF + j0 + j}, s[{ptr}:{ptr + 1}]")
             chunks.append(c)
-        chunks.append([f"s_add_u32 s{ptr}, s{ptr}, s{step}", f"s_addc_u32 s{ptr + 1}, s{ptr + 1}, 0"])
+        if PAGED:
+            lane = KLANE if name == "k" else VLANE
+            addr = block_address(name)
+            chunks.append([f"s_add_u32 s{lane}, s{lane}, 1"] + addr[:2])
+            chunks.append(addr[2:])
+        else:
+            chunks.append([f"s_add_u32 s{ptr}, s{ptr}, s{step}", f"s_addc_u32 s{ptr + 1}, s{ptr + 1}, 0"])
     return chunks
+
+
+def block_address(name):
+    """Block-table variant: s[ptr:ptr+1] of tensor `name` <- base + ids[lane] * blk.  (A scalar instruction may read
+    the register that v_readlane wrote right away; the address is read by a memory instruction only much later.)"""
+    ptr, lane, lo, hi = (KPTR, KLANE, "%[klo]", "%[khi]") if name == "k" else (VPTR, VLANE, "%[vlo]", "%[vhi]")
+    return [f"v_readlane_b32 s{PTMP}, %[ids], s{lane}",
+            f"s_mul_hi_u32 s{PTMP + 1}, s{PTMP}, %[blk]",
+            f"s_mul_i32 s{PTMP}, s{PTMP}, %[blk]",
+            f"s_add_u32 s{ptr}, {lo}, s{PTMP}",
+            f"s_addc_u32 s{ptr + 1}, {hi}, s{PTMP + 1}"]
 
 
 def wait_and_meet(e):
@@ -595,16 +621,25 @@ def entry(e):
             e.raw(f"s_mul_i32 s{VSTEP16}, %[vstep], {j}")
             e.raw(f"v_add_u32 v{DMAOFF + j}, s{KSTEP16}, v{DMAOFF + j}")
             e.raw(f"v_add_u32 v{DMAOFF + 4 + j}, s{VSTEP16}, v{DMAOFF + 4 + j}")
-    e.raw(f"s_lshl_b32 s{KSTEP16}, %[kstep], 4")          # a tile is 64 rows = 16 steps of 4 rows
-    e.raw(f"s_lshl_b32 s{VSTEP16}, %[vstep], 4")
-    e.raw(f"s_mov_b32 s{KPTR}, %[klo]")
-    e.raw(f"s_mov_b32 s{KPTR + 1}, %[khi]")
-    e.raw(f"s_mov_b32 s{VPTR}, %[vlo]")
-    e.raw(f"s_mov_b32 s{VPTR + 1}, %[vhi]")
+    if PAGED:                                              # lane 0 of `ids` is tile + 1: V[t+1] lane 0, K[t+2] lane 1
+        e.raw(f"s_mov_b32 s{KLANE}, 1")
+        e.raw(f"s_mov_b32 s{VLANE}, 0")
+        for name in "kv":
+            for x in block_address(name):
+                e.raw(x)
+    else:
+        e.raw(f"s_lshl_b32 s{KSTEP16}, %[kstep], 4")          # a tile is 64 rows = 16 steps of 4 rows
+        e.raw(f"s_lshl_b32 s{VSTEP16}, %[vstep], 4")
+        e.raw(f"s_mov_b32 s{KPTR}, %[klo]")
+        e.raw(f"s_mov_b32 s{KPTR + 1}, %[khi]")
+        e.raw(f"s_mov_b32 s{VPTR}, %[vlo]")
+        e.raw(f"s_mov_b32 s{VPTR + 1}, %[vhi]")
     e.raw(f"s_mov_b32 s{FLAG}, 0")
 
 
-def generate():
+def generate(paged=False):
+    global PAGED
+    PAGED = paged
     e = Emitter()
     entry(e)
     # first K fragments of the tile the block starts with (its buffer is the tile's parity)
@@ -731,8 +766,9 @@ def snippets():
 
 HEADER = '''// GENERATED by gen_prefill_w64_loop.py -- do not edit; change the generator and run it again.
 // Assembly of prefill_fwd_w64.hip: W64_LOOP is the hand-scheduled loop over the K/V tiles (register map, pipeline
-// and hand-over protocol: see the generator); the other macros are the small statements through which ordinary
-// code reaches the accumulators that live in the AGPRs.
+// and hand-over protocol: see the generator), W64_LOOP_PAGED the same loop with K and V read through a block table;
+// the other macros are the small statements through which ordinary code reaches the accumulators that live in the
+// AGPRs.
 '''
 
 
@@ -746,9 +782,11 @@ def main(out_path=None):
     here = os.path.dirname(os.path.abspath(__file__))
     out_path = out_path or os.path.join(here, "prefill_w64_asm.inc")
     lines = generate()
+    paged = generate(paged=True)
     with open(out_path, "w") as f:
         f.write(HEADER)
         f.write(as_macro("W64_LOOP", lines))
+        f.write(as_macro("W64_LOOP_PAGED", paged))
         for name, body in snippets().items():
             f.write(as_macro(name, body))
         acc = ", ".join('"a%d"' % i for i in range(N_AGPRS))

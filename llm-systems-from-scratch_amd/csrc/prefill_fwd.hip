@@ -798,7 +798,10 @@ extern "C" int mi355_prefill_paged_fwd(const void* q, const void* k_cache, const
     if (int e = set_split(p, D, n_split, total_q_rows, workspace, workspace_bytes, -1)) return e;
     if ((int64_t)p.n_pairs * Hq * B > 0x7fffffffLL) return set_error(MI355_EINVAL, "prefill_paged: too many workgroups");
     hipStream_t s = (hipStream_t)stream;
-    int rc = D == 128 ? launch_prefill_paged<128>(p, s) : (D == 64 ? launch_prefill_paged<64>(p, s) : launch_prefill_paged<32>(p, s));
+    // head_dim 128: the kernel with 64 queries per wavefront, which reads the block table too
+    int rc;
+    if (D == 128 && prefill_w64_takes(p)) rc = launch_prefill_w64(p, s);
+    else rc = D == 128 ? launch_prefill_paged<128>(p, s) : (D == 64 ? launch_prefill_paged<64>(p, s) : launch_prefill_paged<32>(p, s));
     if (rc == 0 && p.n_split > 1) rc = launch_merge(p, D, s);
     if (rc != 0) return set_error(rc, hipGetErrorString((hipError_t)rc));
     return MI355_OK;

@@ -146,6 +146,15 @@ __device__ __forceinline__ void load_bounds(const int32_t* cu_q, const int32_t* 
     k_hi = kb[1];
 }
 
+// One int32 through the scalar cache (block-table entries and context lengths: they do not change while the kernel
+// runs).  An ordinary load here would be a vector load, and the wait the compiler puts in front of its use would also
+// wait for every direct-to-LDS request in flight.
+__device__ __forceinline__ int load_scalar_i32(const int32_t* ptr) {
+    int v;
+    asm volatile("s_nop 4\n\ts_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(v) : "s"(ptr) : "memory");
+    return v;
+}
+
 // heads_per_wg: how the four wavefronts of a workgroup divide a job.
 //   1: a job is 256 query rows of one head, 64 rows per wavefront.  Under a causal mask the wavefronts then see
 //      different numbers of K/V tiles -- in the last four tile steps of a job one to three of them have nothing to
@@ -153,8 +162,14 @@ __device__ __forceinline__ void load_bounds(const int32_t* cu_q, const int32_t* 
 //   4: a job is 64 query rows of FOUR query heads that share a K/V head, one head per wavefront.  The same K/V tiles
 //      serve all four, every wavefront sees the same keys, nobody waits: the launch code takes this whenever a K/V
 //      head has a multiple of four query heads and the mask is causal.
-template <bool CAUSAL>
+// PAGED: K and V are pools of 16-row blocks (num_blocks, Hkv, 16, D) read through a block table (queries and outputs
+// packed; always causal, bottom-right aligned).  A wavefront's share of a K/V tile -- 16 rows -- is exactly one
+// block, so a tile costs every wavefront one table entry: ordinary code fetches it with a scalar load, the assembly
+// loop takes it from a register that holds the entries of the next 64 tiles, one per lane (the loop then runs at
+// most 63 tiles per entry and is entered again with the next window).
+template <bool CAUSAL, bool PAGED>
 __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(PrefillParams p, int tiles_per_unit, int heads_per_wg) {
+    static_assert(CAUSAL || !PAGED, "the block-table variant is causal");
     constexpr int D = kWD, NS = D / 16, NDT = D / 32, CPR = D / 8;
     constexpr float kBias = 32.0f;             // the largest weight sits at 2^-kBias when a reference is set
     constexpr float kUnderflow = 0x1p-92f;     // a row sum below this may have lost terms (see the file header)
@@ -200,6 +215,7 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         const __bf16 *qb, *kb, *vb;
         __bf16* ob;
         float* lb;                       // row 0 of this (sequence, head) in the log-sum-exp output, or null
+        const int32_t* tab;              // PAGED: the sequence's row of the block table (kb, vb: block 0 of the K/V head)
         int sq, sk, q0;
         int split;                       // which share of the query tile's K/V tiles (0 when the keys are not split)
     };
@@ -332,9 +348,15 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
         const int qs1 = (int)a->qs[1], ks1 = (int)a->ks[1], vs1 = (int)a->vs[1], os1 = (int)a->os[1], ls1 = (int)a->ls[1];
         if (a->cu_q) {
             int q_start, q_end, k_start, k_end;
-            load_bounds(a->cu_q, a->cu_k, b, q_start, q_end, k_start, k_end);
+            load_bounds(a->cu_q, PAGED ? a->cu_q : a->cu_k, b, q_start, q_end, k_start, k_end);
             j.sq = q_end - q_start;
             j.sk = k_end - k_start;
+            if constexpr (PAGED) {
+                // a length beyond what the table row addresses is cut, never chased
+                j.sk = max(0, min(load_scalar_i32(a->ctx_lens + b), 16 * a->max_blocks));
+                j.tab = a->block_table + (int64_t)b * a->table_stride;
+                k_start = 0;
+            }
             j.qb = a->q + ((int64_t)q_start * qs2 + (int64_t)h * qs1);
             j.kb = a->k + ((int64_t)k_start * ks2 + (int64_t)hk * ks1);
             j.vb = a->v + ((int64_t)k_start * vs2 + (int64_t)hk * vs1);
@@ -375,12 +397,35 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
     const uint32_t dma_row_k = (uint32_t)(ld_q * ks2 * 2), dma_row_v = (uint32_t)(ld_q * vs2 * 2);
     const uint32_t lds_dst = __builtin_amdgcn_readfirstlane(lds_address(kv_lds + wave * 4096));
     const uint32_t k_step = (uint32_t)(4 * ks2 * 2), v_step = (uint32_t)(4 * vs2 * 2);   // 4 rows, in bytes
+    const int blk_elems = Hkv * 16 * kWD;      // PAGED: elements from one block of the pool to the next
     // K (which == 0) or V (which == 1) rows of tile `tile` into that tensor's LDS buffer `buf`
     auto issue_rows = [&](const Job& jb, int which, int tile, int buf) {
         const __bf16* src = which ? jb.vb : jb.kb;
         const int stride = which ? vs2 : ks2;
         const uint32_t step = which ? v_step : k_step, dma_row = which ? dma_row_v : dma_row_k;
         const uint32_t dst = lds_dst + (2 * which + buf) * kWTile;
+        if constexpr (PAGED) {
+            // this wavefront's 16 rows are logical block 4 * tile + wave of the sequence.  Rows past the last key
+            // re-read the last key's row (finite; their scores are masked); a block past the last one is never looked
+            // up (its table entry need not exist); an entry that points outside the pool is pulled back into it.
+            int last = max(jb.sk - 1, 0);
+            asm volatile("" : "+s"(last));          // (keeps this arithmetic at the request, see below)
+            const int last_b = last >> 4;
+            int bidx = tile * (kWBN / 16) + wave, rin_max = 15;
+            if (bidx >= last_b) {
+                bidx = last_b;
+                rin_max = last & 15;
+            }
+            int phys = load_scalar_i32(jb.tab + bidx);
+            phys = min(max(phys, 0), args()->num_blocks - 1);
+            const unsigned char* base = reinterpret_cast<const unsigned char*>(src + (int64_t)phys * blk_elems);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t row = (uint32_t)min(4 * j + ld_q, rin_max);
+                dma_to_lds_16_m0(base, row * (uint32_t)kWRow + (uint32_t)((ld_c0 ^ j) << 4), dst + j * 1024);
+            }
+            return;
+        }
         if (tile * kWBN + kWBN <= jb.sk) {
             const unsigned char* base = reinterpret_cast<const unsigned char*>(src + (int64_t)(tile * kWBN + 16 * wave) * stride);
 #pragma unroll
@@ -766,8 +811,23 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
                 continue;
             }
             // ---- the hand-scheduled loop over tiles [tile, n_loop); leaves after a tile that took a row sum to 2 ----
-            const uint64_t kptr = (uint64_t)(uintptr_t)(cur.kb + (int64_t)((tile + 2) * kWBN + 16 * wave) * ks2);
-            const uint64_t vptr = (uint64_t)(uintptr_t)(cur.vb + (int64_t)((tile + 1) * kWBN + 16 * wave) * vs2);
+            // (PAGED: at most 63 tiles per entry, see the block ids below; the loop is then entered again)
+            const int n_stop = PAGED ? min(n_loop, tile + 63) : n_loop;
+            uint64_t kptr, vptr;
+            int v_ids = 0;
+            if constexpr (PAGED) {
+                // Block ids of this wavefront's shares of tiles tile + 1 + lane (the loop requests V[t+1] and K[t+2]),
+                // never from past the sequence's last block, pulled into the pool.  The bases are block 0 of the K/V head.
+                int last = max(sk - 1, 0), first = tile + 1;
+                asm volatile("" : "+s"(last), "+s"(first));
+                const int bidx = min((first + lane) * (kWBN / 16) + wave, last >> 4);
+                v_ids = min(max(cur.tab[bidx], 0), args()->num_blocks - 1);
+                kptr = (uint64_t)(uintptr_t)cur.kb;
+                vptr = (uint64_t)(uintptr_t)cur.vb;
+            } else {
+                kptr = (uint64_t)(uintptr_t)(cur.kb + (int64_t)((tile + 2) * kWBN + 16 * wave) * ks2);
+                vptr = (uint64_t)(uintptr_t)(cur.vb + (int64_t)((tile + 1) * kWBN + 16 * wave) * vs2);
+            }
             // mask thresholds for the first masked tile the loop will meet: a key at index j of that tile is kept by
             // query i of the wavefront iff j <= i + (qw0 + coff - k0) and j < sk - k0 (the lane part 4*kg of a key's
             // index is folded in)
@@ -780,19 +840,33 @@ __global__ __launch_bounds__(kWWaves * 64, 1) void prefill_fwd_w64_kernel(Prefil
             uint32_t v_rowk = dma_row_k, v_rowv = dma_row_v, v_c0s = (uint32_t)(ld_c0 << 4);
             int status;
             int tile_s = __builtin_amdgcn_readfirstlane(tile);
-            asm volatile(W64_LOOP
-                : [tile] "+&s"(tile_s), [t2] "=&s"(status),
-                  [nb0] "+v"(v_nb0), [nb1] "+v"(v_nb1), [suma] "+v"(v_sum), [k0] "+v"(v_k0), [vlo0] "+v"(v_vlo),
-                  [vhi0] "+v"(v_vhi), [rowk] "+v"(v_rowk), [rowv] "+v"(v_rowv), [c0s] "+v"(v_c0s),
-                  [thr0] "+v"(v_thr0), [thr1] "+v"(v_thr1)
-                : [n_tiles] "s"(__builtin_amdgcn_readfirstlane(n_tiles)), [n_end] "s"(__builtin_amdgcn_readfirstlane(n_loop)),
-                  [n_pipe] "s"(__builtin_amdgcn_readfirstlane(min(n_plain, n_loop))), [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)),
-                  [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)),
-                  [kstep] "s"(__builtin_amdgcn_readfirstlane(k_step)), [vstep] "s"(__builtin_amdgcn_readfirstlane(v_step)),
-                  [ldsdst] "s"(lds_dst), [scale] "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, p.scale_log2))),
-                  [klo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)kptr)), [khi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kptr >> 32))),
-                  [vlo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)vptr)), [vhi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(vptr >> 32)))
-                : "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS);
+#define W64_LOOP_OUTPUTS                                                                                              \
+    [tile] "+&s"(tile_s), [t2] "=&s"(status), [nb0] "+v"(v_nb0), [nb1] "+v"(v_nb1), [suma] "+v"(v_sum),               \
+        [k0] "+v"(v_k0), [vlo0] "+v"(v_vlo), [vhi0] "+v"(v_vhi), [rowk] "+v"(v_rowk), [rowv] "+v"(v_rowv),            \
+        [c0s] "+v"(v_c0s), [thr0] "+v"(v_thr0), [thr1] "+v"(v_thr1)
+#define W64_LOOP_INPUTS                                                                                               \
+    [n_tiles] "s"(__builtin_amdgcn_readfirstlane(n_tiles)), [n_end] "s"(__builtin_amdgcn_readfirstlane(n_stop)),      \
+        [n_pipe] "s"(__builtin_amdgcn_readfirstlane(min(n_plain, n_stop))),                                           \
+        [n_mask] "s"(__builtin_amdgcn_readfirstlane(n_mask)), [aligned] "s"(__builtin_amdgcn_readfirstlane(aligned)), \
+        [kstep] "s"(__builtin_amdgcn_readfirstlane(k_step)), [vstep] "s"(__builtin_amdgcn_readfirstlane(v_step)),     \
+        [ldsdst] "s"(lds_dst), [scale] "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, p.scale_log2))), \
+        [klo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)kptr)),                                                    \
+        [khi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kptr >> 32))),                                            \
+        [vlo] "s"(__builtin_amdgcn_readfirstlane((uint32_t)vptr)),                                                    \
+        [vhi] "s"(__builtin_amdgcn_readfirstlane((uint32_t)(vptr >> 32)))
+#define W64_LOOP_CLOBBERS "memory", "vcc", "scc", "s36", "s37", "s38", "s39", "s40", "s41", "s42", W64_CLOBBER_ACC, W64_CLOBBER_LOOP_VGPRS
+            if constexpr (PAGED) {
+                asm volatile(W64_LOOP_PAGED
+                             : W64_LOOP_OUTPUTS
+                             : W64_LOOP_INPUTS, [ids] "v"(v_ids),
+                               [blk] "s"(__builtin_amdgcn_readfirstlane((uint32_t)blk_elems * 2u))
+                             : W64_LOOP_CLOBBERS, "s43", "s44");
+            } else {
+                asm volatile(W64_LOOP : W64_LOOP_OUTPUTS : W64_LOOP_INPUTS : W64_LOOP_CLOBBERS);
+            }
+#undef W64_LOOP_OUTPUTS
+#undef W64_LOOP_INPUTS
+#undef W64_LOOP_CLOBBERS
             tile = tile_s;
             // status 0: tiles up to n_loop done.  1: tiles up to `tile` done, and the last of them took a row sum to 2.
             if (status != 0) {
@@ -969,10 +1043,12 @@ int launch_prefill_w64(const PrefillParams& p, hipStream_t stream) {
     int grid = most_units < n_cu ? (int)most_units : n_cu;
     if (grid >= 8) grid -= grid % 8;          // whole number of workgroups per XCD
     dim3 block(kWWaves * 64);
-    if (p.mask_mode == MI355_MASK_CAUSAL)
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit, heads_per_wg);
+    if (p.block_table)
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true, true>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit, heads_per_wg);
+    else if (p.mask_mode == MI355_MASK_CAUSAL)
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<true, false>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit, heads_per_wg);
     else
-        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit, heads_per_wg);
+        hipLaunchKernelGGL((prefill_fwd_w64_kernel<false, false>), dim3((unsigned)grid), block, 0, stream, p, tiles_per_unit, heads_per_wg);
     return (int)hipGetLastError();
 }
 

@@ -702,6 +702,41 @@ def test_paged_prefill_ragged_chunks_match_the_oracle(ops, D, Hq, Hkv):
     assert ret is out and torch.equal(out, got)
 
 
+@pytest.mark.parametrize("Hq,Hkv,splits", [(8, 2, 1), (4, 4, 1), (6, 2, 1), (8, 2, 3)])
+def test_paged_prefill_head_dim_128_long_contexts_through_the_block_table(ops, Hq, Hkv, splits):
+    """head_dim 128 runs on the 64-query kernel, whose tile loop takes its block ids from a register that covers 63
+    tiles at a time: contexts of more than 63, 126 and 189 tiles (so the loop is left and entered again with the next
+    ids), chunk ends inside a block and inside a tile, one token over a long context, a chunk that is the whole
+    context; four query heads per K/V head (the four wavefronts share the rows), one (they share the head) and three;
+    keys split over workgroups; garbage in unused blocks, in the tail of the last block and in the table tail."""
+    ctx = [9000, 2100, 12300, 64, 4033, 8129]
+    chunk = [300, 2100, 1, 64, 257, 520]
+    print(f"case: paged prefill D=128 long contexts Hq={Hq} Hkv={Hkv} splits={splits}", flush=True)
+    D = 128
+    _, kc, vc, bt, cl = orc.make_paged_case(batch=len(ctx), n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, block_size=16,
+                                            context_lens=ctx, pool_factor=1.2, seed=31, dtype=torch.bfloat16)
+    cu = torch.tensor([0] + list(torch.tensor(chunk).cumsum(0)), dtype=torch.int32)
+    q = rnd(int(cu[-1]), Hq, D, seed=32)
+    ref = orc.paged_prefill_reference(q, kc, vc, cu, bt, cl)
+    used = torch.zeros(kc.shape[0], dtype=torch.bool)
+    bt2, kc2, vc2 = bt.clone(), kc.clone(), vc.clone()
+    for b, c in enumerate(ctx):
+        nb = (c + 15) // 16
+        used[bt[b, :nb].long()] = True
+        bt2[b, nb:] = 2 ** 30
+        if c % 16:
+            last = int(bt[b, (c - 1) // 16])
+            kc2[last, :, c % 16:] = float("nan")
+            vc2[last, :, c % 16:] = float("inf")
+    kc2[~used] = float("nan")
+    vc2[~used] = float("nan")
+    dev = "cuda:0"
+    got = ops.flash_attn_paged_prefill(q.to(dev), kc2.to(dev), vc2.to(dev), cu.to(dev), bt2.to(dev), cl.to(dev), max(chunk),
+                                       kv_splits=splits)
+    torch.cuda.synchronize()
+    check(got, ref, what="paged prefill, long contexts")
+
+
 @pytest.mark.parametrize("D,Hq,Hkv", [(128, 8, 2), (64, 4, 4), (128, 32, 8)])
 def test_paged_prefill_over_an_fp8_cache_matches_the_oracle(ops, D, Hq, Hkv):
     """The same ragged chunks over an fp8-e4m3 cache with per-(block, kv head) scales: gathered and dequantised by
