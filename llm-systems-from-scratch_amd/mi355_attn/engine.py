@@ -60,6 +60,7 @@ class PrefillPlan:
     tables: torch.Tensor | None = None        # (B, max_blocks) int32
     context_lens: torch.Tensor | None = None  # (B,) int32: tokens in the cache, this chunk included
     total_context: int = 0                    # their sum (sizes the dequantised rows of an fp8 cache)
+    cu_context: torch.Tensor | None = None    # (B+1,) int32: their running sum (fp8 cache: where each sequence's rows start)
 
 
 @dataclass
@@ -211,6 +212,11 @@ class PagedAttentionEngine:
             plan.tables = rows.to(dev)
             plan.context_lens = torch.tensor([self.lengths[sid] for sid in seq_ids], dtype=torch.int32, device=dev)
             plan.total_context = sum(self.lengths[sid] for sid in seq_ids)
+            if self.kv_dtype != "bf16":
+                run = [0]
+                for sid in seq_ids:
+                    run.append(run[-1] + self.lengths[sid])
+                plan.cu_context = torch.tensor(run, dtype=torch.int32, device=dev)
         return plan
 
     def _reserve_decode(self, seq_ids):
@@ -289,7 +295,8 @@ class PagedAttentionEngine:
         if plan.tables is not None:
             q_rot = self._write_cache(layer, plan, q, k, v)
             scales = {} if self.kv_dtype == "bf16" else {"k_scale": self.k_scales[layer], "v_scale": self.v_scales[layer],
-                                                         "total_context": plan.total_context}
+                                                         "total_context": plan.total_context,
+                                                         "cu_seqlens_k": plan.cu_context}
             return ops.flash_attn_paged_prefill(q_rot, self.k_caches[layer], self.v_caches[layer], plan.cu_seqlens,
                                                 plan.tables, plan.context_lens, plan.max_len, **scales)
         q_rot, k_rot = self._write_cache(layer, plan, q, k, v, k_out=True)

@@ -533,7 +533,7 @@ def paged_attention_decode(q, k_cache, v_cache, block_tables, context_lens, *, s
 
 def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, context_lens, max_seqlen_q, *,
                              softmax_scale=None, out=None, max_context=None, kv_splits=None, workspace=None,
-                             k_scale=None, v_scale=None, total_context=None):
+                             k_scale=None, v_scale=None, total_context=None, cu_seqlens_k=None):
     """Causal prefill of a chunk of new tokens over context that already sits in a paged cache.
 
     q (T,Hq,D) bf16, packed, contiguous heads (token stride free): sequence b owns rows
@@ -548,13 +548,15 @@ def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, co
     of paged_attention_decode): the sequences' keys and values are first gathered and dequantised into packed
     bf16 rows (mi355_gather_kv_fp8; value = bf16(fp8 * scale)), then attended to by the packed prefill kernels.
     total_context (host int, optional): an upper bound on sum(context_lens) that sizes those rows (default
-    batch * max_context).
+    batch * max_context); cu_seqlens_k (int32 (B+1,), optional): the running sum of the context lengths, if the
+    caller has it on the device already (else it is computed here, a few small launches per call).
     The mathematics is that of llm-core/llm_core/model.py:308-325 with the mask of :384; the reference
     itself would re-run the whole prefix (model.py:218)."""
     _require_gpu_bf16("q", q)
     if k_scale is not None or v_scale is not None:
         return _paged_prefill_fp8(q, k_cache, v_cache, k_scale, v_scale, cu_seqlens_q, block_tables, context_lens,
-                                  max_seqlen_q, softmax_scale, out, max_context, kv_splits, workspace, total_context)
+                                  max_seqlen_q, softmax_scale, out, max_context, kv_splits, workspace, total_context,
+                                  cu_seqlens_k)
     if q.dim() != 3 or q.stride(2) != 1 or q.stride(1) != q.shape[2]:
         raise ValueError("q must be (tokens, heads, d_head) with contiguous heads")
     T, Hq, D = q.shape
@@ -610,12 +612,14 @@ def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, co
     return out
 
 
-def gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens, *, max_context=None, total_context=None):
+def gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens, *, max_context=None, total_context=None,
+                  cu_seqlens_k=None):
     """The keys and values of a batch of sequences out of an fp8 paged cache, dequantised, as packed bf16 rows.
     Returns (k (rows,Hkv,D), v (rows,Hkv,D), cu_seqlens_k int32 (B+1,)): sequence b owns rows
     [cu_seqlens_k[b], cu_seqlens_k[b+1]), cu_seqlens_k the running sum of min(context_lens, max_context);
-    rows = total_context when given (a host-side bound on that sum), else batch * max_context.  Nothing is read
-    back from the device."""
+    rows = total_context when given (a host-side bound on that sum), else batch * max_context.  A caller that
+    already holds that running sum on the device (a serving loop computes it once per step, not once per layer)
+    passes it as cu_seqlens_k.  Nothing is read back from the device."""
     for n, c in (("k_cache", k_cache), ("v_cache", v_cache)):
         if c.dtype not in (torch.uint8, torch.float8_e4m3fn) or c.dim() != 4 or c.shape[2] != _BLOCK or not c.is_contiguous() \
                 or not c.is_cuda:
@@ -641,9 +645,15 @@ def gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens
     max_context = width if max_context is None else min(int(max_context), width)
     rows = B * max_context if total_context is None else min(int(total_context), B * max_context)
     dev = k_cache.device
-    cu_k = torch.zeros(B + 1, dtype=torch.int32, device=dev)
-    if B:
-        cu_k[1:] = torch.cumsum(context_lens.clamp(max=max_context), 0)
+    if cu_seqlens_k is not None:
+        if cu_seqlens_k.dtype != torch.int32 or cu_seqlens_k.shape != (B + 1,) or not cu_seqlens_k.is_contiguous() \
+                or cu_seqlens_k.device != dev:
+            raise ValueError("cu_seqlens_k must be a contiguous int32 (batch + 1,) tensor on the caches' device")
+        cu_k = cu_seqlens_k
+    else:
+        cu_k = torch.zeros(B + 1, dtype=torch.int32, device=dev)
+        if B:
+            cu_k[1:] = torch.cumsum(context_lens.clamp(max=max_context), 0)
     k_lin = torch.empty(max(rows, 1), Hkv, D, dtype=torch.bfloat16, device=dev)
     v_lin = torch.empty(max(rows, 1), Hkv, D, dtype=torch.bfloat16, device=dev)
     if B and rows:
@@ -657,7 +667,7 @@ def gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens
 
 
 def _paged_prefill_fp8(q, k_cache, v_cache, k_scale, v_scale, cu_seqlens_q, block_tables, context_lens, max_seqlen_q,
-                       softmax_scale, out, max_context, kv_splits, workspace, total_context):
+                       softmax_scale, out, max_context, kv_splits, workspace, total_context, cu_seqlens_k=None):
     """flash_attn_paged_prefill over an fp8 cache: gather + dequantise, then the packed prefill with more keys than
     queries per sequence (bottom-right aligned causal mask)."""
     if q.dim() != 3:
@@ -667,7 +677,7 @@ def _paged_prefill_fp8(q, k_cache, v_cache, k_scale, v_scale, cu_seqlens_q, bloc
     width = block_tables.shape[1] * _BLOCK
     max_context = width if max_context is None else min(int(max_context), width)
     k_lin, v_lin, cu_k = gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens,
-                                       max_context=max_context, total_context=total_context)
+                                       max_context=max_context, total_context=total_context, cu_seqlens_k=cu_seqlens_k)
     res = flash_attn_varlen_prefill(q, k_lin, v_lin, cu_seqlens_q, cu_k, max_seqlen_q, max_context, causal=True,
                                     softmax_scale=softmax_scale, kv_splits=kv_splits, workspace=workspace)
     if out is not None:

@@ -771,6 +771,11 @@ def test_paged_prefill_over_an_fp8_cache_matches_the_oracle(ops, D, Hq, Hkv):
     torch.cuda.synchronize()
     check(got, ref8, what="paged prefill over fp8, oracle on the dequantised cache")
     check(tight, ref8, what="paged prefill over fp8, rows sized by total_context")
+    # the caller's own running sum of the context lengths instead of one computed per call
+    cu_ctx = torch.tensor([0] + list(torch.tensor(ctx).cumsum(0)), dtype=torch.int32, device=dev)
+    given = ops.flash_attn_paged_prefill(*args, k_scale=ks.to(dev), v_scale=vs.to(dev), total_context=sum(ctx), kv_splits=1,
+                                         cu_seqlens_k=cu_ctx)
+    assert torch.equal(given, tight)
     e16 = (got.float().cpu() - ref16).abs()
     assert bool((e16 <= 0.15 + 2.0 ** -4 * ref16.abs()).all()), float(e16.max())
     assert float((got.float().cpu() - ref16).pow(2).mean().sqrt() / ref16.pow(2).mean().sqrt()) <= 0.06
