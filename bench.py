@@ -206,7 +206,25 @@ def bench_producers(args):
                      "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS, "device_ms": dev_ms,
                      "traffic": _traffic("rope_and_cache_fp8")},
     }
-    del q, k, v, q_out, k8, v8
+    # --- gather_kv_fp8: the way back for a prompt chunk over an fp8 cache: the 8 sequences' 4096 tokens each out of that
+    # pool, dequantised, as packed bf16 rows
+    tables = perm.view(B, S // 16).to(torch.int32)
+    lens = torch.full((B,), S, dtype=torch.int32, device=dev)
+    cu_k = (torch.arange(B + 1, device=dev) * S).to(torch.int32)
+    k_lin = torch.empty(T, Hkv, D, dtype=torch.bfloat16, device=dev)
+    v_lin = torch.empty_like(k_lin)
+    wall_ms, dev_ms = timed(lambda: mi355_attn.gather_kv_fp8(k8, v8, ks, vs, tables, lens, total_context=T, cu_seqlens_k=cu_k,
+                                                             out=(k_lin, v_lin)), args.steps, args.warmup, BURN_MS)
+    nbytes = (k.numel() + v.numel()) * 3 + 2 * ks.numel() * 4 + tables.numel() * 4
+    res["gather_kv_fp8"] = {
+        "value": nbytes / wall_ms / 1e6, "unit": "GB/s", "ms_per_step": wall_ms, "dtype": "fp8-e4m3 -> bf16",
+        "config": {"workload": "gather + dequantise 8 sequences of 4096 tokens out of an fp8 paged cache into packed bf16 "
+                               "rows (8 kv heads, head_dim 128), blocks a random permutation", "algorithmic_bytes": nbytes},
+        "roofline": {"bound": "hbm", "kernel": "gather_kv_fp8_kernel", "achieved": nbytes / dev_ms / 1e6,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": nbytes / dev_ms / 1e6 / HBM_PEAK_GBPS,
+                     "device_ms": dev_ms, "traffic": None},
+    }
+    del q, k, v, q_out, k8, v8, k_lin, v_lin
     # --- quantize_kv_fp8: a pool of configs[4]'s size (about 103k blocks x 8 kv heads x 16 x 128)
     nb = 103_000
     pool = torch.randn(nb, Hkv, 16, D, device=dev, generator=g).to(torch.bfloat16)

@@ -449,8 +449,8 @@ extern "C" int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, fl
 // Gather + dequantise: the keys and values of every sequence of a batch, read through the block tables out of an
 // fp8 cache, written as packed bf16 rows (sequence b owns rows [cu_k[b], cu_k[b+1])) -- the K/V operands of a packed
 // prefill (mi355_prefill_fwd with cu_seqlens), so that a chunk of a prompt can attend to an fp8 cache on the same
-// kernels as to bf16 tensors.  One wavefront per (sequence, logical block, kv head, K or V): a slab of 16 x D bytes in,
-// 16 rows of D bf16 out; value = bf16(fp8 * scale), the scale of the slab.  Rows at or past the context length (the
+// kernels as to bf16 tensors.  One wavefront per (sequence, logical block, kv head): a K and a V slab of 16 x D bytes in,
+// 16 rows of D bf16 out each; value = bf16(fp8 * scale), the scale of the slab.  Rows at or past the context length (the
 // tail of a sequence's last block) and rows past `max_rows` are not written.
 struct GatherFp8Params {
     const unsigned char* k_cache;
@@ -470,43 +470,55 @@ template <int D>
 __global__ __launch_bounds__(256) void gather_kv_fp8_kernel(GatherFp8Params p) {
     const int lane = threadIdx.x & 63;
     const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t n_waves = (int64_t)p.B * p.max_blocks * p.Hkv * 2;
+    const int64_t n_waves = (int64_t)p.B * p.max_blocks * p.Hkv;
     if (w >= n_waves) return;
-    const int which = (int)(w & 1);
-    const int hk = (int)((w >> 1) % p.Hkv);
-    const int64_t bj = (w >> 1) / p.Hkv;
+    const int hk = (int)(w % p.Hkv);
+    const int64_t bj = w / p.Hkv;
     const int j = (int)(bj % p.max_blocks), b = (int)(bj / p.max_blocks);
     const int ctx = min(p.ctx_lens[b], 16 * p.max_blocks);          // a length beyond what the table addresses is truncated
     if (16 * j >= ctx) return;
     int phys = p.tables[(int64_t)b * p.table_stride + j];
     phys = min(max(phys, 0), p.num_blocks - 1);                     // a corrupt table cannot leave the pool
     const int64_t slab = (int64_t)phys * p.Hkv + hk;
-    const unsigned char* src = (which ? p.v_cache : p.k_cache) + slab * (16 * D);
-    const float scale = (which ? p.v_scale : p.k_scale)[slab];
-    __bf16* out = which ? p.v_out : p.k_out;
     const int64_t row0 = (int64_t)p.cu_k[b] + 16 * j;
     constexpr int kPasses = (16 * D + 1023) / 1024;
+    // all loads of the K and the V slab first (one dependent chain for both), then the conversions and the stores
+    u32x4 raw[2][kPasses];
+    float scale[2];
 #pragma unroll
-    for (int pass = 0; pass < kPasses; ++pass) {
-        const int e = (pass * 64 + lane) * 16;                      // first of this lane's 16 elements of the slab
-        if (e >= 16 * D) break;
-        const int row = e / D, col = e % D;
-        const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + e));
-        if (16 * j + row >= ctx || row0 + row >= p.max_rows) continue;
-        uint32_t w16[8];
+    for (int which = 0; which < 2; ++which) {
+        const unsigned char* src = (which ? p.v_cache : p.k_cache) + slab * (16 * D);
+        scale[which] = (which ? p.v_scale : p.k_scale)[slab];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            // (exact: e4m3 is a subset of bf16.  The upper two bytes are shifted down and converted with the same
-            // selector: in this kernel the compiler merged the two conversions of one word that differ only in the
-            // selector, and every second pair of elements came out as a copy of the pair before it.)
-            const bf16x2 lo = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw[i], 1.0f, false);
-            const bf16x2 hi = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw[i] >> 16, 1.0f, false);
-            w16[2 * i] = pack_bf16((float)lo[0] * scale, (float)lo[1] * scale);
-            w16[2 * i + 1] = pack_bf16((float)hi[0] * scale, (float)hi[1] * scale);
+        for (int pass = 0; pass < kPasses; ++pass) {
+            const int e = (pass * 64 + lane) * 16;                  // first of this lane's 16 elements of the slab
+            raw[which][pass] = e < 16 * D ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + e)) : u32x4{0u, 0u, 0u, 0u};
         }
-        u32x4* dst = reinterpret_cast<u32x4*>(out + (row0 + row) * p.out_tok + (int64_t)hk * D + col);
-        __builtin_nontemporal_store(u32x4{w16[0], w16[1], w16[2], w16[3]}, dst);
-        __builtin_nontemporal_store(u32x4{w16[4], w16[5], w16[6], w16[7]}, dst + 1);
+    }
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        __bf16* out = which ? p.v_out : p.k_out;
+#pragma unroll
+        for (int pass = 0; pass < kPasses; ++pass) {
+            const int e = (pass * 64 + lane) * 16;
+            if (e >= 16 * D) break;
+            const int row = e / D, col = e % D;
+            if (16 * j + row >= ctx || row0 + row >= p.max_rows) continue;
+            uint32_t w16[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // (exact: e4m3 is a subset of bf16.  The upper two bytes are shifted down and converted with the same
+                // selector: in this kernel the compiler merged the two conversions of one word that differ only in the
+                // selector, and every second pair of elements came out as a copy of the pair before it.)
+                const bf16x2 lo = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw[which][pass][i], 1.0f, false);
+                const bf16x2 hi = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw[which][pass][i] >> 16, 1.0f, false);
+                w16[2 * i] = pack_bf16((float)lo[0] * scale[which], (float)lo[1] * scale[which]);
+                w16[2 * i + 1] = pack_bf16((float)hi[0] * scale[which], (float)hi[1] * scale[which]);
+            }
+            u32x4* dst = reinterpret_cast<u32x4*>(out + (row0 + row) * p.out_tok + (int64_t)hk * D + col);
+            __builtin_nontemporal_store(u32x4{w16[0], w16[1], w16[2], w16[3]}, dst);
+            __builtin_nontemporal_store(u32x4{w16[4], w16[5], w16[6], w16[7]}, dst + 1);
+        }
     }
 }
 
@@ -543,7 +555,7 @@ extern "C" int mi355_gather_kv_fp8(const void* k_cache_fp8, const void* v_cache_
     p.B = B;
     p.Hkv = Hkv;
     p.num_blocks = (int)num_blocks;
-    const int64_t n_waves = (int64_t)B * max_blocks * Hkv * 2, wgs = (n_waves + 3) / 4;
+    const int64_t n_waves = (int64_t)B * max_blocks * Hkv, wgs = (n_waves + 3) / 4;
     if (wgs > 0x7fffffffLL) return set_error(MI355_EINVAL, "gather_kv_fp8: too many blocks for one launch");
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((unsigned)wgs), block(256);

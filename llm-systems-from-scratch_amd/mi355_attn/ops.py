@@ -613,13 +613,14 @@ def flash_attn_paged_prefill(q, k_cache, v_cache, cu_seqlens_q, block_tables, co
 
 
 def gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens, *, max_context=None, total_context=None,
-                  cu_seqlens_k=None):
+                  cu_seqlens_k=None, out=None):
     """The keys and values of a batch of sequences out of an fp8 paged cache, dequantised, as packed bf16 rows.
     Returns (k (rows,Hkv,D), v (rows,Hkv,D), cu_seqlens_k int32 (B+1,)): sequence b owns rows
     [cu_seqlens_k[b], cu_seqlens_k[b+1]), cu_seqlens_k the running sum of min(context_lens, max_context);
     rows = total_context when given (a host-side bound on that sum), else batch * max_context.  A caller that
     already holds that running sum on the device (a serving loop computes it once per step, not once per layer)
-    passes it as cu_seqlens_k.  Nothing is read back from the device."""
+    passes it as cu_seqlens_k; out=(k, v) reuses two contiguous bf16 (rows, Hkv, D) tensors.  Nothing is read back
+    from the device."""
     for n, c in (("k_cache", k_cache), ("v_cache", v_cache)):
         if c.dtype not in (torch.uint8, torch.float8_e4m3fn) or c.dim() != 4 or c.shape[2] != _BLOCK or not c.is_contiguous() \
                 or not c.is_cuda:
@@ -654,8 +655,14 @@ def gather_kv_fp8(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens
         cu_k = torch.zeros(B + 1, dtype=torch.int32, device=dev)
         if B:
             cu_k[1:] = torch.cumsum(context_lens.clamp(max=max_context), 0)
-    k_lin = torch.empty(max(rows, 1), Hkv, D, dtype=torch.bfloat16, device=dev)
-    v_lin = torch.empty(max(rows, 1), Hkv, D, dtype=torch.bfloat16, device=dev)
+    if out is not None:
+        k_lin, v_lin = out
+        for n, t in (("out[0]", k_lin), ("out[1]", v_lin)):
+            if t.dtype != torch.bfloat16 or tuple(t.shape) != (max(rows, 1), Hkv, D) or not t.is_contiguous() or t.device != dev:
+                raise ValueError(f"{n} must be a contiguous bfloat16 ({max(rows, 1)}, {Hkv}, {D}) tensor on the caches' device")
+    else:
+        k_lin = torch.empty(max(rows, 1), Hkv, D, dtype=torch.bfloat16, device=dev)
+        v_lin = torch.empty(max(rows, 1), Hkv, D, dtype=torch.bfloat16, device=dev)
     if B and rows:
         with _on(k_cache, v_cache, k_scale, v_scale, block_tables, context_lens) as stream:
             rc = _lib.load().mi355_gather_kv_fp8(
