@@ -866,13 +866,16 @@ extern "C" int mi355_prefill_suggest_kv_splits(int B, int Hq, int D, int Sq_max,
         }
         return best_n;
     }
+    // the 8-wavefront kernel: a K/V tile of 64 keys takes a workgroup about 1.5 / 0.9 / 0.6 us at head_dim 128 / 64 / 32
+    // (one 4096-token prompt with 16 heads of 64: 72 us unsplit, 84 us with two shares)
+    const double tile_us = D >= 128 ? 1.5 : (D >= 64 ? 0.9 : 0.6);
     const double jobs = (double)n_pairs * Hq * B;
     const double tiles = keys_pair / kBN;
-    plain = rounds(jobs) * (tiles * 1.5 + 5.0 * halves);
+    plain = rounds(jobs) * (tiles * tile_us + 5.0 * halves);
     double best = plain * 0.85;                       // a split must win clearly
     for (int n : kCandidates) {
         if (tiles / n < 2.0 * halves) break;          // at least two tiles per share and query tile
-        const double t = rounds(jobs * n) * (tiles / n * 1.6 + 5.0 * halves) + partials(n);
+        const double t = rounds(jobs * n) * (tiles / n * tile_us * 1.07 + 5.0 * halves) + partials(n);
         if (t < best) {
             best = t;
             best_n = n;
