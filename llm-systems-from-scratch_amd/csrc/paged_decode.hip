@@ -445,11 +445,75 @@ __global__ __launch_bounds__(kCombineThreads) void paged_decode_combine_kernel(D
     *reinterpret_cast<u32x2*>(p.out + (int64_t)row * D + d) = w;
 }
 
+// Combine for sequences of many chunks (a small batch of long contexts runs short chunks, see tokens_per_wave_for: one
+// sequence of 32 K tokens has 128 of them): one workgroup per row, the chunks dealt to 256 / (D / 4) groups of lanes
+// that each reduce every kGroups-th chunk; the groups' partial sums meet in LDS.  (One thread walking 128 chunks took
+// 12 us of that sequence's 35 us step.)
+template <int D>
+__global__ __launch_bounds__(kCombineThreads) void paged_decode_combine_wide_kernel(DecodeParams p) {
+    constexpr int kLanesPerRow = D / 4;
+    constexpr int kGroups = kCombineThreads / kLanesPerRow;
+    __shared__ float s_m[kGroups], s_den[kGroups];
+    __shared__ f32x4 s_num[kGroups][kLanesPerRow];
+    const int row = blockIdx.x;                    // b * Hq + h
+    const int b = row / p.Hq;
+    const int ctx = min(p.context_lens[b], p.max_ctx);
+    const int chunk_tokens = kDecodeWaves * p.tokens_per_wave;
+    const int n_chunks = (ctx + chunk_tokens - 1) / chunk_tokens;
+    if (n_chunks <= 1) return;                   // written by the split pass (or empty); the whole workgroup leaves
+    const int g = threadIdx.x / kLanesPerRow, ln = threadIdx.x % kLanesPerRow, d = ln * 4;
+    const int64_t base = (int64_t)row * p.max_chunks;
+    float M = -INFINITY;
+    for (int c = g; c < n_chunks; c += kGroups) M = fmaxf(M, p.ws_m[base + c]);
+    f32x4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+    for (int c = g; c < n_chunks; c += kGroups) {
+        const float f = fast_exp2(p.ws_m[base + c] - M);
+        const f32x4 o = *reinterpret_cast<const f32x4*>(p.ws_o + (base + c) * D + d);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) num[i] += f * o[i];
+        den += f * p.ws_l[base + c];
+    }
+    if (ln == 0) {
+        s_m[g] = M;                                // -inf for a group without chunks: its weight below is 0
+        s_den[g] = den;
+    }
+    s_num[g][ln] = num;
+    __syncthreads();
+    if (g != 0) return;
+    float Mall = s_m[0];
+#pragma unroll
+    for (int i = 1; i < kGroups; ++i) Mall = fmaxf(Mall, s_m[i]);
+    f32x4 tot = {0.f, 0.f, 0.f, 0.f};
+    float dtot = 0.f;
+#pragma unroll
+    for (int i = 0; i < kGroups; ++i) {
+        const float f = fast_exp2(s_m[i] - Mall);      // (group 0 always has a chunk, so Mall is finite)
+        const f32x4 o = s_num[i][ln];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) tot[e] += f * o[e];
+        dtot += f * s_den[i];
+    }
+    u32x2 w;
+    w[0] = pack_bf16(tot[0] / dtot, tot[1] / dtot);
+    w[1] = pack_bf16(tot[2] / dtot, tot[3] / dtot);
+    *reinterpret_cast<u32x2*>(p.out + (int64_t)row * D + d) = w;
+}
+
+// The wide combine serves launches of more than kWideCombineChunks chunks per sequence and at most kWideCombineRows rows
+// (a workgroup per row: with thousands of rows of eight chunks -- 16 384 at 256 sequences of 64 query heads -- the
+// narrow kernel's eight rows per workgroup are 8 us against 15).
+constexpr int kWideCombineChunks = 4;
+constexpr int kWideCombineRows = 2048;
+
 template <int D, bool FP8>
 static int launch_decode(const DecodeParams& p, hipStream_t stream) {
     dim3 grid((unsigned)p.max_chunks * p.Hkv * p.n_groups * p.B);
     hipLaunchKernelGGL((paged_decode_split_kernel<D, FP8>), grid, dim3(kDecodeWaves * 64), 0, stream, p);
-    if (p.max_chunks > 1) {
+    if (p.max_chunks > kWideCombineChunks && (int64_t)p.B * p.Hq <= kWideCombineRows) {
+        hipLaunchKernelGGL((paged_decode_combine_wide_kernel<D>), dim3((unsigned)(p.B * p.Hq)), dim3(kCombineThreads), 0,
+                           stream, p);
+    } else if (p.max_chunks > 1) {
         const int rows_per_wg = kCombineThreads / (D / 4);
         hipLaunchKernelGGL((paged_decode_combine_kernel<D>), dim3((p.B * p.Hq + rows_per_wg - 1) / rows_per_wg),
                            dim3(kCombineThreads), 0, stream, p);
