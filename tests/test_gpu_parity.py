@@ -737,6 +737,60 @@ def test_paged_prefill_head_dim_128_long_contexts_through_the_block_table(ops, H
     check(got, ref, what="paged prefill, long contexts")
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_paged_prefill_head_dim_128_random_shapes_with_runaway_keys(ops, seed):
+    """The block-table form of the 64-query kernel on drawn shapes: ragged contexts and chunks, one, two or four query
+    heads per K/V head, and keys whose scores run away in both directions at drawn places, so that the tile loop is
+    left (a row sum reached 2), entered again, and query tiles are computed a second time -- all of which fetch
+    their block ids on the way.  Garbage past every context's end."""
+    g = torch.Generator().manual_seed(2000 + seed)
+    dev = "cuda:0"
+    for case in range(4):
+        B = int(torch.randint(1, 4, (1,), generator=g))
+        Hkv = int(torch.randint(1, 3, (1,), generator=g))
+        Hq = Hkv * int(torch.tensor([1, 2, 4])[int(torch.randint(0, 3, (1,), generator=g))])
+        ctx = [int(torch.randint(1, 6000, (1,), generator=g)) for _ in range(B)]
+        chunk = [int(torch.randint(1, min(c, 700) + 1, (1,), generator=g)) for c in ctx]
+        print(f"case: paged runaway seed={seed} #{case} Hq={Hq} Hkv={Hkv} ctx={ctx} chunk={chunk}", flush=True)
+        nblk = [(c + 15) // 16 for c in ctx]
+        pool = sum(nblk) + 5
+        perm = torch.randperm(pool, generator=g)
+        kc = torch.full((pool, Hkv, 16, 128), float("nan"), dtype=torch.bfloat16)
+        vc = torch.full((pool, Hkv, 16, 128), float("nan"), dtype=torch.bfloat16)
+        bt = torch.full((B, max(nblk)), 2 ** 30, dtype=torch.int32)
+        cu = torch.tensor([0] + list(torch.tensor(chunk).cumsum(0)), dtype=torch.int32)
+        q = torch.randn(int(cu[-1]), Hq, 128, generator=g).to(torch.bfloat16)
+        ref = torch.empty(int(cu[-1]), Hq, 128)
+        off = 0
+        for b in range(B):
+            k = torch.randn(Hkv, ctx[b], 128, generator=g)
+            v = torch.randn(Hkv, ctx[b], 128, generator=g).to(torch.bfloat16)
+            for _ in range(int(torch.randint(0, 5, (1,), generator=g))):          # runaway keys
+                j = int(torch.randint(0, ctx[b], (1,), generator=g))
+                n = int(torch.randint(1, 70, (1,), generator=g))
+                k[:, j:j + n] *= float(torch.tensor([6.0, 20.0, -15.0, 45.0])[int(torch.randint(0, 4, (1,), generator=g))])
+            k = k.to(torch.bfloat16)
+            ids = perm[off:off + nblk[b]]
+            off += nblk[b]
+            bt[b, :nblk[b]] = ids.to(torch.int32)
+            pad = nblk[b] * 16 - ctx[b]
+            kp = torch.cat([k, torch.full((Hkv, pad, 128), float("nan"), dtype=torch.bfloat16)], 1)
+            vp = torch.cat([v, torch.full((Hkv, pad, 128), float("inf"), dtype=torch.bfloat16)], 1)
+            kc[ids] = kp.view(Hkv, nblk[b], 16, 128).transpose(0, 1)
+            vc[ids] = vp.view(Hkv, nblk[b], 16, 128).transpose(0, 1)
+            qb = q[int(cu[b]):int(cu[b + 1])].transpose(0, 1)[None]
+            ref[int(cu[b]):int(cu[b + 1])] = orc.prefill_reference(qb, k[None], v[None], causal=True)[0].transpose(0, 1)
+        cl = torch.tensor(ctx, dtype=torch.int32)
+        got = ops.flash_attn_paged_prefill(q.to(dev), kc.to(dev), vc.to(dev), cu.to(dev), bt.to(dev), cl.to(dev), max(chunk),
+                                           kv_splits=1)
+        n_shares = 2 + (seed + case) % 3
+        shared = ops.flash_attn_paged_prefill(q.to(dev), kc.to(dev), vc.to(dev), cu.to(dev), bt.to(dev), cl.to(dev),
+                                              max(chunk), kv_splits=n_shares)
+        torch.cuda.synchronize()
+        check(got, ref, what=f"paged 64-query kernel seed {seed} #{case}")
+        check(shared, ref, what=f"paged 64-query kernel, keys split {n_shares} ways, seed {seed} #{case}")
+
+
 @pytest.mark.parametrize("D,Hq,Hkv", [(128, 8, 2), (64, 4, 4), (128, 32, 8)])
 def test_paged_prefill_over_an_fp8_cache_matches_the_oracle(ops, D, Hq, Hkv):
     """The same ragged chunks over an fp8-e4m3 cache with per-(block, kv head) scales: gathered and dequantised by
