@@ -55,6 +55,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
     // launches ran 10-23 % slower.  The code below is written for any power of two.)
     constexpr int NB = 2;
     constexpr int kAhead = NB - 1;
+    constexpr float kBias = 32.0f;             // first attempt: the weight of a score x (log2 domain) is 2^(x - kBias)
+    constexpr float kUnderflow = 0x1p-92f;     // a final row sum below this may have lost terms
+    constexpr float kOverflow = 0x1p40f;       // ... above this (or NaN) may have overflowed somewhere
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[NB * kTile];
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[NB * kTile];
     // Staging of the query rows on their way in and of the output rows on their way out, one private slab per
@@ -268,6 +271,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
         // m_ref: exponent reference of this lane's query row, in RAW score units (>= row max - slack);
         // neg_ref = -m_ref * scale_log2 is the additive term of the exponent
         float m_ref = -INFINITY, neg_ref = 0.f, l_run = 0.f;
+        bool redo = false;                   // a row sum overflowed on the way (first attempt)
 
         const uint8_t* mrow = nullptr;
         if (boolmask)     // rows of padded query lanes alias the last real row (their results are never stored)
@@ -308,8 +312,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
 
         // First half of a KV tile: wait for it, start the next one, S^T = K . Q^T, mask, row max.
         // Returns false when the whole tile lies above this wavefront's diagonal (nothing to add).
-        auto head = [&](auto masked_c, int tile) -> bool {
+        auto head = [&](auto masked_c, auto track_c, int tile) -> bool {
             constexpr bool MASKED = decltype(masked_c)::value;
+            constexpr bool TRACK = decltype(track_c)::value;
             // this wavefront's share of tile `tile` has landed: its loads are older than those of the tiles requested
             // after it (2 * NI instructions each), which may stay in flight
             if constexpr (NB == 2) {
@@ -351,12 +356,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
                         s_acc[t][i] = keep ? s_acc[t][i] : -INFINITY;
                     }
             }
-            mx = s_acc[0][0];
+            if constexpr (TRACK) {
+                mx = s_acc[0][0];
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+                for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[t][i]);
-            mx = xor32_max(mx);
+                    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[t][i]);
+                mx = xor32_max(mx);
+            }
             return true;
         };
 
@@ -393,11 +400,40 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
         // The fast loop below therefore only accumulates in place; a tile that needs the
         // reference moved leaves it, rescales, and re-enters.
         constexpr float kSlack = 8.0f;
+        // The first attempt at a query tile does not look at row maxima at all (MODE NONE / CAUSAL): the reference is
+        // preset to 0 (weights 2^(x - kBias), x the score in the log2 domain), and what is watched is the row SUM: a
+        // partial sum that reaches 2 moves the row's reference up by the exponent of its sum, an exact rescaling by a
+        // power of two.  Scores between -60 and +72 binary orders need nothing else.  A row whose final sum left
+        // [2^-92, 2^40] (or is NaN) may have lost terms: the workgroup then runs the query tile again with the
+        // reference tracked from the row maxima (below).  What this saves is the maximum itself: 32 v_max and a
+        // cross-lane step per tile, a tenth of the vector work, which is what bounds head_dim 64 and 32.
+        auto run_tiles_preset = [&](auto masked_c, int tile, const int tile_end) {
+            while (tile < tile_end) {
+                if (head(masked_c, std::false_type{}, tile)) {
+                    accumulate();
+                    if (__builtin_amdgcn_ballot_w64(!(l_run < 2.0f)) != 0) {
+                        const float l = xor32_sum(l_run);                  // the row's sum (its keys are dealt to two lanes)
+                        if (!(l <= kOverflow)) redo = true;
+                        const int expo = (int)((__builtin_bit_cast(uint32_t, l) >> 23) & 0xffu) - 127;
+                        const int k = min(max(expo + (int)kBias, 0), 126);
+                        const float alpha = __builtin_bit_cast(float, (uint32_t)(127 - k) << 23);      // 2^-k
+                        neg_ref -= (float)k;
+                        l_run *= alpha;
+#pragma unroll
+                        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+                    }
+                }
+                flip();
+                ++tile;
+            }
+        };
         auto run_tiles = [&](auto masked_c, int tile, const int tile_end) {
             for (;;) {
                 bool pending = false;
                 while (tile < tile_end) {
-                    if (head(masked_c, tile)) {
+                    if (head(masked_c, std::true_type{}, tile)) {
                         const bool grow = !((mx - m_ref) * p.scale_log2 <= kSlack);   // also true while m_ref = -inf
                         if (__builtin_amdgcn_ballot_w64(grow) != 0) {
                             pending = true;
@@ -425,9 +461,40 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
             }
         };
 
-        set_buf(t0 & (NB - 1));              // the offsets start at the first tile's buffer
-        run_tiles(std::false_type{}, t0, min(n_plain, t1));
-        run_tiles(std::true_type{}, max(n_plain, t0), t1);
+        bool tracked = boolmask;             // explicit masks: tracked from the start
+        if constexpr (!boolmask) {
+            neg_ref = -kBias;
+            set_buf(t0 & (NB - 1));          // the offsets start at the first tile's buffer
+            cur_tile = t0;
+            run_tiles_preset(std::false_type{}, t0, min(n_plain, t1));
+            run_tiles_preset(std::true_type{}, max(n_plain, t0), t1);
+            const float l = xor32_sum(l_run);
+            // (a query that sees none of this share's keys -- causal with fewer keys than queries, or a share of split
+            // keys that lies past its diagonal -- has a sum of zero by right)
+            const int k_first = t0 * kBN;
+            const bool sees = t0 < t1 && k_first < sk && (!causal || k_first <= qi + coff);
+            const bool bad = redo || (sees && !(l >= kUnderflow)) || !(l <= kOverflow);
+            // the workgroup meets (everybody is done with the K/V buffers) and votes
+            if (__syncthreads_or(bad ? 1 : 0)) {
+                tracked = true;
+#pragma unroll
+                for (int i = 0; i < kAhead; ++i)
+                    if (t0 + i < t1) issue_tile(t0 + i, (t0 + i) & (NB - 1));
+#pragma unroll
+                for (int i = 0; i < NDT; ++i)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) o[i][j] = 0.f;
+                m_ref = -INFINITY;
+                neg_ref = 0.f;
+                l_run = 0.f;
+            }
+        }
+        if (tracked) {
+            set_buf(t0 & (NB - 1));
+            cur_tile = t0;
+            run_tiles(std::false_type{}, t0, min(n_plain, t1));
+            run_tiles(std::true_type{}, max(n_plain, t0), t1);
+        }
 
         // ---- normalise and store: lane owns query qi, d = 32dt + 8(i/4) + 4kg + i%4 ---
         l_run = xor32_sum(l_run);
@@ -438,7 +505,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
             if (q_ok) {
                 const int64_t prow = ((int64_t)split * p.Hq + h) * p.part_rows + part_row0 + qi;
                 if (kg == 0)
-                    p.part_lse[prow] = l_run > 0.f ? 0.69314718056f * (m_ref * p.scale_log2 + __log2f(l_run)) : -INFINITY;
+                    p.part_lse[prow] = l_run > 0.f ? 0.69314718056f * (__log2f(l_run) - neg_ref) : -INFINITY;
                 float* po = p.part_o + prow * D + 4 * kg;
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt)
@@ -453,9 +520,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillPa
             continue;
         }
         const float inv = 1.0f / l_run;          // l == 0 (no key kept) -> NaN row, like the reference softmax
-        // sum_j exp(scale * s_j) = 2^(m_ref * scale_log2) * l  ->  lse = ln2 * (m_ref * scale_log2 + log2 l)
+        // sum_j exp(scale * s_j) = 2^(-neg_ref) * l  ->  lse = ln2 * (log2 l - neg_ref)
         if (lb && q_ok && kg == 0)
-            lb[qi] = l_run > 0.f ? 0.69314718056f * (m_ref * p.scale_log2 + __log2f(l_run)) : -INFINITY;
+            lb[qi] = l_run > 0.f ? 0.69314718056f * (__log2f(l_run) - neg_ref) : -INFINITY;
         {
             // (the slab is private to the wavefront and LDS operations of a wavefront execute in order: no barrier)
             unsigned char* slab = o_lds + wave * (32 * kORow);

@@ -336,6 +336,49 @@ def test_prefill_unmasked_scores_that_outgrow_the_reference(ops):
     check(ops.scaled_dot_product_attention(q.cuda(), k.cuda(), v.cuda(), keep), ref, what="reference moves, masked path")
 
 
+@pytest.mark.parametrize("D", [32, 64])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_prefill_head_dim_64_32_preset_reference_against_tracked_maxima(ops, D, seed):
+    """The 8-wavefront kernel first runs a query tile with a preset exponent reference, watching row sums, and runs it
+    again with the reference tracked from the row maxima when a row's sum leaves the safe range.  An explicit
+    all-visible mask takes the tracked path from the start, so the two paths can be compared with each other and with
+    the oracle: drawn shapes (ragged, more keys than queries, GQA, causal or not), keys whose scores run away by
+    tens to thousands of binary orders in both directions (rescaling in the loop, second attempts), keys split over
+    workgroups, and rows whose scores are all hugely negative."""
+    g = torch.Generator().manual_seed(3000 + 10 * D + seed)
+    for case in range(5):
+        B = int(torch.randint(1, 3, (1,), generator=g))
+        Hkv = int(torch.randint(1, 3, (1,), generator=g))
+        Hq = Hkv * int(torch.randint(1, 3, (1,), generator=g))
+        Sq = int(torch.randint(1, 700, (1,), generator=g))
+        Sk = Sq + int(torch.randint(0, 700, (1,), generator=g)) * int(torch.randint(0, 2, (1,), generator=g))
+        causal = bool(torch.randint(0, 2, (1,), generator=g))
+        print(f"case: preset/tracked D={D} seed={seed} #{case} B={B} Hq={Hq} Hkv={Hkv} Sq={Sq} Sk={Sk} causal={causal}", flush=True)
+        q = torch.randn(B, Hq, Sq, D, generator=g).to(torch.bfloat16)
+        k = torch.randn(B, Hkv, Sk, D, generator=g)
+        v = torch.randn(B, Hkv, Sk, D, generator=g).to(torch.bfloat16)
+        for _ in range(int(torch.randint(0, 6, (1,), generator=g))):          # runaway keys
+            j = int(torch.randint(0, Sk, (1,), generator=g))
+            n = int(torch.randint(1, 70, (1,), generator=g))
+            k[:, :, j:j + n] *= float(torch.tensor([6.0, 20.0, -15.0, 45.0, 300.0])[int(torch.randint(0, 5, (1,), generator=g))])
+        if case == 4:                                  # every score of the first head pair far below the preset reference
+            k[:, 0] = k[:, 0].abs() * 12.0
+            q[:, :Hq // Hkv] = -(q[:, :Hq // Hkv].float().abs() * 2.0).to(torch.bfloat16)
+        k = k.to(torch.bfloat16)
+        ref = orc.prefill_reference(q, k, v, causal=causal)
+        fast = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=causal, kv_splits=1)
+        keep = torch.ones(Sq, Sk, dtype=torch.bool)
+        if causal:
+            keep = torch.tril(keep, diagonal=Sk - Sq)
+        slow = ops.scaled_dot_product_attention(q.cuda(), k.cuda().repeat_interleave(Hq // Hkv, 1),
+                                                v.cuda().repeat_interleave(Hq // Hkv, 1), keep.cuda())
+        shared = ops.flash_attn_prefill(q.cuda(), k.cuda(), v.cuda(), causal=causal, kv_splits=2 + (seed + case) % 3)
+        torch.cuda.synchronize()
+        check(fast, ref, what=f"preset reference D={D} seed {seed} #{case}")
+        check(slow, ref, what=f"tracked maxima D={D} seed {seed} #{case}")
+        check(shared, ref, what=f"preset reference, keys split, D={D} seed {seed} #{case}")
+
+
 @pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("splits", [2, 5, 64])
 def test_prefill_split_keys_dense(ops, D, splits):
