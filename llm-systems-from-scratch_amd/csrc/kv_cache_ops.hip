@@ -445,6 +445,8 @@ extern "C" int mi355_quantize_kv_fp8(const void* cache_bf16, void* cache_fp8, fl
 }
 
 
+namespace mi355 {
+
 // ---------------------------------------------------------------------------------------------
 // Gather + dequantise: the keys and values of every sequence of a batch, read through the block tables out of an
 // fp8 cache, written as packed bf16 rows (sequence b owns rows [cu_k[b], cu_k[b+1])) -- the K/V operands of a packed
@@ -521,6 +523,8 @@ __global__ __launch_bounds__(256) void gather_kv_fp8_kernel(GatherFp8Params p) {
         }
     }
 }
+
+}  // namespace mi355
 
 extern "C" int mi355_gather_kv_fp8(const void* k_cache_fp8, const void* v_cache_fp8, const float* k_scale,
                                    const float* v_scale, const int32_t* block_tables, int64_t table_stride,
