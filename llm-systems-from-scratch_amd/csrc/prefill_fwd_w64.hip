@@ -1,5 +1,5 @@
-// Prefill forward for head_dim 128 (no mask or causal; optional log-sum-exp output), one wavefront per SIMD, 64
-// queries per wavefront.
+// Prefill forward for head_dim 128 (no mask or causal; optional log-sum-exp output; K/V packed, dense, or read through
+// the block table of a paged cache), one wavefront per SIMD, 64 queries per wavefront.
 //
 // One workgroup = 4 wavefronts = one tile of 256 queries of one (batch, head); a wavefront owns 64 query rows as two
 // column blocks A and B of 32.  It runs alone on its SIMD with the whole register file: the output accumulators
@@ -35,8 +35,10 @@
 // next.  The next job is worked out at the top of the current one, and its first requests (K[0], query rows, V[0],
 // then K[1]) go out between the pieces of output work -- the query rows earlier still where a causal mask leaves
 // wavefronts without work in the last tiles of a job: they request them then, also for the others.  No ordinary
-// vector load sits in the job loop, so the only waits on memory are the ones written here (the compiler would add s_waitcnt vmcnt(0), which also waits for every
-// request in flight, in front of the first use of a loaded register).
+// vector load sits in the job loop of the packed forms, so the only waits on memory are the ones written here (the
+// compiler would add s_waitcnt vmcnt(0), which also waits for every request in flight, in front of the first use of
+// a loaded register).  The block-table form has one such load, of the block ids of the next 64 tiles, directly in
+// front of the tile loop: its wait lands where the first hand-over would wait for the same requests anyway.
 //
 // Hand-over protocol between the two (and between tiles), one "boundary" per tile t and wavefront: K[t] and V[t]
 // live in LDS buffers t % 2.  When tile t starts, K[t] has landed and the workgroup has met since; K[t+1] and V[t]
