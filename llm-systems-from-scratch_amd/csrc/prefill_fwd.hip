@@ -39,8 +39,13 @@ constexpr int kBN = 64;    // keys per LDS tile
 // PAGED: keys and values are read from a paged cache through a block table (16 rows per block, so
 // every direct-to-LDS instruction -- 4, 8 or 16 whole rows -- stays inside one block and needs one
 // table entry, a scalar load); queries and outputs are packed.
+// Occupancy: at head_dim 64 the kernel is held to the registers of four wavefronts per SIMD (128; left alone the
+// compiler takes 163 and a compute unit then holds ONE workgroup, whose barriers and waits nobody fills): two
+// workgroups per compute unit, 7-8 % faster at throughput shapes and 14 % on short sequences, a handful of spilled
+// registers outside the tile loop.  Head_dim 32 has two workgroups per compute unit as it is (117 registers; a third
+// would need 85 and spills by the hundred: three to four times slower), head_dim 128 needs its 250.
 template <int D, int MODE, bool PAGED = false>
-__global__ __launch_bounds__(kPfWaves * 64, 1) void prefill_fwd_kernel(PrefillParams p) {
+__global__ __launch_bounds__(kPfWaves * 64, D == 64 ? 4 : 1) void prefill_fwd_kernel(PrefillParams p) {
     constexpr int NS = D / 16;                    // MFMA k-steps of K.Q^T
     constexpr int NDT = D / 32;                   // 32-row tiles of O^T
     constexpr int CPR = D / 8;                    // 16-byte chunks per row
