@@ -834,6 +834,26 @@ def test_paged_prefill_head_dim_128_random_shapes_with_runaway_keys(ops, seed):
         check(shared, ref, what=f"paged 64-query kernel, keys split {n_shares} ways, seed {seed} #{case}")
 
 
+@pytest.mark.parametrize("B", [4096, 4097])
+def test_paged_prefill_head_dim_128_thousands_of_short_sequences(ops, B):
+    """As many sequences as the 64-query kernel keeps counts for in LDS (4096: 64 groups of 64), and one more (the
+    8-wavefront kernel then serves the launch): chunks of one to three tokens over contexts of a few blocks."""
+    print(f"case: paged prefill D=128, {B} sequences", flush=True)
+    g = torch.Generator().manual_seed(40)
+    ctx = [int(x) for x in torch.randint(1, 40, (B,), generator=g)]
+    chunk = [min(c, int(x)) for c, x in zip(ctx, torch.randint(1, 4, (B,), generator=g))]
+    _, kc, vc, bt, cl = orc.make_paged_case(batch=B, n_q_heads=4, n_kv_heads=1, head_dim=128, block_size=16,
+                                            context_lens=ctx, pool_factor=1.1, seed=41, dtype=torch.bfloat16)
+    cu = torch.tensor([0] + list(torch.tensor(chunk).cumsum(0)), dtype=torch.int32)
+    q = rnd(int(cu[-1]), 4, 128, seed=42)
+    ref = orc.paged_prefill_reference(q, kc, vc, cu, bt, cl)
+    dev = "cuda:0"
+    got = ops.flash_attn_paged_prefill(q.to(dev), kc.to(dev), vc.to(dev), cu.to(dev), bt.to(dev), cl.to(dev), max(chunk),
+                                       kv_splits=1)
+    torch.cuda.synchronize()
+    check(got, ref, what=f"paged prefill, {B} sequences")
+
+
 @pytest.mark.parametrize("D,Hq,Hkv", [(128, 8, 2), (64, 4, 4), (128, 32, 8)])
 def test_paged_prefill_over_an_fp8_cache_matches_the_oracle(ops, D, Hq, Hkv):
     """The same ragged chunks over an fp8-e4m3 cache with per-(block, kv head) scales: gathered and dequantised by
