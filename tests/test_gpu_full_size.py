@@ -244,3 +244,65 @@ def test_prefill_and_backward_full_size(ops):
         err = (got.float().cpu() - ref).abs()
         bound = 2e-2 * float(ref.abs().max()) + 2e-2 * ref.abs()
         assert bool((err <= bound).all()), f"{name}: max err {float(err.max()):.4g} (max |ref| {float(ref.abs().max()):.4g})"
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_prompt_chunks_over_a_cached_prefix_at_serving_size(ops, fp8):
+    """Four chunks of 2048 rows over 8192 cached tokens each, 32 query / 8 kv heads, head_dim 128, keys and values read
+    through the block table (the shape of bench.py's paged legs).  The oracle on one sequence and the eight query
+    heads of two kv heads; relocation: after moving every block to another physical position (tables rewritten) the
+    output is identical bit for bit; and the packed kernel on the gathered rows gives the same bits (bf16 cache)."""
+    print(f"case: paged chunks 4 x 2048 over 8192, fp8={fp8}", flush=True)
+    dev = "cuda:0"
+    B, chunk, ctx, Hq, Hkv, D = 4, 2048, 8192, 32, 8, 128
+    nblk = ctx // 16
+    g = torch.Generator(device=dev).manual_seed(77)
+    pool = B * nblk + 9
+    kc = (torch.randn(pool, Hkv, 16, D, device=dev, generator=g) * 0.7).to(torch.bfloat16)
+    vc = (torch.randn(pool, Hkv, 16, D, device=dev, generator=g) * 0.7).to(torch.bfloat16)
+    perm = torch.randperm(pool, device=dev, generator=g)
+    table = perm[:B * nblk].view(B, nblk).to(torch.int32)
+    lens = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    cu = (torch.arange(B + 1, device=dev) * chunk).to(torch.int32)
+    q = (torch.randn(B * chunk, Hq, D, device=dev, generator=g) * 0.7).to(torch.bfloat16)
+    kw = {}
+    kq, vq = kc, vc
+    if fp8:
+        kq, ks = ops.quantize_kv_cache_fp8(kc)
+        vq, vs = ops.quantize_kv_cache_fp8(vc)
+        kw = {"k_scale": ks, "v_scale": vs, "total_context": B * ctx}
+    got = ops.flash_attn_paged_prefill(q, kq, vq, cu, table, lens, chunk, **kw)
+    # oracle: sequence 2, query heads 0..7 (kv heads 0, 1), on the cache the kernel read (dequantised for fp8)
+    b = 2
+    ids = table[b].long()
+    if fp8:
+        k_seq = orc.dequantize_kv_fp8(kq[ids].cpu(), ks[ids].cpu())[:, :2]
+        v_seq = orc.dequantize_kv_fp8(vq[ids].cpu(), vs[ids].cpu())[:, :2]
+    else:
+        k_seq, v_seq = kc[ids, :2].float().cpu(), vc[ids, :2].float().cpu()
+    k_lin = k_seq.permute(1, 0, 2, 3).reshape(1, 2, ctx, D)
+    v_lin = v_seq.permute(1, 0, 2, 3).reshape(1, 2, ctx, D)
+    q_seq = q[b * chunk:(b + 1) * chunk, :8].transpose(0, 1)[None].cpu()
+    ref = orc.prefill_reference(q_seq, k_lin, v_lin, causal=True, head_chunk=4)[0].transpose(0, 1)
+    _close(got[b * chunk:(b + 1) * chunk, :8], ref)
+    # relocation
+    perm2 = torch.randperm(pool, device=dev, generator=g)
+    k2, v2 = torch.empty_like(kq), torch.empty_like(vq)
+    k2[perm2] = kq
+    v2[perm2] = vq
+    table2 = perm2[table.long()].to(torch.int32)
+    kw2 = dict(kw)
+    if fp8:
+        ks2, vs2 = torch.empty_like(ks), torch.empty_like(vs)
+        ks2[perm2] = ks
+        vs2[perm2] = vs
+        kw2.update(k_scale=ks2, v_scale=vs2)
+    moved = ops.flash_attn_paged_prefill(q, k2, v2, cu, table2, lens, chunk, **kw2)
+    assert torch.equal(moved, got)
+    if not fp8:
+        rows = kc[table.long()]                                         # (B, nblk, Hkv, 16, D) -> packed (B*ctx, Hkv, D)
+        k_pack = rows.permute(0, 1, 3, 2, 4).reshape(B * ctx, Hkv, D).contiguous()
+        v_pack = vc[table.long()].permute(0, 1, 3, 2, 4).reshape(B * ctx, Hkv, D).contiguous()
+        cu_k = (torch.arange(B + 1, device=dev) * ctx).to(torch.int32)
+        packed = ops.flash_attn_varlen_prefill(q, k_pack, v_pack, cu, cu_k, chunk, ctx, causal=True, kv_splits=1)
+        assert torch.equal(packed, got)
