@@ -116,6 +116,21 @@ def test_decode_of_one_sequence_uses_the_shortest_chunks(ops, fp8, ctx):
     check(got, ref, what=f"one sequence ctx={ctx} fp8={fp8}")
 
 
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("batch,ctx", [(1, 20000), (3, 5000), (9, 1500)])
+def test_decode_of_few_sequences_combines_many_chunks(ops, D, batch, ctx):
+    """Few sequences of long contexts run short chunks, up to hundreds per sequence, and their partial results are
+    merged by the combine kernel that gives a workgroup to every row (more than four chunks per sequence, at most
+    2048 rows): ragged lengths, so that rows of one launch have 1 to n chunks, every head size."""
+    print(f"case: decode few sequences D={D} batch={batch} ctx={ctx}", flush=True)
+    lens = [max(1, ctx - 977 * i) for i in range(batch)]
+    q, kc, vc, bt, cl = orc.make_paged_case(batch=batch, n_q_heads=8, n_kv_heads=2, head_dim=D, block_size=16,
+                                            context_lens=lens, pool_factor=1.2, seed=93, dtype=torch.bfloat16)
+    got = run_decode(ops, q, kc, vc, bt, cl)
+    ref = orc.paged_decode_reference(q, kc, vc, bt, cl)
+    check(got, ref, what=f"few sequences D={D} batch={batch} ctx={ctx}")
+
+
 @pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("slope", [0.4, 0.02, -0.02, -0.4])
 def test_decode_scores_that_ramp_along_the_context(ops, fp8, slope):
